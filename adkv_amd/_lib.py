@@ -1,0 +1,69 @@
+"""ctypes binding of libadkv_hip.so (C ABI: include/adkv_hip.h).
+
+There is deliberately no fallback: if the library is absent or a symbol is missing, importing the
+kernels raises.  torch must be imported before the library is opened so that the HIP runtime torch
+already loaded (same soname) is the one the kernels register with.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import torch  # noqa: F401  (loads libamdhip64 first)
+
+_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_DIR, "libadkv_hip.so")
+ABI_VERSION = 1
+
+_vp, _i, _f = C.c_void_p, C.c_int, C.c_float
+
+# name -> (restype, argtypes); must list every symbol include/adkv_hip.h declares
+PROTOTYPES = {
+    "adkv_abi_version": (_i, []),
+    "adkv_strerror": (C.c_char_p, [_i]),
+    "adkv_last_hip_error": (_i, []),
+    "adkv_encode_kv": (_i, [_vp] * 7 + [_i] * 5 + [_f, _f, _vp, _vp]),
+    "adkv_forward_qk": (_i, [_vp] * 9 + [_i] * 5 + [_f, _f, _vp, _vp]),
+    "adkv_forward_ov": (_i, [_vp] * 9 + [_i] * 5 + [_f, _f, _vp, _vp]),
+    "adkv_softmax": (_i, [_vp] * 3 + [_i] * 3 + [_f, _vp]),
+}
+
+_lib = None
+
+
+class ADKVLibraryError(RuntimeError):
+    pass
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ADKVLibraryError(
+                f"{LIB_PATH} is missing: build it with `python -m adkv_amd.build` "
+                "(hipcc --offload-arch=gfx950). There is no CPU fallback.")
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in PROTOTYPES.items():
+            try:
+                fn = getattr(L, name)
+            except AttributeError as e:
+                raise ADKVLibraryError(f"{LIB_PATH} does not export {name}") from e
+            fn.restype, fn.argtypes = res, args
+        v = L.adkv_abi_version()
+        if v != ABI_VERSION:
+            raise ADKVLibraryError(f"libadkv_hip ABI {v} != expected {ABI_VERSION}; rebuild")
+        _lib = L
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        L = lib()
+        msg = L.adkv_strerror(rc).decode()
+        if rc == -100:
+            msg += f" (hipError {L.adkv_last_hip_error()})"
+        raise RuntimeError(f"{what}: {msg}")
+
+
+def current_stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream

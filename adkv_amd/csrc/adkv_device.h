@@ -1,0 +1,92 @@
+// Device-side building blocks of the ADKV kernels (gfx950, wave64).
+//
+// Arithmetic contract (reference: src/adkv/kernel/gemv.cu:79-88,150-164,220-221): the per-channel
+// state (zp, sc) is fp16 and every step below is ONE IEEE round-to-nearest-even fp16 operation, so
+// the state trajectory is bit-identical to the reference's half2 code.  This file must be compiled
+// with -ffp-contract=off: "q*sc + zp" has to stay two roundings where the reference has two.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#pragma clang fp contract(off)
+
+namespace adkv {
+
+typedef _Float16 h1;
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ h2 as_h2(uint32_t u) { return __builtin_bit_cast(h2, u); }
+__device__ __forceinline__ uint32_t as_u32(h2 h) { return __builtin_bit_cast(uint32_t, h); }
+__device__ __forceinline__ h2 pk_fma(h2 a, h2 b, h2 c) { return __builtin_elementwise_fma(a, b, c); }
+__device__ __forceinline__ h2 pk_abs(h2 a) { return as_h2(as_u32(a) & 0x7FFF7FFFu); }
+__device__ __forceinline__ h2 splat(h1 x) { return (h2){x, x}; }
+
+// One channel pair's filter state and fixed parameters (two channels packed per register).
+struct Pair {
+    h2 zp, sc, al, be, omt;
+};
+
+// Loads the pair starting at parameter index pi (even).  omt = 1 - beta*target with both steps
+// rounded to fp16 (gemv.cu:220-221).
+__device__ __forceinline__ void load_pair(Pair &p, const h1 *zp, const h1 *sc, const h1 *al,
+                                          const h1 *be, const h1 *tg, int pi)
+{
+    p.zp = *reinterpret_cast<const h2 *>(zp + pi);
+    p.sc = *reinterpret_cast<const h2 *>(sc + pi);
+    p.al = *reinterpret_cast<const h2 *>(al + pi);
+    p.be = *reinterpret_cast<const h2 *>(be + pi);
+    const h2 t = *reinterpret_cast<const h2 *>(tg + pi);
+    const h2 bt = p.be * t;
+    p.omt = splat((h1)1.0f) - bt;
+}
+
+// EMA update with an already computed qs = r16(q*sc) (gemv.cu:158-164):
+//   zp <- r16(alpha*qs + zp)   sc <- r16(sc * r16(beta*|q| + omt))
+__device__ __forceinline__ void update_pair(Pair &p, h2 q, h2 qs)
+{
+    p.zp = pk_fma(p.al, qs, p.zp);
+    const h2 f = pk_fma(p.be, pk_abs(q), p.omt);
+    p.sc = p.sc * f;
+}
+
+// Byte row br of two channel words -> the two tokens' code pairs as exact fp16 integers.
+//   x = [0, B.byte[br], 0, A.byte[br]]
+//   low nibbles : 0x6400|n = 1024+n  -> minus 1032 = n-8   (gemv.cu:79-88)
+//   high nibbles: 0x5400|(n<<4) = 64+n -> minus 72 = n-8   (same trick one binade lower: no shift)
+template <int BR>
+__device__ __forceinline__ void unpack_row(uint32_t wa, uint32_t wb, h2 &q_even, h2 &q_odd)
+{
+    constexpr uint32_t sel = 0x0C000C00u | ((4u + BR) << 16) | (uint32_t)BR;
+    const uint32_t x = __builtin_amdgcn_perm(wb, wa, sel);
+    q_even = as_h2((x & 0x000F000Fu) | 0x64006400u) - splat((h1)1032.0f);
+    q_odd = as_h2((x & 0x00F000F0u) | 0x54005400u) - splat((h1)72.0f);
+}
+
+// gemv.cu:150-154: fp32 subtract, IEEE fp32 divide, round-half-even, NaN -> 0, clamp to [-8,7].
+__device__ __forceinline__ int quantize(h1 x, h1 zp, h1 sc)
+{
+    const float d = (float)x - (float)zp;
+    const float u = d / (float)sc;
+    float r = __builtin_rintf(u);
+    r = (u != u) ? 0.0f : r;
+    r = __builtin_fminf(__builtin_fmaxf(r, -8.0f), 7.0f);
+    return (int)r;
+}
+
+__device__ __forceinline__ h2 codes_to_h2(int q0, int q1) { return (h2){(h1)q0, (h1)q1}; }
+
+// Quantise one new token's channel pair with the current state and patch its two nibbles into the
+// channel words at token slot tt (0..7) of the supergroup (gemv.cu:91-146).  Returns the code pair.
+__device__ __forceinline__ h2 append_pair(uint32_t &wa, uint32_t &wb, int tt, h2 x, const Pair &p)
+{
+    const int q0 = quantize(x.x, p.zp.x, p.sc.x);
+    const int q1 = quantize(x.y, p.zp.y, p.sc.y);
+    const uint32_t sh = 4u * (uint32_t)tt;
+    const uint32_t m = ~(0xFu << sh);
+    wa = (wa & m) | (((uint32_t)(q0 + 8) & 0xFu) << sh);
+    wb = (wb & m) | (((uint32_t)(q1 + 8) & 0xFu) << sh);
+    return codes_to_h2(q0, q1);
+}
+
+} // namespace adkv

@@ -1,0 +1,665 @@
+// ADKV hot-path kernels for MI355X (gfx950, wave64) and their C ABI (include/adkv_hip.h).
+//
+// Work decomposition.  Every (batch, head, channel) is an independent fp16 recurrence over the
+// time axis (reference: src/adkv/kernel/gemv.cu:187-191), and without stored intermediate states
+// it has to be replayed from token 0.  So a LANE owns CPL consecutive channels of one head for the
+// whole sequence; D/CPL lanes make a head; a wave64 carries 64*CPL/D heads.  One supergroup
+// (8 tokens) of a head is D*4 contiguous bytes, which a head's lanes fetch as one run of 16-byte
+// loads; loads for the next PF supergroups are in flight while the current one is decoded.
+//
+// The three kernels below keep the reference's call structure (encode / QK+append / OV+append) so
+// that they are drop-ins for src/adkv/kernel/gemv.cu:368-414, 883-939, 1233-1288.
+#include "adkv_device.h"
+
+#include "../../include/adkv_hip.h"
+
+#pragma clang fp contract(off)
+
+namespace adkv {
+
+constexpr int BLOCK = 256;  // 4 waves
+constexpr int PF = 4;       // supergroups in flight per lane
+
+template <int D, int CPL>
+struct Geo {
+    static constexpr int LPH = D / CPL;       // lanes per head
+    static constexpr int NV = CPL / 4;        // 16-byte vectors per lane per supergroup
+    static constexpr int NP = CPL / 2;        // channel pairs per lane
+    static constexpr int VPS = D / 4;         // 16-byte vectors per supergroup of one head
+    static_assert(LPH == 32 || LPH == 64, "a head must fit in one wave");
+};
+
+__device__ __forceinline__ float wave_xor_add(float v, int mask)
+{
+    return v + __shfl_xor(v, mask, 64);
+}
+
+// Sum over the LPH lanes of a head; every lane of the head gets the total.
+template <int LPH>
+__device__ __forceinline__ float head_allreduce(float v)
+{
+#pragma unroll
+    for (int m = 1; m < LPH; m <<= 1)
+        v = wave_xor_add(v, m);
+    return v;
+}
+
+// ---------------------------------------------------------------------------------------------
+// encode_kv  (gemv.cu:168-308)
+// ---------------------------------------------------------------------------------------------
+template <int D, int CPL>
+__global__ __launch_bounds__(BLOCK) void encode_kernel(
+    uint4 *__restrict__ cache, const h1 *__restrict__ kv_new,
+    const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
+    const h1 *__restrict__ be, const h1 *__restrict__ tg,
+    int BH, int H, int T, int n_super_cap, h1 *__restrict__ state_out)
+{
+    using G = Geo<D, CPL>;
+    const int gl = blockIdx.x * BLOCK + threadIdx.x;
+    int bx = gl / G::LPH;
+    const int lh = gl % G::LPH;
+    const bool active = bx < BH;
+    if (!active)
+        bx = BH - 1;
+    const int h = bx % H;
+    const int c0 = lh * CPL;
+
+    Pair st[G::NP];
+#pragma unroll
+    for (int p = 0; p < G::NP; p++)
+        load_pair(st[p], zp, sc, al, be, tg, h * D + c0 + 2 * p);
+
+    uint4 *cb = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV;
+    const h1 *xb = kv_new + (size_t)bx * T * D + c0;
+    const int n_super = (T + 7) / 8;
+
+    for (int sg = 0; sg < n_super; sg++) {
+        uint32_t w[CPL];
+#pragma unroll
+        for (int c = 0; c < CPL; c++)
+            w[c] = 0u;
+        // issue the supergroup's loads first, then run the serial chain over them
+        h2 x[8][G::NP];
+#pragma unroll
+        for (int tt = 0; tt < 8; tt++) {
+            const int t = sg * 8 + tt;
+            if (t < T) {
+#pragma unroll
+                for (int p = 0; p < G::NP; p++)
+                    x[tt][p] = *reinterpret_cast<const h2 *>(xb + (size_t)t * D + 2 * p);
+            }
+        }
+#pragma unroll
+        for (int tt = 0; tt < 8; tt++) {
+            const int t = sg * 8 + tt;
+            if (t < T) {
+#pragma unroll
+                for (int p = 0; p < G::NP; p++) {
+                    const h2 q = append_pair(w[2 * p], w[2 * p + 1], tt, x[tt][p], st[p]);
+                    update_pair(st[p], q, q * st[p].sc);
+                }
+            }
+        }
+        if (active) {
+#pragma unroll
+            for (int v = 0; v < G::NV; v++)
+                cb[(size_t)sg * G::VPS + v] =
+                    make_uint4(w[4 * v], w[4 * v + 1], w[4 * v + 2], w[4 * v + 3]);
+        }
+    }
+    if (state_out != nullptr && active) {
+        h2 *so = reinterpret_cast<h2 *>(state_out + ((size_t)bx * D + c0) * 2);
+#pragma unroll
+        for (int p = 0; p < G::NP; p++) {
+            so[2 * p] = (h2){st[p].zp.x, st[p].sc.x};
+            so[2 * p + 1] = (h2){st[p].zp.y, st[p].sc.y};
+        }
+    }
+}
+
+// Shared tail of the two decode kernels: quantise the new token with the state after token T-1,
+// patch it into slot T, return the fused dequant r16(q*sc + zp) per pair (gemv.cu:744-798,
+// 1105-1157).  The state is NOT advanced.
+template <int D, int CPL>
+__device__ __forceinline__ void append_new_token(uint4 *cb, int T, const h1 *xnew, const Pair *st,
+                                                 h2 *deq, bool active)
+{
+    using G = Geo<D, CPL>;
+    const int sg = T >> 3, tt = T & 7;
+#pragma unroll
+    for (int v = 0; v < G::NV; v++) {
+        uint4 *slot = cb + (size_t)sg * G::VPS + v;
+        uint4 u = *slot;
+        uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int pp = 0; pp < 2; pp++) {
+            const int p = 2 * v + pp;
+            const h2 x = *reinterpret_cast<const h2 *>(xnew + 2 * p);
+            const h2 q = append_pair(w[2 * pp], w[2 * pp + 1], tt, x, st[p]);
+            deq[p] = pk_fma(q, st[p].sc, st[p].zp);
+        }
+        if (active)
+            *slot = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
+template <int D, int CPL>
+__device__ __forceinline__ void store_state(h1 *state_out, int bx, int c0, const Pair *st)
+{
+    h2 *so = reinterpret_cast<h2 *>(state_out + ((size_t)bx * D + c0) * 2);
+#pragma unroll
+    for (int p = 0; p < CPL / 2; p++) {
+        so[2 * p] = (h2){st[p].zp.x, st[p].sc.x};
+        so[2 * p + 1] = (h2){st[p].zp.y, st[p].sc.y};
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward_qk  (gemv.cu:435-815)
+// ---------------------------------------------------------------------------------------------
+// Per lane and supergroup: 8 fp32 partial logits (v_dot2_f32_f16 over the lane's channel pairs).
+// They are summed across the head's lanes through a wave-private, conflict-free (stride 9) LDS
+// transpose: lane (g, tk) adds the partials of token tk from lanes 8g..8g+7, then xor-shuffles
+// fold the remaining LPH/8 groups.
+template <int D, int CPL>
+__global__ __launch_bounds__(BLOCK) void qk_kernel(
+    const h1 *__restrict__ q, uint4 *__restrict__ cache, const h1 *__restrict__ k_new,
+    h1 *__restrict__ out,
+    const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
+    const h1 *__restrict__ be, const h1 *__restrict__ tg,
+    int BH, int H, int T, int n_super_cap, h1 *__restrict__ state_out)
+{
+    using G = Geo<D, CPL>;
+    __shared__ float red[BLOCK / 64][64 * 9];
+
+    const int lane = threadIdx.x & 63;
+    float *myred = red[threadIdx.x >> 6];
+    const int gl = blockIdx.x * BLOCK + threadIdx.x;
+    int bx = gl / G::LPH;
+    const int lh = gl % G::LPH;
+    const bool active = bx < BH;
+    if (!active)
+        bx = BH - 1;
+    const int h = bx % H;
+    const int c0 = lh * CPL;
+
+    Pair st[G::NP];
+    h2 qv[G::NP];
+#pragma unroll
+    for (int p = 0; p < G::NP; p++) {
+        load_pair(st[p], zp, sc, al, be, tg, h * D + c0 + 2 * p);
+        qv[p] = *reinterpret_cast<const h2 *>(q + (size_t)bx * D + c0 + 2 * p);
+    }
+
+    uint4 *cb = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV;
+    h1 *ob = out + (size_t)bx * (T + 1);
+    const int nfull = T >> 3;
+    const int tk = lane & 7, g8 = lane >> 3;
+
+    auto reduce_store = [&](const float *part, int sg, int ntok) {
+#pragma unroll
+        for (int k = 0; k < 8; k++)
+            myred[lane * 9 + k] = part[k];
+        float s = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 8; r++)
+            s += myred[(g8 * 8 + r) * 9 + tk];
+#pragma unroll
+        for (int m = 8; m < G::LPH; m <<= 1)
+            s = wave_xor_add(s, m);
+        if (active && lh < 8 && tk < ntok)
+            ob[sg * 8 + tk] = (h1)s;
+    };
+
+    auto decode_sg = [&](const uint4 *u, float *part) {
+#pragma unroll
+        for (int v = 0; v < G::NV; v++) {
+            const uint32_t w[4] = {u[v].x, u[v].y, u[v].z, u[v].w};
+#pragma unroll
+            for (int pp = 0; pp < 2; pp++) {
+                Pair &s = st[2 * v + pp];
+                const h2 qq = qv[2 * v + pp];
+                auto row = [&](h2 qe, h2 qo, int br) {
+                    const h2 qs0 = qe * s.sc;
+                    part[2 * br] = __builtin_amdgcn_fdot2(qq, qs0 + s.zp, part[2 * br], false);
+                    update_pair(s, qe, qs0);
+                    const h2 qs1 = qo * s.sc;
+                    part[2 * br + 1] = __builtin_amdgcn_fdot2(qq, qs1 + s.zp, part[2 * br + 1], false);
+                    update_pair(s, qo, qs1);
+                };
+                h2 qe, qo;
+                unpack_row<0>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 0);
+                unpack_row<1>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 1);
+                unpack_row<2>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 2);
+                unpack_row<3>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 3);
+            }
+        }
+    };
+
+    // software pipeline over full supergroups
+    uint4 buf[PF][G::NV];
+#pragma unroll
+    for (int i = 0; i < PF; i++)
+        if (i < nfull) {
+#pragma unroll
+            for (int v = 0; v < G::NV; v++)
+                buf[i][v] = cb[(size_t)i * G::VPS + v];
+        }
+    for (int sg0 = 0; sg0 < nfull; sg0 += PF) {
+#pragma unroll
+        for (int i = 0; i < PF; i++) {
+            const int sg = sg0 + i;
+            if (sg < nfull) {
+                uint4 cur[G::NV];
+#pragma unroll
+                for (int v = 0; v < G::NV; v++)
+                    cur[v] = buf[i][v];
+                if (sg + PF < nfull) {
+#pragma unroll
+                    for (int v = 0; v < G::NV; v++)
+                        buf[i][v] = cb[(size_t)(sg + PF) * G::VPS + v];
+                }
+                float part[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+                decode_sg(cur, part);
+                reduce_store(part, sg, 8);
+            }
+        }
+    }
+
+    // ragged tail: T % 8 tokens of the last supergroup, state advances only for t < T
+    // (gemv.cu:648-654)
+    const int ntail = T & 7;
+    if (ntail) {
+        float part[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int v = 0; v < G::NV; v++) {
+            const uint4 u = cb[(size_t)nfull * G::VPS + v];
+            const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+            for (int pp = 0; pp < 2; pp++) {
+                Pair &s = st[2 * v + pp];
+                for (int tt = 0; tt < ntail; tt++) {
+                    const uint32_t na = (w[2 * pp] >> (4 * tt)) & 0xFu;
+                    const uint32_t nb = (w[2 * pp + 1] >> (4 * tt)) & 0xFu;
+                    const h2 qc = codes_to_h2((int)na - 8, (int)nb - 8);
+                    const h2 qs = qc * s.sc;
+                    const float d = __builtin_amdgcn_fdot2(qv[2 * v + pp], qs + s.zp, 0.0f, false);
+#pragma unroll
+                    for (int k = 0; k < 8; k++)
+                        part[k] += (k == tt) ? d : 0.0f;
+                    update_pair(s, qc, qs);
+                }
+            }
+        }
+        reduce_store(part, nfull, ntail);
+    }
+
+    if (state_out != nullptr && active)
+        store_state<D, CPL>(state_out, bx, c0, st);
+
+    h2 deq[G::NP];
+    append_new_token<D, CPL>(cb, T, k_new + (size_t)bx * D + c0, st, deq, active);
+    float self = 0.0f;
+#pragma unroll
+    for (int p = 0; p < G::NP; p++)
+        self = __builtin_amdgcn_fdot2(qv[p], deq[p], self, false);
+    self = head_allreduce<G::LPH>(self);
+    if (active && lh == 0)
+        ob[T] = (h1)self;
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward_ov  (gemv.cu:946-1178)
+// ---------------------------------------------------------------------------------------------
+// acc[c] accumulates w_t * v_hat[t,c].  Within one supergroup the 8 products are summed with packed
+// fp16 fma (as the reference does for the whole sequence, gemv.cu:1087,1096); each supergroup's
+// partial is then added into an fp32 accumulator so the error does not grow with T.
+template <int D, int CPL>
+__global__ __launch_bounds__(BLOCK) void ov_kernel(
+    const h1 *__restrict__ attn, uint4 *__restrict__ cache, const h1 *__restrict__ v_new,
+    h1 *__restrict__ out,
+    const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
+    const h1 *__restrict__ be, const h1 *__restrict__ tg,
+    int BH, int H, int T, int n_super_cap, h1 *__restrict__ state_out)
+{
+    using G = Geo<D, CPL>;
+    const int gl = blockIdx.x * BLOCK + threadIdx.x;
+    int bx = gl / G::LPH;
+    const int lh = gl % G::LPH;
+    const bool active = bx < BH;
+    if (!active)
+        bx = BH - 1;
+    const int h = bx % H;
+    const int c0 = lh * CPL;
+
+    Pair st[G::NP];
+    float acc[CPL];
+#pragma unroll
+    for (int p = 0; p < G::NP; p++) {
+        load_pair(st[p], zp, sc, al, be, tg, h * D + c0 + 2 * p);
+        acc[2 * p] = 0.0f;
+        acc[2 * p + 1] = 0.0f;
+    }
+
+    uint4 *cb = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV;
+    const h1 *wb = attn + (size_t)bx * (T + 1);
+    const int nfull = T >> 3;
+
+    auto load_w = [&](int sg) {
+        uint4 r;
+        __builtin_memcpy(&r, wb + (size_t)sg * 8, 16); // row base is only 2-byte aligned
+        return r;
+    };
+
+    auto decode_sg = [&](const uint4 *u, const uint4 wv) {
+        const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+        for (int v = 0; v < G::NV; v++) {
+            const uint32_t w[4] = {u[v].x, u[v].y, u[v].z, u[v].w};
+#pragma unroll
+            for (int pp = 0; pp < 2; pp++) {
+                Pair &s = st[2 * v + pp];
+                h2 a16 = splat((h1)0.0f);
+                auto row = [&](h2 qe, h2 qo, int br) {
+                    const h2 wp = as_h2(ww[br]);
+                    const h2 qs0 = qe * s.sc;
+                    a16 = pk_fma(splat(wp.x), qs0 + s.zp, a16);
+                    update_pair(s, qe, qs0);
+                    const h2 qs1 = qo * s.sc;
+                    a16 = pk_fma(splat(wp.y), qs1 + s.zp, a16);
+                    update_pair(s, qo, qs1);
+                };
+                h2 qe, qo;
+                unpack_row<0>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 0);
+                unpack_row<1>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 1);
+                unpack_row<2>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 2);
+                unpack_row<3>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 3);
+                acc[4 * v + 2 * pp] += (float)a16.x;
+                acc[4 * v + 2 * pp + 1] += (float)a16.y;
+            }
+        }
+    };
+
+    uint4 buf[PF][G::NV];
+    uint4 wbuf[PF];
+#pragma unroll
+    for (int i = 0; i < PF; i++)
+        if (i < nfull) {
+#pragma unroll
+            for (int v = 0; v < G::NV; v++)
+                buf[i][v] = cb[(size_t)i * G::VPS + v];
+            wbuf[i] = load_w(i);
+        }
+    for (int sg0 = 0; sg0 < nfull; sg0 += PF) {
+#pragma unroll
+        for (int i = 0; i < PF; i++) {
+            const int sg = sg0 + i;
+            if (sg < nfull) {
+                uint4 cur[G::NV];
+#pragma unroll
+                for (int v = 0; v < G::NV; v++)
+                    cur[v] = buf[i][v];
+                const uint4 wcur = wbuf[i];
+                if (sg + PF < nfull) {
+#pragma unroll
+                    for (int v = 0; v < G::NV; v++)
+                        buf[i][v] = cb[(size_t)(sg + PF) * G::VPS + v];
+                    wbuf[i] = load_w(sg + PF);
+                }
+                decode_sg(cur, wcur);
+            }
+        }
+    }
+
+    const int ntail = T & 7;
+    if (ntail) {
+#pragma unroll
+        for (int v = 0; v < G::NV; v++) {
+            const uint4 u = cb[(size_t)nfull * G::VPS + v];
+            const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+            for (int pp = 0; pp < 2; pp++) {
+                Pair &s = st[2 * v + pp];
+                for (int tt = 0; tt < ntail; tt++) {
+                    const uint32_t na = (w[2 * pp] >> (4 * tt)) & 0xFu;
+                    const uint32_t nb = (w[2 * pp + 1] >> (4 * tt)) & 0xFu;
+                    const h2 qc = codes_to_h2((int)na - 8, (int)nb - 8);
+                    const h2 qs = qc * s.sc;
+                    const h2 vd = qs + s.zp;
+                    const float wt = (float)wb[nfull * 8 + tt];
+                    acc[4 * v + 2 * pp] += wt * (float)vd.x;
+                    acc[4 * v + 2 * pp + 1] += wt * (float)vd.y;
+                    update_pair(s, qc, qs);
+                }
+            }
+        }
+    }
+
+    if (state_out != nullptr && active)
+        store_state<D, CPL>(state_out, bx, c0, st);
+
+    h2 deq[G::NP];
+    append_new_token<D, CPL>(cb, T, v_new + (size_t)bx * D + c0, st, deq, active);
+    const float wT = (float)wb[T];
+    if (active) {
+        h2 *o = reinterpret_cast<h2 *>(out + (size_t)bx * D + c0);
+#pragma unroll
+        for (int p = 0; p < G::NP; p++) {
+            const float o0 = acc[2 * p] + wT * (float)deq[p].x;
+            const float o1 = acc[2 * p + 1] + wT * (float)deq[p].y;
+            o[p] = (h2){(h1)o0, (h1)o1};
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// softmax(float(logits)*scaling + mask) -> fp16   (llama_adkv.py:266-271)
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float block_reduce(float v, float *sm, bool is_max)
+{
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) {
+        const float o = __shfl_xor(v, m, 64);
+        v = is_max ? fmaxf(v, o) : v + o;
+    }
+    const int w = threadIdx.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0)
+        sm[w] = v;
+    __syncthreads();
+    float r = sm[0];
+#pragma unroll
+    for (int i = 1; i < BLOCK / 64; i++)
+        r = is_max ? fmaxf(r, sm[i]) : r + sm[i];
+    return r;
+}
+
+__global__ __launch_bounds__(BLOCK) void softmax_kernel(
+    const h1 *__restrict__ logits, h1 *__restrict__ weights, const float *__restrict__ mask,
+    int n, int rows_per_mask_row, float scaling)
+{
+    __shared__ float sm[BLOCK / 64];
+    const int row = blockIdx.x;
+    const h1 *l = logits + (size_t)row * n;
+    h1 *w = weights + (size_t)row * n;
+    const float *mk = mask ? mask + (size_t)(row / rows_per_mask_row) * n : nullptr;
+
+    float mx = -INFINITY;
+    for (int i = threadIdx.x; i < n; i += BLOCK) {
+        float x = (float)l[i] * scaling;
+        if (mk)
+            x += mk[i];
+        mx = fmaxf(mx, x);
+    }
+    mx = block_reduce(mx, sm, true);
+    float sum = 0.0f;
+    for (int i = threadIdx.x; i < n; i += BLOCK) {
+        float x = (float)l[i] * scaling;
+        if (mk)
+            x += mk[i];
+        sum += __expf(x - mx);
+    }
+    sum = block_reduce(sum, sm, false);
+    const float inv = 1.0f / sum;
+    for (int i = threadIdx.x; i < n; i += BLOCK) {
+        float x = (float)l[i] * scaling;
+        if (mk)
+            x += mk[i];
+        w[i] = (h1)(__expf(x - mx) * inv);
+    }
+}
+
+} // namespace adkv
+
+// ---------------------------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------------------------
+using namespace adkv;
+
+static thread_local int g_last_hip_error = 0;
+
+static int check_launch()
+{
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        g_last_hip_error = (int)e;
+        return ADKV_E_LAUNCH;
+    }
+    return ADKV_OK;
+}
+
+static int check_common(int B, int H, int T, int D, int n_super_cap)
+{
+    if (B <= 0 || H <= 0 || T < 0 || n_super_cap <= 0)
+        return ADKV_E_SHAPE;
+    if (D != 128 && D != 256 && D != 512)
+        return ADKV_E_DIM;
+    if ((int64_t)B * H > (int64_t)INT32_MAX / 64)
+        return ADKV_E_SHAPE;
+    return ADKV_OK;
+}
+
+static inline dim3 grid_for(int BH, int lph)
+{
+    return dim3((unsigned)(((int64_t)BH * lph + BLOCK - 1) / BLOCK));
+}
+
+#define ADKV_DISPATCH_D(KERNEL, ...)                                                          \
+    switch (D) {                                                                              \
+    case 128:                                                                                 \
+        hipLaunchKernelGGL((KERNEL<128, 4>), grid_for(BH, 32), dim3(BLOCK), 0, st, __VA_ARGS__); \
+        break;                                                                                \
+    case 256:                                                                                 \
+        hipLaunchKernelGGL((KERNEL<256, 4>), grid_for(BH, 64), dim3(BLOCK), 0, st, __VA_ARGS__); \
+        break;                                                                                \
+    default:                                                                                  \
+        hipLaunchKernelGGL((KERNEL<512, 8>), grid_for(BH, 64), dim3(BLOCK), 0, st, __VA_ARGS__); \
+        break;                                                                                \
+    }
+
+extern "C" {
+
+int adkv_abi_version(void) { return 1; }
+
+int adkv_last_hip_error(void) { return g_last_hip_error; }
+
+const char *adkv_strerror(int code)
+{
+    switch (code) {
+    case ADKV_OK: return "ok";
+    case ADKV_E_NULL: return "required pointer is NULL";
+    case ADKV_E_DIM: return "DIM must be 128, 256 or 512";
+    case ADKV_E_SHAPE: return "invalid shape";
+    case ADKV_E_CAPACITY: return "cache capacity too small";
+    case ADKV_E_ALIGN: return "pointer not sufficiently aligned";
+    case ADKV_E_UNSUPPORTED: return "unsupported configuration";
+    case ADKV_E_LAUNCH: return "HIP launch failed";
+    default: return "unknown error";
+    }
+}
+
+int adkv_encode_kv(void *cache, const void *kv_new,
+                   const void *zp, const void *sc, const void *alpha, const void *beta,
+                   const void *tgt,
+                   int B, int H, int T, int D, int n_super_cap,
+                   float, float, void *state_out, void *stream)
+{
+    if (!cache || !kv_new || !zp || !sc || !alpha || !beta || !tgt)
+        return ADKV_E_NULL;
+    int rc = check_common(B, H, T, D, n_super_cap);
+    if (rc)
+        return rc;
+    if ((T + 7) / 8 > n_super_cap)
+        return ADKV_E_CAPACITY;
+    if (((uintptr_t)cache & 15) || ((uintptr_t)kv_new & 3))
+        return ADKV_E_ALIGN;
+    if (T == 0 && state_out == nullptr)
+        return ADKV_OK;
+    const int BH = B * H;
+    hipStream_t st = (hipStream_t)stream;
+    ADKV_DISPATCH_D(encode_kernel, (uint4 *)cache, (const h1 *)kv_new, (const h1 *)zp,
+                    (const h1 *)sc, (const h1 *)alpha, (const h1 *)beta, (const h1 *)tgt, BH, H, T,
+                    n_super_cap, (h1 *)state_out);
+    return check_launch();
+}
+
+int adkv_forward_qk(const void *q, void *k_cache, const void *k_new, void *logits,
+                    const void *zp, const void *sc, const void *alpha, const void *beta,
+                    const void *tgt,
+                    int B, int H, int T, int D, int n_super_cap,
+                    float, float, void *state_out, void *stream)
+{
+    if (!q || !k_cache || !k_new || !logits || !zp || !sc || !alpha || !beta || !tgt)
+        return ADKV_E_NULL;
+    int rc = check_common(B, H, T, D, n_super_cap);
+    if (rc)
+        return rc;
+    if ((T >> 3) >= n_super_cap)
+        return ADKV_E_CAPACITY;
+    if (((uintptr_t)k_cache & 15) || ((uintptr_t)q & 3) || ((uintptr_t)k_new & 3))
+        return ADKV_E_ALIGN;
+    const int BH = B * H;
+    hipStream_t st = (hipStream_t)stream;
+    ADKV_DISPATCH_D(qk_kernel, (const h1 *)q, (uint4 *)k_cache, (const h1 *)k_new, (h1 *)logits,
+                    (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha, (const h1 *)beta,
+                    (const h1 *)tgt, BH, H, T, n_super_cap, (h1 *)state_out);
+    return check_launch();
+}
+
+int adkv_forward_ov(const void *attn, void *v_cache, const void *v_new, void *out,
+                    const void *zp, const void *sc, const void *alpha, const void *beta,
+                    const void *tgt,
+                    int B, int H, int T, int D, int n_super_cap,
+                    float, float, void *state_out, void *stream)
+{
+    if (!attn || !v_cache || !v_new || !out || !zp || !sc || !alpha || !beta || !tgt)
+        return ADKV_E_NULL;
+    int rc = check_common(B, H, T, D, n_super_cap);
+    if (rc)
+        return rc;
+    if ((T >> 3) >= n_super_cap)
+        return ADKV_E_CAPACITY;
+    if (((uintptr_t)v_cache & 15) || ((uintptr_t)out & 3) || ((uintptr_t)v_new & 3))
+        return ADKV_E_ALIGN;
+    const int BH = B * H;
+    hipStream_t st = (hipStream_t)stream;
+    ADKV_DISPATCH_D(ov_kernel, (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new, (h1 *)out,
+                    (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha, (const h1 *)beta,
+                    (const h1 *)tgt, BH, H, T, n_super_cap, (h1 *)state_out);
+    return check_launch();
+}
+
+int adkv_softmax(const void *logits, void *weights, const void *mask,
+                 int rows, int n, int rows_per_mask_row, float scaling, void *stream)
+{
+    if (!logits || !weights)
+        return ADKV_E_NULL;
+    if (rows <= 0 || n <= 0 || (mask && rows_per_mask_row <= 0))
+        return ADKV_E_SHAPE;
+    hipLaunchKernelGGL(softmax_kernel, dim3((unsigned)rows), dim3(BLOCK), 0, (hipStream_t)stream,
+                       (const h1 *)logits, (h1 *)weights, (const float *)mask, n,
+                       mask ? rows_per_mask_row : 1, scaling);
+    return check_launch();
+}
+
+} // extern "C"

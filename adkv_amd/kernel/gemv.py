@@ -1,0 +1,246 @@
+"""Drop-in for the reference's ``adkv.kernel.gemv`` (src/adkv/kernel/gemv.py:16-132).
+
+Same three functions, same argument order, same tensor layouts and the same error messages as the
+reference's C++ bindings (src/adkv/kernel/gemv.cu:368-414, 883-939, 1233-1288); the work is done
+by hand-written gfx950 kernels behind ``libadkv_hip.so``.  Differences, all on the safe side:
+
+* launches go to PyTorch's *current* stream (the reference uses legacy stream 0);
+* an unsupported head dim raises in ``forward_qk`` / ``forward_ov`` too (the reference's launcher
+  silently skips the launch and returns uninitialised memory, gemv.cu:875-878, 1226-1229);
+* logits and outputs are accumulated in fp32 and rounded once to fp16 (the reference accumulates in
+  fp16); codes written to the cache and the filter state are bit-identical.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+
+_TILE = 4
+_DIMS = (128, 256, 512)
+
+
+def _chk(cond: bool, msg: str) -> None:
+    # TORCH_CHECK surfaces as RuntimeError in Python
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _need_device(*tensors: torch.Tensor) -> torch.device:
+    dev = tensors[0].device
+    for t in tensors:
+        _chk(t.is_cuda, "ADKV kernels need every tensor on a HIP device; there is no CPU path")
+        _chk(t.device == dev, "ADKV kernels need all tensors on the same device")
+    return dev
+
+
+def _params(tensors, names, nh, dim):
+    out = []
+    for t, n in zip(tensors, names):
+        _chk(t.dtype == torch.float16, f"{n} must be float16")
+        out.append(t)
+    res = []
+    for t, n in zip(out, names):
+        _chk(t.numel() == nh * dim, f"{n} must have nh*DIM = {nh * dim} elements")
+        res.append(t.contiguous())
+    return res
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def forward_qk(
+    q: torch.Tensor,
+    k_cache: torch.Tensor,
+    k_new: torch.Tensor,
+    k_zp: torch.Tensor,
+    k_sc: torch.Tensor,
+    k_alpha: torch.Tensor,
+    k_beta: torch.Tensor,
+    k_t: torch.Tensor,
+    T: int,
+    scale_min: float,
+    scale_max: float,
+    *,
+    state_out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Decode-phase QK^T over the nibble-packed ADKV cache (reference gemv.py:16-55).
+
+    ``o[b,h,t] = sum_c q[b,h,c] * k_deq[b,h,t,c]`` for the ``T`` cached tokens; then ``k_new`` is
+    quantised with the filter state after token ``T-1`` and written at position ``T`` in place, and
+    its own logit is returned as the last element.
+
+    Args:
+        q, k_new: ``[B, nh, 1, DIM]`` float16.
+        k_cache:  ``[B, nh, n_super_cap, DIM/4, 4, 4]`` uint8, contiguous, appended in place.
+        k_zp, k_sc, k_alpha, k_beta, k_t: ``[nh, DIM]`` float16 ADKV parameters.
+        T: number of cached tokens.
+        scale_min, scale_max: kept for API compatibility (unused by the fp16 recurrence).
+        state_out: optional ``[B, nh, DIM, 2]`` float16, receives (zp, sc) after token ``T-1``
+            (extension; not in the reference).
+
+    Returns ``[B, nh, T+1]`` float16 logits.
+    """
+    _chk(q.dtype == torch.float16, "q must be float16")
+    _chk(k_new.dtype == torch.float16, "k_new must be float16")
+    _chk(k_cache.dtype == torch.uint8, "k_cache must be uint8")
+    _chk(k_cache.is_contiguous(), "k_cache must be contiguous (appended in place)")
+    B, nh = q.shape[0], q.shape[1]
+    n_super_cap, n_cgroup = k_cache.shape[2], k_cache.shape[3]
+    DIM = n_cgroup * _TILE
+    zp, sc, al, be, tg = _params((k_zp, k_sc, k_alpha, k_beta, k_t),
+                                 ("k_zp", "k_sc", "k_alpha", "k_beta", "k_t"), nh, DIM)
+    _chk(DIM == q.shape[3], "q head dimension does not match k_cache")
+    _chk(T >= 0, "T must be non-negative")
+    _chk((T >> 1) // _TILE < n_super_cap, f"k_cache has no free supergroup to append token {T}")
+    _chk(DIM in _DIMS, "DIM must be 128, 256 or 512")
+    dev = _need_device(q, k_cache, k_new, zp, sc, al, be, tg)
+
+    q_flat = q.contiguous()
+    k_new_flat = k_new.reshape(B * nh, DIM).contiguous()
+    o = torch.empty((B * nh, T + 1), dtype=torch.float16, device=dev)
+    if state_out is not None:
+        _chk(state_out.dtype == torch.float16 and state_out.is_contiguous()
+             and state_out.numel() == B * nh * DIM * 2, "state_out must be contiguous fp16 [B,nh,DIM,2]")
+    with torch.cuda.device(dev):
+        rc = _lib.lib().adkv_forward_qk(
+            q_flat.data_ptr(), k_cache.data_ptr(), k_new_flat.data_ptr(), o.data_ptr(),
+            zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
+            B, nh, T, DIM, n_super_cap, float(scale_min), float(scale_max),
+            _ptr(state_out), _lib.current_stream_ptr(dev))
+    _lib.check(rc, "forward_qk")
+    return o.reshape(B, nh, T + 1)
+
+
+def forward_ov(
+    attn: torch.Tensor,
+    v_cache: torch.Tensor,
+    v_new: torch.Tensor,
+    v_zp: torch.Tensor,
+    v_sc: torch.Tensor,
+    v_alpha: torch.Tensor,
+    v_beta: torch.Tensor,
+    v_t: torch.Tensor,
+    scale_min: float,
+    scale_max: float,
+    *,
+    state_out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Decode-phase OV over the nibble-packed ADKV cache (reference gemv.py:58-97).
+
+    ``o[b,h,c] = sum_t attn[b,h,t] * v_deq[b,h,t,c]`` over the ``T = attn.shape[2]-1`` cached
+    tokens plus ``attn[T] * v_deq_new``; ``v_new`` is quantised with the state after token ``T-1``
+    and written at position ``T`` in place.
+
+    Returns ``[B, nh, DIM]`` float16.
+    """
+    _chk(attn.dtype == torch.float16, "attn must be float16")
+    _chk(v_new.dtype == torch.float16, "v_new must be float16")
+    _chk(v_cache.dtype == torch.uint8, "v_cache must be uint8")
+    _chk(v_cache.is_contiguous(), "v_cache must be contiguous (appended in place)")
+    B, nh = attn.shape[0], attn.shape[1]
+    _chk(attn.shape[2] >= 1, "attn must contain the cached weights plus the self weight")
+    T = attn.shape[2] - 1
+    n_super_cap, n_cgroup = v_cache.shape[2], v_cache.shape[3]
+    DIM = n_cgroup * _TILE
+    zp, sc, al, be, tg = _params((v_zp, v_sc, v_alpha, v_beta, v_t),
+                                 ("v_zp", "v_sc", "v_alpha", "v_beta", "v_t"), nh, DIM)
+    _chk(DIM == v_new.shape[-1], "v_new head dimension does not match v_cache")
+    _chk(T >= 0, "T must be non-negative")
+    _chk((T >> 1) // _TILE < n_super_cap, f"v_cache has no free supergroup to append token {T}")
+    _chk(DIM in _DIMS, "DIM must be 128, 256 or 512")
+    dev = _need_device(attn, v_cache, v_new, zp, sc, al, be, tg)
+
+    attn_flat = attn.contiguous()
+    v_new_flat = v_new.reshape(B * nh, DIM).contiguous()
+    o = torch.empty((B * nh, DIM), dtype=torch.float16, device=dev)
+    if state_out is not None:
+        _chk(state_out.dtype == torch.float16 and state_out.is_contiguous()
+             and state_out.numel() == B * nh * DIM * 2, "state_out must be contiguous fp16 [B,nh,DIM,2]")
+    with torch.cuda.device(dev):
+        rc = _lib.lib().adkv_forward_ov(
+            attn_flat.data_ptr(), v_cache.data_ptr(), v_new_flat.data_ptr(), o.data_ptr(),
+            zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
+            B, nh, T, DIM, n_super_cap, float(scale_min), float(scale_max),
+            _ptr(state_out), _lib.current_stream_ptr(dev))
+    _lib.check(rc, "forward_ov")
+    return o.view(attn.shape[0], attn.shape[1], -1)
+
+
+def encode_kv(
+    kv_cache: torch.Tensor,
+    kv_new: torch.Tensor,
+    kv_zp: torch.Tensor,
+    kv_sc: torch.Tensor,
+    kv_alpha: torch.Tensor,
+    kv_beta: torch.Tensor,
+    kv_t: torch.Tensor,
+    scale_min: float,
+    scale_max: float,
+    *,
+    state_out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Prefill: quantise tokens ``[0, T)`` into the uint4-tiled KV cache (reference gemv.py:100-132).
+
+    Replays the ADKV filter from ``(kv_zp, kv_sc)``; token ``t`` goes to byte row ``t/2``, low
+    nibble for even ``t`` and high nibble for odd ``t``.  Purely in place; returns ``kv_cache``.
+    """
+    _chk(kv_new.dtype == torch.float16, "kv_new must be float16")
+    _chk(kv_cache.dtype == torch.uint8, "kv_cache must be uint8")
+    _chk(kv_cache.is_contiguous(), "kv_cache must be contiguous (written in place)")
+    B, nh, T, DIM = kv_new.shape
+    zp, sc, al, be, tg = _params((kv_zp, kv_sc, kv_alpha, kv_beta, kv_t),
+                                 ("kv_zp", "kv_sc", "kv_alpha", "kv_beta", "kv_t"), nh, DIM)
+    n_super_cap = kv_cache.shape[2]
+    _chk(kv_cache.shape[3] * _TILE == DIM, "kv_cache channel groups do not match kv_new head dim")
+    n_super = ((T + 1) // 2 + _TILE - 1) // _TILE
+    _chk(n_super <= n_super_cap,
+         f"kv_cache capacity too small: need {n_super} supergroups for {T} tokens, have {n_super_cap}")
+    _chk(DIM in _DIMS, "DIM must be 128, 256 or 512")
+    dev = _need_device(kv_cache, kv_new, zp, sc, al, be, tg)
+
+    kv_new_flat = kv_new.contiguous()
+    if state_out is not None:
+        _chk(state_out.dtype == torch.float16 and state_out.is_contiguous()
+             and state_out.numel() == B * nh * DIM * 2, "state_out must be contiguous fp16 [B,nh,DIM,2]")
+    if B * nh * T == 0 and state_out is None:
+        return kv_cache
+    with torch.cuda.device(dev):
+        rc = _lib.lib().adkv_encode_kv(
+            kv_cache.data_ptr(), kv_new_flat.data_ptr(),
+            zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
+            B, nh, T, DIM, n_super_cap, float(scale_min), float(scale_max),
+            _ptr(state_out), _lib.current_stream_ptr(dev))
+    _lib.check(rc, "encode_kv")
+    return kv_cache
+
+
+def softmax_scale_mask(logits: torch.Tensor, scaling: float,
+                       mask: torch.Tensor | None = None) -> torch.Tensor:
+    """``softmax(logits.float()*scaling + mask) -> fp16`` in one launch.
+
+    Fuses the element-wise chain the reference runs in torch between the two GEMVs
+    (src/adkv/hf/llama_adkv.py:266-271).  ``logits``: fp16 ``[B, nh, n]``; ``mask``: optional
+    ``[B, 1, n]`` / ``[B, nh, n]`` / ``[B, 1, 1, n]`` additive mask (any float dtype).
+    """
+    _chk(logits.dtype == torch.float16, "logits must be float16")
+    _chk(logits.dim() == 3, "logits must be [B, nh, n]")
+    B, nh, n = logits.shape
+    dev = _need_device(logits)
+    lg = logits.contiguous()
+    out = torch.empty_like(lg)
+    rpm, mptr = 1, None
+    mk = None
+    if mask is not None:
+        mk = mask[:, :, 0, :] if mask.dim() == 4 else mask
+        _chk(mk.dim() == 3 and mk.shape[0] == B and mk.shape[2] == n and mk.shape[1] in (1, nh),
+             "mask must broadcast to [B, nh, n]")
+        rpm = nh if mk.shape[1] == 1 else 1
+        mk = mk.to(device=dev, dtype=torch.float32).contiguous()
+        mptr = mk.data_ptr()
+    with torch.cuda.device(dev):
+        rc = _lib.lib().adkv_softmax(lg.data_ptr(), out.data_ptr(), mptr, B * nh, n, rpm,
+                                     float(scaling), _lib.current_stream_ptr(dev))
+    _lib.check(rc, "softmax_scale_mask")
+    return out

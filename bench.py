@@ -1,0 +1,197 @@
+#!/usr/bin/env python3
+"""Headline benchmark: ADKV decode attention, Llama-2-7B shape, one MI355X.
+
+One "step" is one layer's decode-attention for a batch: forward_qk (+append) -> softmax ->
+forward_ov (+append) over a resident 4-bit K/V cache, the protocol of the reference's
+tools/perf_kernel.py:28-76.  Throughput follows its convention (perf_kernel.py:91-104):
+tokens/s = B / (32 layers * seconds per layer-step).  Caches are produced by running the encoder
+on seeded synthetic K/V (closed loop), and the timed steps rotate over several distinct layer
+buffers so no cache level can serve re-reads.
+
+Prints ONE JSON line.  `roofline` prices the dominant kernel (the QK scan) on its algorithmic
+bytes, B*H*T*d*bits/8 code bytes per launch, against the 8 TB/s HBM peak; `cpu_baseline` times the
+C oracle of the same step on a bounded sample on the host.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+N_LAYERS_MODEL = 32
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=40)
+    ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--batch", type=int, default=128)
+    ap.add_argument("--heads", type=int, default=32)
+    ap.add_argument("--dim", type=int, default=128)
+    ap.add_argument("--ctx", type=int, default=4096)
+    ap.add_argument("--layer-buffers", type=int, default=4,
+                    help="distinct K/V caches rotated through (defeats on-die cache reuse)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-heads", type=int, default=0,
+                    help="heads of one sequence timed on the host (0 = auto, about 10-30 s)")
+    return ap.parse_args()
+
+
+def cpu_baseline(args, T, D):
+    """C oracle (a scalar port of the same fp16 recurrence) timed on one host core over a sample:
+    `hs` heads of one sequence, full context; scaled to a whole sequence of H heads."""
+    import numpy as np
+    import torch
+    from adkv_amd import synth
+    from oracle import oracle as O
+
+    H = args.heads
+    hs = args.cpu_sample_heads or min(H, 16)
+    kp, vp = synth.make_params(H, D, seed=3), synth.make_params(H, D, seed=4)
+    np16 = lambda t: t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.float16)
+    kpn = [np16(t)[:hs] for t in kp.astuple()]
+    vpn = [np16(t)[:hs] for t in vp.astuple()]
+    k = np16(synth.make_k(1, hs, T + 1, D, dtype=torch.float16))
+    v = np16(synth.make_v(1, hs, T + 1, D, dtype=torch.float16))
+    q = np16(synth.make_q(1, hs, D))
+    kc, vc = O.alloc_cache(1, hs, T + 8, D), O.alloc_cache(1, hs, T + 8, D)
+    O.encode_kv_f16(kc, k[:, :, :T], *kpn)
+    O.encode_kv_f16(vc, v[:, :, :T], *vpn)
+    t0 = time.perf_counter()
+    O.decode_step_f16(q, kc, vc, k[:, :, T:], v[:, :, T:], kpn, vpn, T, D ** -0.5)
+    dt = time.perf_counter() - t0
+    t_seq = dt * (H / hs)                      # one layer-step for one whole sequence
+    return {
+        "value": 1.0 / (N_LAYERS_MODEL * t_seq),
+        "unit": "tokens/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": f"C oracle, 1 sequence x {hs} of {H} heads x ctx {T}, one layer-step = {dt:.2f} s; "
+                  f"scaled linearly to {H} heads",
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (the path shards over batch/heads with no "
+              "exchange; nothing multi-GPU is built). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from adkv_amd import synth
+    from adkv_amd.kernel import gemv
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    B, H, D, T = args.batch, args.heads, args.dim, args.ctx
+    smin, smax = math.exp(-4.0), math.exp(4.0)
+    NL = args.layer_buffers
+
+    kps, vps, kcs, vcs = [], [], [], []
+    for l in range(NL):
+        kp = synth.make_params(H, D, seed=3, layer=l).to(dev)
+        vp = synth.make_params(H, D, seed=4, layer=l).to(dev)
+        kc = synth.alloc_cache(B, H, T + 8, D, dev)
+        vc = synth.alloc_cache(B, H, T + 8, D, dev)
+        x = synth.make_k(B, H, T, D, layer=l, dtype=torch.float16, device=dev)
+        gemv.encode_kv(kc, x, *kp.astuple(), smin, smax)
+        del x
+        x = synth.make_v(B, H, T, D, layer=l, dtype=torch.float16, device=dev)
+        gemv.encode_kv(vc, x, *vp.astuple(), smin, smax)
+        del x
+        kps.append(kp.astuple()); vps.append(vp.astuple()); kcs.append(kc); vcs.append(vc)
+    q = synth.make_q(B, H, D, device=dev)
+    k_new = synth.make_k(B, H, 1, D, seed=11, dtype=torch.float16, device=dev, t0=T)
+    v_new = synth.make_v(B, H, 1, D, seed=12, dtype=torch.float16, device=dev)
+    scaling = D ** -0.5
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    marks = []
+
+    def step(i, timed):
+        l = i % NL
+        if timed:
+            e = [ev() for _ in range(4)]
+            e[0].record()
+        logits = gemv.forward_qk(q, kcs[l], k_new, *kps[l], T, smin, smax)
+        if timed:
+            e[1].record()
+        w = gemv.softmax_scale_mask(logits, scaling)
+        if timed:
+            e[2].record()
+        out = gemv.forward_ov(w, vcs[l], v_new, *vps[l], smin, smax)
+        if timed:
+            e[3].record()
+            marks.append(e)
+        return out
+
+    for i in range(args.warmup):
+        step(i, False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i, True)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    ms_step = wall * 1e3 / args.steps
+    qk_ms = sum(e[0].elapsed_time(e[1]) for e in marks) / len(marks)
+    sm_ms = sum(e[1].elapsed_time(e[2]) for e in marks) / len(marks)
+    ov_ms = sum(e[2].elapsed_time(e[3]) for e in marks) / len(marks)
+    dev_ms = sorted(e[0].elapsed_time(e[3]) for e in marks)[len(marks) // 2]
+
+    code_bytes = B * H * T * D * 0.5                    # one tensor's codes: bytes per QK launch
+    achieved = code_bytes / (qk_ms * 1e-3) / 1e9
+    tokens_s = B / (N_LAYERS_MODEL * ms_step * 1e-3)
+
+    res = {
+        "metric": "decode-attention tokens/sec (B / (32 layers * layer-step time))",
+        "value": tokens_s,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"cfg2 Llama-2-7B-shaped ADKV decode attention: B={B} H={H} d={D} ctx={T} "
+                        f"4-bit K+V codes, step = forward_qk+softmax+forward_ov, {NL} rotating layer caches",
+            "batch": B, "heads": H, "head_dim": D, "ctx": T, "bits": 4,
+            "parallelism": "1 GPU",
+        },
+        "kernel_ms": {"forward_qk": qk_ms, "softmax": sm_ms, "forward_ov": ov_ms,
+                      "step_device_median": dev_ms},
+        "step_code_GBps": 2 * code_bytes / (ms_step * 1e-3) / 1e9,
+        "roofline": {
+            "kernel": "qk_kernel<128,4>",
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS,
+            "traffic": None,
+        },
+    }
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(args, T, D)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,90 @@
+/*
+ * libadkv_hip — C ABI of the MI355X (gfx950) ADKV hot path.
+ *
+ * Plain pointers and sizes only: every pointer is a DEVICE pointer unless stated otherwise, every
+ * fp16 tensor is IEEE binary16, `stream` is a hipStream_t passed as void* (NULL = default stream).
+ * All calls are asynchronous with respect to the host and return 0 on success or a negative
+ * ADKV_E_* code; adkv_strerror() names it.  Nothing here allocates device memory.
+ *
+ * Packed cache layout (reference: src/adkv/hf/llama_adkv.py:47-55, src/adkv/kernel/gemv.cu:502-510):
+ *   uint8 [B, H, n_super_cap, D/4, 4, 4]; one supergroup = 8 tokens; viewed as 32-bit words, word
+ *   (sg, c) holds channel c's eight 4-bit codes, code of token 8*sg+i at bits 4i..4i+3, code = q+8.
+ * Parameter tensors zp/sc/alpha/beta/tgt are fp16 [H, D].
+ */
+#ifndef ADKV_HIP_H
+#define ADKV_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ADKV_OK 0
+#define ADKV_E_NULL (-1)       /* a required pointer is NULL */
+#define ADKV_E_DIM (-2)        /* head dim not in {128, 256, 512} */
+#define ADKV_E_SHAPE (-3)      /* negative / zero sizes */
+#define ADKV_E_CAPACITY (-4)   /* cache has too few supergroups */
+#define ADKV_E_ALIGN (-5)      /* pointer alignment requirement violated */
+#define ADKV_E_UNSUPPORTED (-6)
+#define ADKV_E_LAUNCH (-100)   /* HIP reported a launch error; see adkv_last_hip_error() */
+
+/* ABI version of this header; bumped on any signature change. */
+int adkv_abi_version(void);
+const char *adkv_strerror(int code);
+/* hipError_t (as int) of the last failed launch in this thread, 0 if none. */
+int adkv_last_hip_error(void);
+
+/*
+ * Prefill quantise: tokens [0,T) of kv_new [B,H,T,D] fp16 -> codes, starting from (zp, sc).
+ * Replaces encode_kv (src/adkv/kernel/gemv.cu:368-414, kernel :168-308; Python wrapper
+ * src/adkv/kernel/gemv.py:100-132).  Whole supergroups [0, ceil(T/8)) are overwritten.
+ * scale_min/scale_max are accepted for signature parity and ignored, as the reference kernel does.
+ * state_out (optional, may be NULL): fp16 [B,H,D,2] = (zp, sc) after token T-1.
+ */
+int adkv_encode_kv(void *cache, const void *kv_new,
+                   const void *zp, const void *sc, const void *alpha, const void *beta,
+                   const void *tgt,
+                   int B, int H, int T, int D, int n_super_cap,
+                   float scale_min, float scale_max,
+                   void *state_out, void *stream);
+
+/*
+ * Decode q.K^T over T cached tokens, then quantise k_new with the state after token T-1, write it
+ * at slot T in place and emit its self logit.  logits: fp16 [B,H,T+1].
+ * Replaces forward_qk (src/adkv/kernel/gemv.cu:883-939, kernel :435-815; gemv.py:16-55).
+ * q, k_new: fp16 [B,H,D] (the reference's [B,H,1,D] made contiguous).
+ * state_out (optional): fp16 [B,H,D,2] state after token T-1 (the state k_new was quantised with).
+ */
+int adkv_forward_qk(const void *q, void *k_cache, const void *k_new, void *logits,
+                    const void *zp, const void *sc, const void *alpha, const void *beta,
+                    const void *tgt,
+                    int B, int H, int T, int D, int n_super_cap,
+                    float scale_min, float scale_max,
+                    void *state_out, void *stream);
+
+/*
+ * Decode P.V: out[b,h,:] = sum_{t<T} attn[t]*v_hat[t,:] + attn[T]*v_hat_new, appending v_new at
+ * slot T in place.  attn: fp16 [B,H,T+1]; out: fp16 [B,H,D].
+ * Replaces forward_ov (src/adkv/kernel/gemv.cu:1233-1288, kernel :946-1178; gemv.py:58-97).
+ */
+int adkv_forward_ov(const void *attn, void *v_cache, const void *v_new, void *out,
+                    const void *zp, const void *sc, const void *alpha, const void *beta,
+                    const void *tgt,
+                    int B, int H, int T, int D, int n_super_cap,
+                    float scale_min, float scale_max,
+                    void *state_out, void *stream);
+
+/*
+ * weights = softmax(float(logits) * scaling + mask) over the last axis, written as fp16.
+ * Replaces the torch ops between the two GEMVs (src/adkv/hf/llama_adkv.py:266-271).
+ * logits, weights: fp16 [rows, n]; mask (optional, NULL = none): fp32 [mask_rows, n] with row r of
+ * logits using mask row (r / rows_per_mask_row) — pass rows_per_mask_row = H for a [B,1,1,n] mask.
+ */
+int adkv_softmax(const void *logits, void *weights, const void *mask,
+                 int rows, int n, int rows_per_mask_row, float scaling, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,140 @@
+"""CPU-only checks of the boundary: the C-ABI library loads and exports every symbol the public
+header declares, and the Python drop-in raises the reference's error messages
+(src/adkv/kernel/gemv.cu:375-398, 892-912, 1241-1266) before touching a device."""
+import ctypes
+import math
+import os
+import re
+
+import pytest
+import torch
+
+from adkv_amd import _lib
+from adkv_amd.kernel import gemv
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SMIN, SMAX = math.exp(-4.0), math.exp(4.0)
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "adkv_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(adkv_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_symbols()
+    assert {"adkv_encode_kv", "adkv_forward_qk", "adkv_forward_ov", "adkv_softmax"} <= set(names)
+    L = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(L, n), f"{n} declared in include/adkv_hip.h but not exported"
+    assert set(names) == set(_lib.PROTOTYPES), "ctypes prototypes out of sync with the header"
+
+
+def test_abi_version_and_strerror():
+    L = _lib.lib()
+    assert L.adkv_abi_version() == _lib.ABI_VERSION
+    assert L.adkv_strerror(0) == b"ok"
+    assert b"128, 256 or 512" in L.adkv_strerror(-2)
+
+
+def test_argument_validation_in_c_abi_needs_no_device():
+    """NULL pointers, bad dims and capacity are rejected on the host before any launch."""
+    L = _lib.lib()
+    one = ctypes.c_void_p(16)
+    args = lambda D, T, cap: [one] * 7 + [1, 1, T, D, cap, 0.0, 1.0, None, None]
+    assert L.adkv_encode_kv(*([None] + args(128, 8, 1)[1:])) == -1
+    assert L.adkv_encode_kv(*args(64, 8, 1)) == -2
+    assert L.adkv_encode_kv(*args(128, 9, 1)) == -4
+    assert L.adkv_encode_kv(*args(128, -1, 1)) == -3
+    qk = [one] * 9 + [1, 1, 8, 128, 1, 0.0, 1.0, None, None]
+    assert L.adkv_forward_qk(*qk) == -4          # slot 8 needs a second supergroup
+    qk[12] = 96
+    assert L.adkv_forward_qk(*qk) == -2
+
+
+def _p(nh, D, dtype=torch.float16):
+    return [torch.zeros(nh, D, dtype=dtype) for _ in range(5)]
+
+
+def _cache(B, nh, cap, D):
+    return torch.zeros(B, nh, cap, D // 4, 4, 4, dtype=torch.uint8)
+
+
+def _h(*s):
+    return torch.zeros(*s, dtype=torch.float16)
+
+
+def test_forward_qk_errors():
+    B, nh, D = 1, 2, 128
+    ok = dict(q=_h(B, nh, 1, D), c=_cache(B, nh, 2, D), k=_h(B, nh, 1, D))
+    call = lambda q=None, c=None, k=None, p=None, T=3: gemv.forward_qk(
+        ok["q"] if q is None else q, ok["c"] if c is None else c, ok["k"] if k is None else k,
+        *(_p(nh, D) if p is None else p), T, SMIN, SMAX)
+    with pytest.raises(RuntimeError, match="q must be float16"):
+        call(q=torch.zeros(B, nh, 1, D))
+    with pytest.raises(RuntimeError, match="k_new must be float16"):
+        call(k=torch.zeros(B, nh, 1, D))
+    with pytest.raises(RuntimeError, match="k_cache must be uint8"):
+        call(c=_cache(B, nh, 2, D).to(torch.int8))
+    with pytest.raises(RuntimeError, match="k_cache must be contiguous"):
+        call(c=_cache(B, nh, 4, D)[:, :, ::2])
+    with pytest.raises(RuntimeError, match="k_alpha must be float16"):
+        p = _p(nh, D)
+        p[2] = p[2].float()
+        call(p=p)
+    with pytest.raises(RuntimeError, match="q head dimension does not match k_cache"):
+        call(q=_h(B, nh, 1, 256))
+    with pytest.raises(RuntimeError, match="T must be non-negative"):
+        call(T=-1)
+    with pytest.raises(RuntimeError, match="k_cache has no free supergroup to append token 16"):
+        call(T=16)
+    with pytest.raises(RuntimeError, match="DIM must be 128, 256 or 512"):
+        gemv.forward_qk(_h(B, nh, 1, 64), _cache(B, nh, 2, 64), _h(B, nh, 1, 64), *_p(nh, 64), 3, SMIN, SMAX)
+    # everything valid but on the CPU: loud failure, no fallback
+    with pytest.raises(RuntimeError, match="HIP device"):
+        call()
+
+
+def test_forward_ov_errors():
+    B, nh, D = 1, 2, 128
+    call = lambda a=None, c=None, v=None: gemv.forward_ov(
+        _h(B, nh, 4) if a is None else a, _cache(B, nh, 2, D) if c is None else c,
+        _h(B, nh, 1, D) if v is None else v, *_p(nh, D), SMIN, SMAX)
+    with pytest.raises(RuntimeError, match="attn must be float16"):
+        call(a=torch.zeros(B, nh, 4))
+    with pytest.raises(RuntimeError, match="v_cache must be uint8"):
+        call(c=_cache(B, nh, 2, D).float())
+    with pytest.raises(RuntimeError, match="attn must contain the cached weights plus the self weight"):
+        call(a=_h(B, nh, 0))
+    with pytest.raises(RuntimeError, match="v_new head dimension does not match v_cache"):
+        call(v=_h(B, nh, 1, 256))
+    with pytest.raises(RuntimeError, match="v_cache has no free supergroup to append token 16"):
+        call(a=_h(B, nh, 17))
+    with pytest.raises(RuntimeError, match="HIP device"):
+        call()
+
+
+def test_encode_kv_errors():
+    B, nh, D = 1, 2, 128
+    call = lambda c=None, x=None: gemv.encode_kv(
+        _cache(B, nh, 2, D) if c is None else c, _h(B, nh, 9, D) if x is None else x,
+        *_p(nh, D), SMIN, SMAX)
+    with pytest.raises(RuntimeError, match="kv_new must be float16"):
+        call(x=torch.zeros(B, nh, 9, D))
+    with pytest.raises(RuntimeError, match="kv_cache must be contiguous \\(written in place\\)"):
+        call(c=_cache(B, nh, 4, D)[:, :, ::2])
+    with pytest.raises(RuntimeError, match="kv_cache channel groups do not match kv_new head dim"):
+        call(c=_cache(B, nh, 2, 256))
+    with pytest.raises(RuntimeError,
+                       match="kv_cache capacity too small: need 3 supergroups for 17 tokens, have 2"):
+        call(x=_h(B, nh, 17, D))
+    with pytest.raises(RuntimeError, match="HIP device"):
+        call()
+
+
+def test_missing_library_is_loud(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_lib.ADKVLibraryError, match="no CPU fallback"):
+        _lib.lib()
