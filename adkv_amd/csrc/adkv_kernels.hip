@@ -311,9 +311,8 @@ __global__ __launch_bounds__(BLOCK) void qk_kernel(
 // ---------------------------------------------------------------------------------------------
 // forward_ov  (gemv.cu:946-1178)
 // ---------------------------------------------------------------------------------------------
-// acc[c] accumulates w_t * v_hat[t,c].  Within one supergroup the 8 products are summed with packed
-// fp16 fma (as the reference does for the whole sequence, gemv.cu:1087,1096); each supergroup's
-// partial is then added into an fp32 accumulator so the error does not grow with T.
+// acc[c] accumulates w_t * v_hat[t,c] in fp32 (fp16 operands, exact products: v_fma_mix_f32); the
+// reference accumulates in fp16 for the whole sequence (gemv.cu:1087,1096).
 template <int D, int CPL>
 __global__ __launch_bounds__(BLOCK) void ov_kernel(
     const h1 *__restrict__ attn, uint4 *__restrict__ cache, const h1 *__restrict__ v_new,
@@ -359,14 +358,18 @@ __global__ __launch_bounds__(BLOCK) void ov_kernel(
 #pragma unroll
             for (int pp = 0; pp < 2; pp++) {
                 Pair &s = st[2 * v + pp];
-                h2 a16 = splat((h1)0.0f);
+                float &a0 = acc[4 * v + 2 * pp], &a1 = acc[4 * v + 2 * pp + 1];
                 auto row = [&](h2 qe, h2 qo, int br) {
                     const h2 wp = as_h2(ww[br]);
                     const h2 qs0 = qe * s.sc;
-                    a16 = pk_fma(splat(wp.x), qs0 + s.zp, a16);
+                    const h2 vd0 = qs0 + s.zp;
+                    a0 = __builtin_fmaf((float)wp.x, (float)vd0.x, a0);
+                    a1 = __builtin_fmaf((float)wp.x, (float)vd0.y, a1);
                     update_pair(s, qe, qs0);
                     const h2 qs1 = qo * s.sc;
-                    a16 = pk_fma(splat(wp.y), qs1 + s.zp, a16);
+                    const h2 vd1 = qs1 + s.zp;
+                    a0 = __builtin_fmaf((float)wp.y, (float)vd1.x, a0);
+                    a1 = __builtin_fmaf((float)wp.y, (float)vd1.y, a1);
                     update_pair(s, qo, qs1);
                 };
                 h2 qe, qo;
@@ -374,8 +377,6 @@ __global__ __launch_bounds__(BLOCK) void ov_kernel(
                 unpack_row<1>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 1);
                 unpack_row<2>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 2);
                 unpack_row<3>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 3);
-                acc[4 * v + 2 * pp] += (float)a16.x;
-                acc[4 * v + 2 * pp + 1] += (float)a16.y;
             }
         }
     };
@@ -427,8 +428,8 @@ __global__ __launch_bounds__(BLOCK) void ov_kernel(
                     const h2 qs = qc * s.sc;
                     const h2 vd = qs + s.zp;
                     const float wt = (float)wb[nfull * 8 + tt];
-                    acc[4 * v + 2 * pp] += wt * (float)vd.x;
-                    acc[4 * v + 2 * pp + 1] += wt * (float)vd.y;
+                    acc[4 * v + 2 * pp] = __builtin_fmaf(wt, (float)vd.x, acc[4 * v + 2 * pp]);
+                    acc[4 * v + 2 * pp + 1] = __builtin_fmaf(wt, (float)vd.y, acc[4 * v + 2 * pp + 1]);
                     update_pair(s, qc, qs);
                 }
             }
@@ -445,8 +446,8 @@ __global__ __launch_bounds__(BLOCK) void ov_kernel(
         h2 *o = reinterpret_cast<h2 *>(out + (size_t)bx * D + c0);
 #pragma unroll
         for (int p = 0; p < G::NP; p++) {
-            const float o0 = acc[2 * p] + wT * (float)deq[p].x;
-            const float o1 = acc[2 * p + 1] + wT * (float)deq[p].y;
+            const float o0 = __builtin_fmaf(wT, (float)deq[p].x, acc[2 * p]);
+            const float o1 = __builtin_fmaf(wT, (float)deq[p].y, acc[2 * p + 1]);
             o[p] = (h2){(h1)o0, (h1)o1};
         }
     }
