@@ -63,6 +63,56 @@ __device__ __forceinline__ void unpack_row(uint32_t wa, uint32_t wb, h2 &q_even,
     q_odd = as_h2((x & 0x00F000F0u) | 0x54005400u) - splat((h1)72.0f);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Code-pair lookup table in LDS.
+//
+// Decoding a nibble pair in registers costs ~4.5 VALU ops per channel-pair-token (byte permute,
+// mask, or, bias subtract, abs) and the scan is VALU-issue-bound, so the conversion is moved to
+// the otherwise idle LDS pipe: the byte b = code_A | code_B << 4 of one token indexes a table whose
+// entry holds the fp16 pair (q_A, q_B) and its absolute value.  Entry stride is 256 B = 32 copies of
+// the 8-byte entry; lane l reads copy l % 32, so the 16 lanes a ds_read_b64 serves per clock always
+// hit 16 distinct bank pairs, whatever their codes are.  Address = (b << 8) | (copy << 3) is built
+// by ONE v_perm_b32 from the packed code word and a per-lane constant.
+// ---------------------------------------------------------------------------------------------
+constexpr int LUT_ENTRIES = 256;
+constexpr int LUT_COPIES = 32;
+constexpr int LUT_WORDS64 = LUT_ENTRIES * LUT_COPIES; // uint2 elements = 64 KB
+
+__device__ __forceinline__ void lut_fill(uint2 *lut, int tid, int nthreads)
+{
+    for (int i = tid; i < LUT_WORDS64; i += nthreads) {
+        const int b = i / LUT_COPIES;
+        const h2 q = (h2){(h1)((b & 15) - 8), (h1)((b >> 4) - 8)};
+        lut[i] = make_uint2(as_u32(q), as_u32(q) & 0x7FFF7FFFu);
+    }
+}
+
+// Channel words A, B (8 codes each, token i at bits 4i..4i+3) -> per-token code bytes:
+// even.byte[k] = token 2k, odd.byte[k] = token 2k+1, each byte = code_A | code_B << 4.
+__device__ __forceinline__ void pair_bytes(uint32_t wa, uint32_t wb, uint32_t &even, uint32_t &odd)
+{
+    constexpr uint32_t m = 0x0F0F0F0Fu;
+    even = (wa & m) | ((wb << 4) & ~m);
+    odd = ((wa >> 4) & m) | (wb & ~m);
+}
+
+// lane_copy = (lane % 32) * 8.  Returns (q pair, |q| pair) of byte k (0..3) of `bytes`.  k must be
+// a compile-time constant after unrolling (the selector becomes a literal).
+__device__ __forceinline__ uint2 lut_get(const uint2 *lut, uint32_t bytes, uint32_t lane_copy, int k)
+{
+    const uint32_t sel = 0x0C0C0000u | ((4u + (uint32_t)k) << 8); // [0, 0, bytes.byte[k], lane_copy.byte[0]]
+    const uint32_t addr = __builtin_amdgcn_perm(bytes, lane_copy, sel);
+    return *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(lut) + addr);
+}
+
+// EMA update given qs = r16(q*sc) and |q| (gemv.cu:158-164).
+__device__ __forceinline__ void update_pair_abs(Pair &p, h2 qabs, h2 qs)
+{
+    p.zp = pk_fma(p.al, qs, p.zp);
+    const h2 f = pk_fma(p.be, qabs, p.omt);
+    p.sc = p.sc * f;
+}
+
 // gemv.cu:150-154: fp32 subtract, IEEE fp32 divide, round-half-even, NaN -> 0, clamp to [-8,7].
 __device__ __forceinline__ int quantize(h1 x, h1 zp, h1 sc)
 {

@@ -17,8 +17,14 @@
 
 namespace adkv {
 
-constexpr int BLOCK = 256;  // 4 waves
-constexpr int PF = 4;       // supergroups in flight per lane
+#ifndef ADKV_BLOCK
+#define ADKV_BLOCK 256
+#endif
+constexpr int BLOCK = ADKV_BLOCK; // threads per workgroup
+#ifndef ADKV_PF
+#define ADKV_PF 4
+#endif
+constexpr int PF = ADKV_PF; // supergroups in flight per lane
 
 template <int D, int CPL>
 struct Geo {
@@ -32,6 +38,38 @@ struct Geo {
 __device__ __forceinline__ float wave_xor_add(float v, int mask)
 {
     return v + __shfl_xor(v, mask, 64);
+}
+
+// s + s[lane ^ 8]: DPP rotate by 8 within each row of 16 lanes (no LDS round trip).
+__device__ __forceinline__ float xor8_add(float s)
+{
+    const int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, s), 0x128 /*row_ror:8*/,
+                                              0xF, 0xF, false);
+    return s + __builtin_bit_cast(float, r);
+}
+
+typedef unsigned u2v __attribute__((ext_vector_type(2)));
+
+// s + s[lane ^ 16] / s + s[lane ^ 32] through the gfx950 row/half swap instructions.  The copy goes
+// through an opaque asm so that the two operands are distinct values for the compiler.
+__device__ __forceinline__ float xor16_add(float s)
+{
+    unsigned a = __builtin_bit_cast(unsigned, s), b;
+    asm volatile("v_mov_b32 %0, %1" : "=v"(b) : "v"(a));
+    const u2v r = __builtin_amdgcn_permlane16_swap(a, b, false, false);
+    unsigned x = r.x, y = r.y;
+    asm volatile("" : "+v"(x), "+v"(y)); // keeps both results distinct for the float add below
+    return __builtin_bit_cast(float, x) + __builtin_bit_cast(float, y);
+}
+
+__device__ __forceinline__ float xor32_add(float s)
+{
+    unsigned a = __builtin_bit_cast(unsigned, s), b;
+    asm volatile("v_mov_b32 %0, %1" : "=v"(b) : "v"(a));
+    const u2v r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+    unsigned x = r.x, y = r.y;
+    asm volatile("" : "+v"(x), "+v"(y));
+    return __builtin_bit_cast(float, x) + __builtin_bit_cast(float, y);
 }
 
 // Sum over the LPH lanes of a head; every lane of the head gets the total.
@@ -170,10 +208,15 @@ __global__ __launch_bounds__(BLOCK) void qk_kernel(
     int BH, int H, int T, int n_super_cap, h1 *__restrict__ state_out)
 {
     using G = Geo<D, CPL>;
-    __shared__ float red[BLOCK / 64][64 * 9];
+    // one allocation so the table sits at LDS offset 0 (its byte address is used as is)
+    __shared__ uint2 smem[LUT_WORDS64 + (BLOCK / 64) * 64 * 9 / 2];
+    const uint2 *lut = smem;
+    lut_fill(smem, threadIdx.x, BLOCK);
+    __syncthreads();
 
     const int lane = threadIdx.x & 63;
-    float *myred = red[threadIdx.x >> 6];
+    const uint32_t lane_copy = (uint32_t)(lane & (LUT_COPIES - 1)) * 8u;
+    float *myred = reinterpret_cast<float *>(smem + LUT_WORDS64) + (threadIdx.x >> 6) * 64 * 9;
     const int gl = blockIdx.x * BLOCK + threadIdx.x;
     int bx = gl / G::LPH;
     const int lh = gl % G::LPH;
@@ -196,74 +239,110 @@ __global__ __launch_bounds__(BLOCK) void qk_kernel(
     const int nfull = T >> 3;
     const int tk = lane & 7, g8 = lane >> 3;
 
-    auto reduce_store = [&](const float *part, int sg, int ntok) {
+    // ---- cross-lane sum of the 8 per-token partials, split in three phases so that the LDS round
+    // trip of supergroup sg-1 hides under the arithmetic of supergroup sg
+    auto red_write = [&](const float *part) {
 #pragma unroll
         for (int k = 0; k < 8; k++)
             myred[lane * 9 + k] = part[k];
-        float s = 0.0f;
+    };
+    auto red_read = [&](float *tmp) {
 #pragma unroll
         for (int r = 0; r < 8; r++)
-            s += myred[(g8 * 8 + r) * 9 + tk];
-#pragma unroll
-        for (int m = 8; m < G::LPH; m <<= 1)
-            s = wave_xor_add(s, m);
+            tmp[r] = myred[(g8 * 8 + r) * 9 + tk];
+    };
+    auto red_finish = [&](const float *tmp, int sg, int ntok) {
+        float s = ((tmp[0] + tmp[1]) + (tmp[2] + tmp[3])) + ((tmp[4] + tmp[5]) + (tmp[6] + tmp[7]));
+        s = xor8_add(s);
+        s = xor16_add(s);
+        if (G::LPH == 64)
+            s = xor32_add(s);
         if (active && lh < 8 && tk < ntok)
             ob[sg * 8 + tk] = (h1)s;
     };
+    auto reduce_store = [&](const float *part, int sg, int ntok) {
+        float tmp[8];
+        red_write(part);
+        red_read(tmp);
+        red_finish(tmp, sg, ntok);
+    };
 
-    auto decode_sg = [&](const uint4 *u, float *part) {
+    // ---- software pipeline over the full supergroups.  Global loads run PF supergroups ahead.
+    // Table lookups run one supergroup ahead and are issued token by token between the arithmetic
+    // of the current supergroup (the LDS counter holds only 15 outstanding operations, so issuing a
+    // whole supergroup's lookups at once would stall on them).  The logit reduction of supergroup
+    // sg-1 is read at the start of iteration sg and finished at its end.
+    auto pair_bytes_of = [&](const uint4 *u, uint32_t (*nb)[2]) {
 #pragma unroll
         for (int v = 0; v < G::NV; v++) {
             const uint32_t w[4] = {u[v].x, u[v].y, u[v].z, u[v].w};
-#pragma unroll
-            for (int pp = 0; pp < 2; pp++) {
-                Pair &s = st[2 * v + pp];
-                const h2 qq = qv[2 * v + pp];
-                auto row = [&](h2 qe, h2 qo, int br) {
-                    const h2 qs0 = qe * s.sc;
-                    part[2 * br] = __builtin_amdgcn_fdot2(qq, qs0 + s.zp, part[2 * br], false);
-                    update_pair(s, qe, qs0);
-                    const h2 qs1 = qo * s.sc;
-                    part[2 * br + 1] = __builtin_amdgcn_fdot2(qq, qs1 + s.zp, part[2 * br + 1], false);
-                    update_pair(s, qo, qs1);
-                };
-                h2 qe, qo;
-                unpack_row<0>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 0);
-                unpack_row<1>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 1);
-                unpack_row<2>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 2);
-                unpack_row<3>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 3);
-            }
+            pair_bytes(w[0], w[1], nb[2 * v][0], nb[2 * v][1]);
+            pair_bytes(w[2], w[3], nb[2 * v + 1][0], nb[2 * v + 1][1]);
         }
     };
-
-    // software pipeline over full supergroups
-    uint4 buf[PF][G::NV];
+    auto token = [&](int t, const uint2 (*ecur)[8], uint2 (*enext)[8], const uint32_t (*nb)[2],
+                     float &out_t) {
 #pragma unroll
-    for (int i = 0; i < PF; i++)
-        if (i < nfull) {
+        for (int p = 0; p < G::NP; p++)
+            enext[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+        float acc = 0.0f;
 #pragma unroll
-            for (int v = 0; v < G::NV; v++)
-                buf[i][v] = cb[(size_t)i * G::VPS + v];
+        for (int p = 0; p < G::NP; p++) {
+            Pair &s = st[p];
+            const h2 qs = as_h2(ecur[p][t].x) * s.sc;
+            acc = __builtin_amdgcn_fdot2(qv[p], qs + s.zp, acc, false);
+            update_pair_abs(s, as_h2(ecur[p][t].y), qs);
         }
+        out_t = acc;
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    uint4 buf[PF][G::NV];
+    uint2 lk[2][G::NP][8];
+    uint32_t nb[G::NP][2];
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+#pragma unroll
+        for (int v = 0; v < G::NV; v++)
+            buf[i][v] = (i < nfull) ? cb[(size_t)i * G::VPS + v] : make_uint4(0, 0, 0, 0);
+    }
+    if (nfull > 0) {
+        pair_bytes_of(buf[0], nb);
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+#pragma unroll
+            for (int p = 0; p < G::NP; p++)
+                lk[0][p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+    }
     for (int sg0 = 0; sg0 < nfull; sg0 += PF) {
 #pragma unroll
         for (int i = 0; i < PF; i++) {
             const int sg = sg0 + i;
             if (sg < nfull) {
-                uint4 cur[G::NV];
-#pragma unroll
-                for (int v = 0; v < G::NV; v++)
-                    cur[v] = buf[i][v];
+                float tmp[8], part[8];
+                // bytes of supergroup sg+1 (stale data past the end: looked up, never used)
+                pair_bytes_of(buf[(i + 1) % PF], nb);
+                if (sg > 0)
+                    red_read(tmp);
                 if (sg + PF < nfull) {
 #pragma unroll
                     for (int v = 0; v < G::NV; v++)
                         buf[i][v] = cb[(size_t)(sg + PF) * G::VPS + v];
                 }
-                float part[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-                decode_sg(cur, part);
-                reduce_store(part, sg, 8);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int t = 0; t < 8; t++)
+                    token(t, lk[i & 1], lk[(i + 1) & 1], nb, part[t]);
+                if (sg > 0)
+                    red_finish(tmp, sg - 1, 8);
+                red_write(part);
             }
         }
+    }
+    if (nfull > 0) {
+        float tmp[8];
+        red_read(tmp);
+        red_finish(tmp, nfull - 1, 8);
     }
 
     // ragged tail: T % 8 tokens of the last supergroup, state advances only for t < T
@@ -322,6 +401,11 @@ __global__ __launch_bounds__(BLOCK) void ov_kernel(
     int BH, int H, int T, int n_super_cap, h1 *__restrict__ state_out)
 {
     using G = Geo<D, CPL>;
+    __shared__ uint2 lut[LUT_WORDS64];
+    lut_fill(lut, threadIdx.x, BLOCK);
+    __syncthreads();
+    const uint32_t lane_copy = (uint32_t)(threadIdx.x & (LUT_COPIES - 1)) * 8u;
+
     const int gl = blockIdx.x * BLOCK + threadIdx.x;
     int bx = gl / G::LPH;
     const int lh = gl % G::LPH;
@@ -350,56 +434,61 @@ __global__ __launch_bounds__(BLOCK) void ov_kernel(
         return r;
     };
 
-    auto decode_sg = [&](const uint4 *u, const uint4 wv) {
-        const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+    auto pair_bytes_of = [&](const uint4 *u, uint32_t (*nb)[2]) {
 #pragma unroll
         for (int v = 0; v < G::NV; v++) {
             const uint32_t w[4] = {u[v].x, u[v].y, u[v].z, u[v].w};
-#pragma unroll
-            for (int pp = 0; pp < 2; pp++) {
-                Pair &s = st[2 * v + pp];
-                float &a0 = acc[4 * v + 2 * pp], &a1 = acc[4 * v + 2 * pp + 1];
-                auto row = [&](h2 qe, h2 qo, int br) {
-                    const h2 wp = as_h2(ww[br]);
-                    const h2 qs0 = qe * s.sc;
-                    const h2 vd0 = qs0 + s.zp;
-                    a0 = __builtin_fmaf((float)wp.x, (float)vd0.x, a0);
-                    a1 = __builtin_fmaf((float)wp.x, (float)vd0.y, a1);
-                    update_pair(s, qe, qs0);
-                    const h2 qs1 = qo * s.sc;
-                    const h2 vd1 = qs1 + s.zp;
-                    a0 = __builtin_fmaf((float)wp.y, (float)vd1.x, a0);
-                    a1 = __builtin_fmaf((float)wp.y, (float)vd1.y, a1);
-                    update_pair(s, qo, qs1);
-                };
-                h2 qe, qo;
-                unpack_row<0>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 0);
-                unpack_row<1>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 1);
-                unpack_row<2>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 2);
-                unpack_row<3>(w[2 * pp], w[2 * pp + 1], qe, qo); row(qe, qo, 3);
-            }
+            pair_bytes(w[0], w[1], nb[2 * v][0], nb[2 * v][1]);
+            pair_bytes(w[2], w[3], nb[2 * v + 1][0], nb[2 * v + 1][1]);
         }
+    };
+    // one token of the current supergroup, preceded by the lookups of the same token slot of the
+    // next supergroup (see qk_kernel for why they are interleaved)
+    auto token = [&](int t, const uint2 (*ecur)[8], uint2 (*enext)[8], const uint32_t (*nb)[2],
+                     const uint4 wv) {
+#pragma unroll
+        for (int p = 0; p < G::NP; p++)
+            enext[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+        const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+        const h2 wp = as_h2(ww[t >> 1]);
+        const float wt = (t & 1) ? (float)wp.y : (float)wp.x;
+#pragma unroll
+        for (int p = 0; p < G::NP; p++) {
+            Pair &s = st[p];
+            const h2 qs = as_h2(ecur[p][t].x) * s.sc;
+            const h2 vd = qs + s.zp;
+            acc[2 * p] = __builtin_fmaf(wt, (float)vd.x, acc[2 * p]);
+            acc[2 * p + 1] = __builtin_fmaf(wt, (float)vd.y, acc[2 * p + 1]);
+            update_pair_abs(s, as_h2(ecur[p][t].y), qs);
+        }
+        __builtin_amdgcn_sched_barrier(0);
     };
 
     uint4 buf[PF][G::NV];
     uint4 wbuf[PF];
+    uint2 lk[2][G::NP][8];
+    uint32_t nb[G::NP][2];
 #pragma unroll
-    for (int i = 0; i < PF; i++)
-        if (i < nfull) {
+    for (int i = 0; i < PF; i++) {
 #pragma unroll
-            for (int v = 0; v < G::NV; v++)
-                buf[i][v] = cb[(size_t)i * G::VPS + v];
-            wbuf[i] = load_w(i);
-        }
+        for (int v = 0; v < G::NV; v++)
+            buf[i][v] = (i < nfull) ? cb[(size_t)i * G::VPS + v] : make_uint4(0, 0, 0, 0);
+        wbuf[i] = (i < nfull) ? load_w(i) : make_uint4(0, 0, 0, 0);
+    }
+    if (nfull > 0) {
+        pair_bytes_of(buf[0], nb);
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+#pragma unroll
+            for (int p = 0; p < G::NP; p++)
+                lk[0][p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+    }
     for (int sg0 = 0; sg0 < nfull; sg0 += PF) {
 #pragma unroll
         for (int i = 0; i < PF; i++) {
             const int sg = sg0 + i;
             if (sg < nfull) {
-                uint4 cur[G::NV];
-#pragma unroll
-                for (int v = 0; v < G::NV; v++)
-                    cur[v] = buf[i][v];
+                pair_bytes_of(buf[(i + 1) % PF], nb);
                 const uint4 wcur = wbuf[i];
                 if (sg + PF < nfull) {
 #pragma unroll
@@ -407,7 +496,10 @@ __global__ __launch_bounds__(BLOCK) void ov_kernel(
                         buf[i][v] = cb[(size_t)(sg + PF) * G::VPS + v];
                     wbuf[i] = load_w(sg + PF);
                 }
-                decode_sg(cur, wcur);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int t = 0; t < 8; t++)
+                    token(t, lk[i & 1], lk[(i + 1) & 1], nb, wcur);
             }
         }
     }
