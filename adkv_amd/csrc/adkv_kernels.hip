@@ -1,14 +1,20 @@
 // ADKV hot-path kernels for MI355X (gfx950, wave64) and their C ABI (include/adkv_hip.h).
 //
 // Work decomposition.  Every (batch, head, channel) is an independent fp16 recurrence over the
-// time axis (reference: src/adkv/kernel/gemv.cu:187-191), and without stored intermediate states
-// it has to be replayed from token 0.  So a LANE owns CPL consecutive channels of one head for the
-// whole sequence; D/CPL lanes make a head; a wave64 carries 64*CPL/D heads.  One supergroup
-// (8 tokens) of a head is D*4 contiguous bytes, which a head's lanes fetch as one run of 16-byte
-// loads; loads for the next PF supergroups are in flight while the current one is decoded.
+// time axis (reference: src/adkv/kernel/gemv.cu:187-191).  A LANE owns CPL consecutive channels of
+// one head; D/CPL lanes make a head; a wave64 carries 64*CPL/D heads.  One supergroup (8 tokens) of
+// a head is D*4 contiguous bytes, which the head's lanes fetch as one run of 16-byte loads; loads
+// for the next PF supergroups are in flight while the current one is decoded.
 //
-// The three kernels below keep the reference's call structure (encode / QK+append / OV+append) so
-// that they are drop-ins for src/adkv/kernel/gemv.cu:368-414, 883-939, 1233-1288.
+// The recurrence rounds to fp16 at every step, so it cannot be re-associated: a sequence can only be
+// split where the exact state is known.  The encoder therefore can record the state every
+// `ckpt_interval` tokens ("checkpoints", 4 bytes per channel each); given those, the decode kernels
+// cut the time axis into segments that replay independently and bit-exactly.  Without checkpoints
+// they replay from token 0 exactly like the reference.  More waves matter on this machine: a SIMD
+// needs about four resident waves to issue packed-f16 instructions at full rate.
+//
+// The kernels keep the reference's call structure (encode / QK+append / OV+append) so that they are
+// drop-ins for src/adkv/kernel/gemv.cu:368-414, 883-939, 1233-1288.
 #include "adkv_device.h"
 
 #include "../../include/adkv_hip.h"
@@ -17,10 +23,6 @@
 
 namespace adkv {
 
-#ifndef ADKV_BLOCK
-#define ADKV_BLOCK 256
-#endif
-constexpr int BLOCK = ADKV_BLOCK; // threads per workgroup
 #ifndef ADKV_PF
 #define ADKV_PF 4
 #endif
@@ -33,6 +35,17 @@ struct Geo {
     static constexpr int NP = CPL / 2;        // channel pairs per lane
     static constexpr int VPS = D / 4;         // 16-byte vectors per supergroup of one head
     static_assert(LPH == 32 || LPH == 64, "a head must fit in one wave");
+};
+
+// How the time axis is cut.  seg_tokens is a multiple of ckpt_interval (itself a multiple of 8);
+// segment s covers tokens [s*seg_tokens, min((s+1)*seg_tokens, T)) and starts from checkpoint
+// s*seg_tokens/ckpt_interval - 1 (segment 0 starts from the initial parameters).
+struct Seg {
+    h1 *ckpt;           // [B*H, n_ckpt_cap, D, 2] (zp, sc) before token (j+1)*ckpt_interval; may be null
+    int n_ckpt_cap;
+    int ckpt_interval;  // 0 when ckpt is null
+    int seg_tokens;     // >= T when there is one segment
+    int nseg;
 };
 
 __device__ __forceinline__ float wave_xor_add(float v, int mask)
@@ -50,15 +63,16 @@ __device__ __forceinline__ float xor8_add(float s)
 
 typedef unsigned u2v __attribute__((ext_vector_type(2)));
 
-// s + s[lane ^ 16] / s + s[lane ^ 32] through the gfx950 row/half swap instructions.  The copy goes
-// through an opaque asm so that the two operands are distinct values for the compiler.
+// s + s[lane ^ 16] / s + s[lane ^ 32] through the gfx950 row/half swap instructions.  Both the copy
+// and the results go through opaque asm statements: handed two identical values, or asked for the
+// float sum of the two results directly, this compiler folds the pair into one register.
 __device__ __forceinline__ float xor16_add(float s)
 {
     unsigned a = __builtin_bit_cast(unsigned, s), b;
     asm volatile("v_mov_b32 %0, %1" : "=v"(b) : "v"(a));
     const u2v r = __builtin_amdgcn_permlane16_swap(a, b, false, false);
     unsigned x = r.x, y = r.y;
-    asm volatile("" : "+v"(x), "+v"(y)); // keeps both results distinct for the float add below
+    asm volatile("" : "+v"(x), "+v"(y));
     return __builtin_bit_cast(float, x) + __builtin_bit_cast(float, y);
 }
 
@@ -82,32 +96,87 @@ __device__ __forceinline__ float head_allreduce(float v)
     return v;
 }
 
+// (zp, sc) of CPL consecutive channels <-> the interleaved [channel][2] fp16 layout used for
+// state_out and checkpoints.
+template <int CPL>
+__device__ __forceinline__ void store_state(h1 *dst, const Pair *st)
+{
+    h2 *so = reinterpret_cast<h2 *>(dst);
+#pragma unroll
+    for (int p = 0; p < CPL / 2; p++) {
+        so[2 * p] = (h2){st[p].zp.x, st[p].sc.x};
+        so[2 * p + 1] = (h2){st[p].zp.y, st[p].sc.y};
+    }
+}
+
+template <int CPL>
+__device__ __forceinline__ void load_state(const h1 *src, Pair *st)
+{
+    const h2 *so = reinterpret_cast<const h2 *>(src);
+#pragma unroll
+    for (int p = 0; p < CPL / 2; p++) {
+        const h2 a = so[2 * p], b = so[2 * p + 1];
+        st[p].zp = (h2){a.x, b.x};
+        st[p].sc = (h2){a.y, b.y};
+    }
+}
+
+// Which (head, segment) this lane works on.  Units beyond the end are clamped to the last one and
+// flagged inactive: they compute but never store.
+template <int D, int CPL, int BLK>
+struct Unit {
+    int bx, seg, lh, c0;
+    bool active;
+    __device__ __forceinline__ Unit(int BH, int nseg)
+    {
+        using G = Geo<D, CPL>;
+        const long gl = (long)blockIdx.x * BLK + threadIdx.x;
+        long u = gl / G::LPH;
+        lh = (int)(gl % G::LPH);
+        active = u < (long)BH * nseg;
+        if (!active)
+            u = (long)BH * nseg - 1;
+        bx = (int)(u / nseg);
+        seg = (int)(u % nseg);
+        c0 = lh * CPL;
+    }
+};
+
+// Parameters plus the state this segment starts from.
+template <int D, int CPL>
+__device__ __forceinline__ void init_pairs(Pair *st, const h1 *zp, const h1 *sc, const h1 *al,
+                                           const h1 *be, const h1 *tg, int h, int bx, int c0, int seg,
+                                           const Seg &sa)
+{
+#pragma unroll
+    for (int p = 0; p < CPL / 2; p++)
+        load_pair(st[p], zp, sc, al, be, tg, h * D + c0 + 2 * p);
+    if (seg > 0) {
+        const int j = seg * (sa.seg_tokens / sa.ckpt_interval) - 1;
+        load_state<CPL>(sa.ckpt + (((size_t)bx * sa.n_ckpt_cap + j) * D + c0) * 2, st);
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // encode_kv  (gemv.cu:168-308)
 // ---------------------------------------------------------------------------------------------
-template <int D, int CPL>
-__global__ __launch_bounds__(BLOCK) void encode_kernel(
+template <int D, int CPL, int BLK>
+__global__ __launch_bounds__(BLK) void encode_kernel(
     uint4 *__restrict__ cache, const h1 *__restrict__ kv_new,
     const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
     const h1 *__restrict__ be, const h1 *__restrict__ tg,
-    int BH, int H, int T, int n_super_cap, h1 *__restrict__ state_out)
+    int BH, int H, int T, int n_super_cap, h1 *__restrict__ state_out, Seg sa)
 {
     using G = Geo<D, CPL>;
-    const int gl = blockIdx.x * BLOCK + threadIdx.x;
-    int bx = gl / G::LPH;
-    const int lh = gl % G::LPH;
-    const bool active = bx < BH;
-    if (!active)
-        bx = BH - 1;
+    const Unit<D, CPL, BLK> un(BH, 1);
+    const int bx = un.bx, c0 = un.c0;
+    const bool active = un.active;
     const int h = bx % H;
-    const int c0 = lh * CPL;
 
     Pair st[G::NP];
-#pragma unroll
-    for (int p = 0; p < G::NP; p++)
-        load_pair(st[p], zp, sc, al, be, tg, h * D + c0 + 2 * p);
+    init_pairs<D, CPL>(st, zp, sc, al, be, tg, h, bx, c0, 0, sa);
 
-    uint4 *cb = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV;
+    uint4 *cb = cache + (size_t)bx * n_super_cap * G::VPS + un.lh * G::NV;
     const h1 *xb = kv_new + (size_t)bx * T * D + c0;
     const int n_super = (T + 7) / 8;
 
@@ -143,16 +212,17 @@ __global__ __launch_bounds__(BLOCK) void encode_kernel(
             for (int v = 0; v < G::NV; v++)
                 cb[(size_t)sg * G::VPS + v] =
                     make_uint4(w[4 * v], w[4 * v + 1], w[4 * v + 2], w[4 * v + 3]);
+            // state before token (j+1)*interval
+            const int tend = sg * 8 + 8;
+            if (sa.ckpt != nullptr && tend <= T && tend % sa.ckpt_interval == 0) {
+                const int j = tend / sa.ckpt_interval - 1;
+                if (j < sa.n_ckpt_cap)
+                    store_state<CPL>(sa.ckpt + (((size_t)bx * sa.n_ckpt_cap + j) * D + c0) * 2, st);
+            }
         }
     }
-    if (state_out != nullptr && active) {
-        h2 *so = reinterpret_cast<h2 *>(state_out + ((size_t)bx * D + c0) * 2);
-#pragma unroll
-        for (int p = 0; p < G::NP; p++) {
-            so[2 * p] = (h2){st[p].zp.x, st[p].sc.x};
-            so[2 * p + 1] = (h2){st[p].zp.y, st[p].sc.y};
-        }
-    }
+    if (state_out != nullptr && active)
+        store_state<CPL>(state_out + ((size_t)bx * D + c0) * 2, st);
 }
 
 // Shared tail of the two decode kernels: quantise the new token with the state after token T-1,
@@ -181,14 +251,28 @@ __device__ __forceinline__ void append_new_token(uint4 *cb, int T, const h1 *xne
     }
 }
 
+// What the last segment does once it holds the state after token T-1: hand it out, and record it
+// as a checkpoint when token T opens a new checkpoint interval.
 template <int D, int CPL>
-__device__ __forceinline__ void store_state(h1 *state_out, int bx, int c0, const Pair *st)
+__device__ __forceinline__ void publish_state(const Pair *st, h1 *state_out, const Seg &sa, int bx,
+                                              int c0, int T)
 {
-    h2 *so = reinterpret_cast<h2 *>(state_out + ((size_t)bx * D + c0) * 2);
+    if (state_out != nullptr)
+        store_state<CPL>(state_out + ((size_t)bx * D + c0) * 2, st);
+    if (sa.ckpt != nullptr && T > 0 && T % sa.ckpt_interval == 0) {
+        const int j = T / sa.ckpt_interval - 1;
+        if (j < sa.n_ckpt_cap)
+            store_state<CPL>(sa.ckpt + (((size_t)bx * sa.n_ckpt_cap + j) * D + c0) * 2, st);
+    }
+}
+
+template <int D, int CPL>
+__device__ __forceinline__ void pair_bytes_of(const uint4 *u, uint32_t (*nb)[2])
+{
 #pragma unroll
-    for (int p = 0; p < CPL / 2; p++) {
-        so[2 * p] = (h2){st[p].zp.x, st[p].sc.x};
-        so[2 * p + 1] = (h2){st[p].zp.y, st[p].sc.y};
+    for (int v = 0; v < CPL / 4; v++) {
+        pair_bytes(u[v].x, u[v].y, nb[2 * v][0], nb[2 * v][1]);
+        pair_bytes(u[v].z, u[v].w, nb[2 * v + 1][0], nb[2 * v + 1][1]);
     }
 }
 
@@ -197,46 +281,46 @@ __device__ __forceinline__ void store_state(h1 *state_out, int bx, int c0, const
 // ---------------------------------------------------------------------------------------------
 // Per lane and supergroup: 8 fp32 partial logits (v_dot2_f32_f16 over the lane's channel pairs).
 // They are summed across the head's lanes through a wave-private, conflict-free (stride 9) LDS
-// transpose: lane (g, tk) adds the partials of token tk from lanes 8g..8g+7, then xor-shuffles
+// transpose: lane (g, tk) adds the partials of token tk from lanes 8g..8g+7, then row/half swaps
 // fold the remaining LPH/8 groups.
-template <int D, int CPL>
-__global__ __launch_bounds__(BLOCK) void qk_kernel(
+template <int D, int CPL, int BLK>
+__global__ __launch_bounds__(BLK) void qk_kernel(
     const h1 *__restrict__ q, uint4 *__restrict__ cache, const h1 *__restrict__ k_new,
     h1 *__restrict__ out,
     const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
     const h1 *__restrict__ be, const h1 *__restrict__ tg,
-    int BH, int H, int T, int n_super_cap, h1 *__restrict__ state_out)
+    int BH, int H, int T, int n_super_cap, h1 *__restrict__ state_out, Seg sa)
 {
     using G = Geo<D, CPL>;
     // one allocation so the table sits at LDS offset 0 (its byte address is used as is)
-    __shared__ uint2 smem[LUT_WORDS64 + (BLOCK / 64) * 64 * 9 / 2];
+    __shared__ uint2 smem[LUT_WORDS64 + (BLK / 64) * 64 * 9 / 2];
     const uint2 *lut = smem;
-    lut_fill(smem, threadIdx.x, BLOCK);
+    lut_fill(smem, threadIdx.x, BLK);
     __syncthreads();
 
     const int lane = threadIdx.x & 63;
     const uint32_t lane_copy = (uint32_t)(lane & (LUT_COPIES - 1)) * 8u;
     float *myred = reinterpret_cast<float *>(smem + LUT_WORDS64) + (threadIdx.x >> 6) * 64 * 9;
-    const int gl = blockIdx.x * BLOCK + threadIdx.x;
-    int bx = gl / G::LPH;
-    const int lh = gl % G::LPH;
-    const bool active = bx < BH;
-    if (!active)
-        bx = BH - 1;
+
+    const Unit<D, CPL, BLK> un(BH, sa.nseg);
+    const int bx = un.bx, lh = un.lh, c0 = un.c0;
+    const bool active = un.active;
+    const bool last = un.seg == sa.nseg - 1;
     const int h = bx % H;
-    const int c0 = lh * CPL;
 
     Pair st[G::NP];
     h2 qv[G::NP];
+    init_pairs<D, CPL>(st, zp, sc, al, be, tg, h, bx, c0, un.seg, sa);
 #pragma unroll
-    for (int p = 0; p < G::NP; p++) {
-        load_pair(st[p], zp, sc, al, be, tg, h * D + c0 + 2 * p);
+    for (int p = 0; p < G::NP; p++)
         qv[p] = *reinterpret_cast<const h2 *>(q + (size_t)bx * D + c0 + 2 * p);
-    }
 
-    uint4 *cb = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV;
-    h1 *ob = out + (size_t)bx * (T + 1);
-    const int nfull = T >> 3;
+    const int t0 = un.seg * sa.seg_tokens;
+    const int t1 = last ? T : t0 + sa.seg_tokens;
+    uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV; // this head, this lane
+    const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;                  // this segment
+    h1 *ob = out + (size_t)bx * (T + 1) + t0;
+    const int nfull = (t1 - t0) >> 3;
     const int tk = lane & 7, g8 = lane >> 3;
 
     // ---- cross-lane sum of the 8 per-token partials, split in three phases so that the LDS round
@@ -260,45 +344,32 @@ __global__ __launch_bounds__(BLOCK) void qk_kernel(
         if (active && lh < 8 && tk < ntok)
             ob[sg * 8 + tk] = (h1)s;
     };
-    auto reduce_store = [&](const float *part, int sg, int ntok) {
-        float tmp[8];
-        red_write(part);
-        red_read(tmp);
-        red_finish(tmp, sg, ntok);
-    };
 
     // ---- software pipeline over the full supergroups.  Global loads run PF supergroups ahead.
     // Table lookups run one supergroup ahead and are issued token by token between the arithmetic
     // of the current supergroup (the LDS counter holds only 15 outstanding operations, so issuing a
     // whole supergroup's lookups at once would stall on them).  The logit reduction of supergroup
-    // sg-1 is read at the start of iteration sg and finished at its end.
-    auto pair_bytes_of = [&](const uint4 *u, uint32_t (*nb)[2]) {
-#pragma unroll
-        for (int v = 0; v < G::NV; v++) {
-            const uint32_t w[4] = {u[v].x, u[v].y, u[v].z, u[v].w};
-            pair_bytes(w[0], w[1], nb[2 * v][0], nb[2 * v][1]);
-            pair_bytes(w[2], w[3], nb[2 * v + 1][0], nb[2 * v + 1][1]);
-        }
-    };
-    auto token = [&](int t, const uint2 (*ecur)[8], uint2 (*enext)[8], const uint32_t (*nb)[2],
-                     float &out_t) {
-#pragma unroll
-        for (int p = 0; p < G::NP; p++)
-            enext[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+    // sg-1 is read at the start of iteration sg and finished a few tokens into it.
+    // The lookup for the next supergroup goes into the slot the current token has just vacated, so
+    // one supergroup's worth of registers holds both.
+    auto token = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2], float &out_t) {
         float acc = 0.0f;
 #pragma unroll
         for (int p = 0; p < G::NP; p++) {
             Pair &s = st[p];
-            const h2 qs = as_h2(ecur[p][t].x) * s.sc;
+            const h2 qs = as_h2(e[p][t].x) * s.sc;
             acc = __builtin_amdgcn_fdot2(qv[p], qs + s.zp, acc, false);
-            update_pair_abs(s, as_h2(ecur[p][t].y), qs);
+            update_pair_abs(s, as_h2(e[p][t].y), qs);
         }
         out_t = acc;
+#pragma unroll
+        for (int p = 0; p < G::NP; p++)
+            e[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
         __builtin_amdgcn_sched_barrier(0);
     };
 
     uint4 buf[PF][G::NV];
-    uint2 lk[2][G::NP][8];
+    uint2 lk[G::NP][8];
     uint32_t nb[G::NP][2];
 #pragma unroll
     for (int i = 0; i < PF; i++) {
@@ -307,12 +378,12 @@ __global__ __launch_bounds__(BLOCK) void qk_kernel(
             buf[i][v] = (i < nfull) ? cb[(size_t)i * G::VPS + v] : make_uint4(0, 0, 0, 0);
     }
     if (nfull > 0) {
-        pair_bytes_of(buf[0], nb);
+        pair_bytes_of<D, CPL>(buf[0], nb);
 #pragma unroll
         for (int t = 0; t < 8; t++)
 #pragma unroll
             for (int p = 0; p < G::NP; p++)
-                lk[0][p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+                lk[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
     }
     for (int sg0 = 0; sg0 < nfull; sg0 += PF) {
 #pragma unroll
@@ -321,7 +392,7 @@ __global__ __launch_bounds__(BLOCK) void qk_kernel(
             if (sg < nfull) {
                 float tmp[8], part[8];
                 // bytes of supergroup sg+1 (stale data past the end: looked up, never used)
-                pair_bytes_of(buf[(i + 1) % PF], nb);
+                pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
                 if (sg > 0)
                     red_read(tmp);
                 if (sg + PF < nfull) {
@@ -331,10 +402,13 @@ __global__ __launch_bounds__(BLOCK) void qk_kernel(
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int t = 0; t < 8; t++)
-                    token(t, lk[i & 1], lk[(i + 1) & 1], nb, part[t]);
+                for (int t = 0; t < 3; t++)
+                    token(t, lk, nb, part[t]);
                 if (sg > 0)
-                    red_finish(tmp, sg - 1, 8);
+                    red_finish(tmp, sg - 1, 8); // early, so tmp[] is dead while part[] fills up
+#pragma unroll
+                for (int t = 3; t < 8; t++)
+                    token(t, lk, nb, part[t]);
                 red_write(part);
             }
         }
@@ -344,10 +418,12 @@ __global__ __launch_bounds__(BLOCK) void qk_kernel(
         red_read(tmp);
         red_finish(tmp, nfull - 1, 8);
     }
+    if (!last)
+        return;
 
     // ragged tail: T % 8 tokens of the last supergroup, state advances only for t < T
     // (gemv.cu:648-654)
-    const int ntail = T & 7;
+    const int ntail = (t1 - t0) & 7;
     if (ntail) {
         float part[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
@@ -359,8 +435,8 @@ __global__ __launch_bounds__(BLOCK) void qk_kernel(
                 Pair &s = st[2 * v + pp];
                 for (int tt = 0; tt < ntail; tt++) {
                     const uint32_t na = (w[2 * pp] >> (4 * tt)) & 0xFu;
-                    const uint32_t nb = (w[2 * pp + 1] >> (4 * tt)) & 0xFu;
-                    const h2 qc = codes_to_h2((int)na - 8, (int)nb - 8);
+                    const uint32_t nbb = (w[2 * pp + 1] >> (4 * tt)) & 0xFu;
+                    const h2 qc = codes_to_h2((int)na - 8, (int)nbb - 8);
                     const h2 qs = qc * s.sc;
                     const float d = __builtin_amdgcn_fdot2(qv[2 * v + pp], qs + s.zp, 0.0f, false);
 #pragma unroll
@@ -370,103 +446,97 @@ __global__ __launch_bounds__(BLOCK) void qk_kernel(
                 }
             }
         }
-        reduce_store(part, nfull, ntail);
+        float tmp[8];
+        red_write(part);
+        red_read(tmp);
+        red_finish(tmp, nfull, ntail);
     }
 
-    if (state_out != nullptr && active)
-        store_state<D, CPL>(state_out, bx, c0, st);
+    if (active)
+        publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
 
     h2 deq[G::NP];
-    append_new_token<D, CPL>(cb, T, k_new + (size_t)bx * D + c0, st, deq, active);
+    append_new_token<D, CPL>(cbh, T, k_new + (size_t)bx * D + c0, st, deq, active);
     float self = 0.0f;
 #pragma unroll
     for (int p = 0; p < G::NP; p++)
         self = __builtin_amdgcn_fdot2(qv[p], deq[p], self, false);
     self = head_allreduce<G::LPH>(self);
     if (active && lh == 0)
-        ob[T] = (h1)self;
+        out[(size_t)bx * (T + 1) + T] = (h1)self;
 }
 
 // ---------------------------------------------------------------------------------------------
 // forward_ov  (gemv.cu:946-1178)
 // ---------------------------------------------------------------------------------------------
 // acc[c] accumulates w_t * v_hat[t,c] in fp32 (fp16 operands, exact products: v_fma_mix_f32); the
-// reference accumulates in fp16 for the whole sequence (gemv.cu:1087,1096).
-template <int D, int CPL>
-__global__ __launch_bounds__(BLOCK) void ov_kernel(
+// reference accumulates in fp16 for the whole sequence (gemv.cu:1087,1096).  With one segment the
+// result is rounded to fp16 and stored; with several, each segment stores its fp32 partial into
+// `partial` [nseg, B*H, D] and ov_finalize_kernel adds them up.
+template <int D, int CPL, int BLK>
+__global__ __launch_bounds__(BLK) void ov_kernel(
     const h1 *__restrict__ attn, uint4 *__restrict__ cache, const h1 *__restrict__ v_new,
-    h1 *__restrict__ out,
+    h1 *__restrict__ out, float *__restrict__ partial,
     const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
     const h1 *__restrict__ be, const h1 *__restrict__ tg,
-    int BH, int H, int T, int n_super_cap, h1 *__restrict__ state_out)
+    int BH, int H, int T, int n_super_cap, h1 *__restrict__ state_out, Seg sa)
 {
     using G = Geo<D, CPL>;
     __shared__ uint2 lut[LUT_WORDS64];
-    lut_fill(lut, threadIdx.x, BLOCK);
+    lut_fill(lut, threadIdx.x, BLK);
     __syncthreads();
     const uint32_t lane_copy = (uint32_t)(threadIdx.x & (LUT_COPIES - 1)) * 8u;
 
-    const int gl = blockIdx.x * BLOCK + threadIdx.x;
-    int bx = gl / G::LPH;
-    const int lh = gl % G::LPH;
-    const bool active = bx < BH;
-    if (!active)
-        bx = BH - 1;
+    const Unit<D, CPL, BLK> un(BH, sa.nseg);
+    const int bx = un.bx, lh = un.lh, c0 = un.c0;
+    const bool active = un.active;
+    const bool last = un.seg == sa.nseg - 1;
     const int h = bx % H;
-    const int c0 = lh * CPL;
 
     Pair st[G::NP];
     float acc[CPL];
+    init_pairs<D, CPL>(st, zp, sc, al, be, tg, h, bx, c0, un.seg, sa);
 #pragma unroll
-    for (int p = 0; p < G::NP; p++) {
-        load_pair(st[p], zp, sc, al, be, tg, h * D + c0 + 2 * p);
-        acc[2 * p] = 0.0f;
-        acc[2 * p + 1] = 0.0f;
-    }
+    for (int c = 0; c < CPL; c++)
+        acc[c] = 0.0f;
 
-    uint4 *cb = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV;
-    const h1 *wb = attn + (size_t)bx * (T + 1);
-    const int nfull = T >> 3;
+    const int t0 = un.seg * sa.seg_tokens;
+    const int t1 = last ? T : t0 + sa.seg_tokens;
+    uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV;
+    const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;
+    const h1 *wrow = attn + (size_t)bx * (T + 1);
+    const h1 *wb = wrow + t0;
+    const int nfull = (t1 - t0) >> 3;
 
     auto load_w = [&](int sg) {
         uint4 r;
         __builtin_memcpy(&r, wb + (size_t)sg * 8, 16); // row base is only 2-byte aligned
         return r;
     };
-
-    auto pair_bytes_of = [&](const uint4 *u, uint32_t (*nb)[2]) {
-#pragma unroll
-        for (int v = 0; v < G::NV; v++) {
-            const uint32_t w[4] = {u[v].x, u[v].y, u[v].z, u[v].w};
-            pair_bytes(w[0], w[1], nb[2 * v][0], nb[2 * v][1]);
-            pair_bytes(w[2], w[3], nb[2 * v + 1][0], nb[2 * v + 1][1]);
-        }
-    };
-    // one token of the current supergroup, preceded by the lookups of the same token slot of the
+    // one token of the current supergroup, followed by the lookups of the same token slot of the
     // next supergroup (see qk_kernel for why they are interleaved)
-    auto token = [&](int t, const uint2 (*ecur)[8], uint2 (*enext)[8], const uint32_t (*nb)[2],
-                     const uint4 wv) {
-#pragma unroll
-        for (int p = 0; p < G::NP; p++)
-            enext[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+    auto token = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2], const uint4 wv) {
         const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
         const h2 wp = as_h2(ww[t >> 1]);
         const float wt = (t & 1) ? (float)wp.y : (float)wp.x;
 #pragma unroll
         for (int p = 0; p < G::NP; p++) {
             Pair &s = st[p];
-            const h2 qs = as_h2(ecur[p][t].x) * s.sc;
+            const h2 qs = as_h2(e[p][t].x) * s.sc;
             const h2 vd = qs + s.zp;
             acc[2 * p] = __builtin_fmaf(wt, (float)vd.x, acc[2 * p]);
             acc[2 * p + 1] = __builtin_fmaf(wt, (float)vd.y, acc[2 * p + 1]);
-            update_pair_abs(s, as_h2(ecur[p][t].y), qs);
+            update_pair_abs(s, as_h2(e[p][t].y), qs);
         }
+#pragma unroll
+        for (int p = 0; p < G::NP; p++)
+            e[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
         __builtin_amdgcn_sched_barrier(0);
     };
 
     uint4 buf[PF][G::NV];
     uint4 wbuf[PF];
-    uint2 lk[2][G::NP][8];
+    uint2 lk[G::NP][8];
     uint32_t nb[G::NP][2];
 #pragma unroll
     for (int i = 0; i < PF; i++) {
@@ -476,19 +546,19 @@ __global__ __launch_bounds__(BLOCK) void ov_kernel(
         wbuf[i] = (i < nfull) ? load_w(i) : make_uint4(0, 0, 0, 0);
     }
     if (nfull > 0) {
-        pair_bytes_of(buf[0], nb);
+        pair_bytes_of<D, CPL>(buf[0], nb);
 #pragma unroll
         for (int t = 0; t < 8; t++)
 #pragma unroll
             for (int p = 0; p < G::NP; p++)
-                lk[0][p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+                lk[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
     }
     for (int sg0 = 0; sg0 < nfull; sg0 += PF) {
 #pragma unroll
         for (int i = 0; i < PF; i++) {
             const int sg = sg0 + i;
             if (sg < nfull) {
-                pair_bytes_of(buf[(i + 1) % PF], nb);
+                pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
                 const uint4 wcur = wbuf[i];
                 if (sg + PF < nfull) {
 #pragma unroll
@@ -499,55 +569,80 @@ __global__ __launch_bounds__(BLOCK) void ov_kernel(
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int t = 0; t < 8; t++)
-                    token(t, lk[i & 1], lk[(i + 1) & 1], nb, wcur);
+                    token(t, lk, nb, wcur);
             }
         }
     }
 
-    const int ntail = T & 7;
-    if (ntail) {
+    if (last) {
+        const int ntail = (t1 - t0) & 7;
+        if (ntail) {
 #pragma unroll
-        for (int v = 0; v < G::NV; v++) {
-            const uint4 u = cb[(size_t)nfull * G::VPS + v];
-            const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+            for (int v = 0; v < G::NV; v++) {
+                const uint4 u = cb[(size_t)nfull * G::VPS + v];
+                const uint32_t w[4] = {u.x, u.y, u.z, u.w};
 #pragma unroll
-            for (int pp = 0; pp < 2; pp++) {
-                Pair &s = st[2 * v + pp];
-                for (int tt = 0; tt < ntail; tt++) {
-                    const uint32_t na = (w[2 * pp] >> (4 * tt)) & 0xFu;
-                    const uint32_t nb = (w[2 * pp + 1] >> (4 * tt)) & 0xFu;
-                    const h2 qc = codes_to_h2((int)na - 8, (int)nb - 8);
-                    const h2 qs = qc * s.sc;
-                    const h2 vd = qs + s.zp;
-                    const float wt = (float)wb[nfull * 8 + tt];
-                    acc[4 * v + 2 * pp] = __builtin_fmaf(wt, (float)vd.x, acc[4 * v + 2 * pp]);
-                    acc[4 * v + 2 * pp + 1] = __builtin_fmaf(wt, (float)vd.y, acc[4 * v + 2 * pp + 1]);
-                    update_pair(s, qc, qs);
+                for (int pp = 0; pp < 2; pp++) {
+                    Pair &s = st[2 * v + pp];
+                    for (int tt = 0; tt < ntail; tt++) {
+                        const uint32_t na = (w[2 * pp] >> (4 * tt)) & 0xFu;
+                        const uint32_t nbb = (w[2 * pp + 1] >> (4 * tt)) & 0xFu;
+                        const h2 qc = codes_to_h2((int)na - 8, (int)nbb - 8);
+                        const h2 qs = qc * s.sc;
+                        const h2 vd = qs + s.zp;
+                        const float wt = (float)wb[nfull * 8 + tt];
+                        acc[4 * v + 2 * pp] = __builtin_fmaf(wt, (float)vd.x, acc[4 * v + 2 * pp]);
+                        acc[4 * v + 2 * pp + 1] = __builtin_fmaf(wt, (float)vd.y, acc[4 * v + 2 * pp + 1]);
+                        update_pair(s, qc, qs);
+                    }
                 }
             }
         }
-    }
+        if (active)
+            publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
 
-    if (state_out != nullptr && active)
-        store_state<D, CPL>(state_out, bx, c0, st);
-
-    h2 deq[G::NP];
-    append_new_token<D, CPL>(cb, T, v_new + (size_t)bx * D + c0, st, deq, active);
-    const float wT = (float)wb[T];
-    if (active) {
-        h2 *o = reinterpret_cast<h2 *>(out + (size_t)bx * D + c0);
+        h2 deq[G::NP];
+        append_new_token<D, CPL>(cbh, T, v_new + (size_t)bx * D + c0, st, deq, active);
+        const float wT = (float)wrow[T];
 #pragma unroll
         for (int p = 0; p < G::NP; p++) {
-            const float o0 = __builtin_fmaf(wT, (float)deq[p].x, acc[2 * p]);
-            const float o1 = __builtin_fmaf(wT, (float)deq[p].y, acc[2 * p + 1]);
-            o[p] = (h2){(h1)o0, (h1)o1};
+            acc[2 * p] = __builtin_fmaf(wT, (float)deq[p].x, acc[2 * p]);
+            acc[2 * p + 1] = __builtin_fmaf(wT, (float)deq[p].y, acc[2 * p + 1]);
         }
     }
+    if (!active)
+        return;
+    if (sa.nseg == 1) {
+        h2 *o = reinterpret_cast<h2 *>(out + (size_t)bx * D + c0);
+#pragma unroll
+        for (int p = 0; p < G::NP; p++)
+            o[p] = (h2){(h1)acc[2 * p], (h1)acc[2 * p + 1]};
+    } else {
+        float4 *o = reinterpret_cast<float4 *>(partial + ((size_t)un.seg * BH + bx) * D + c0);
+#pragma unroll
+        for (int v = 0; v < G::NV; v++)
+            o[v] = make_float4(acc[4 * v], acc[4 * v + 1], acc[4 * v + 2], acc[4 * v + 3]);
+    }
+}
+
+// out[i] = fp16(sum over segments, in segment order, of partial[s][i])
+__global__ __launch_bounds__(256) void ov_finalize_kernel(const float *__restrict__ partial,
+                                                           h1 *__restrict__ out, long n, int nseg)
+{
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n)
+        return;
+    float s = 0.0f;
+    for (int k = 0; k < nseg; k++)
+        s += partial[(size_t)k * n + i];
+    out[i] = (h1)s;
 }
 
 // ---------------------------------------------------------------------------------------------
 // softmax(float(logits)*scaling + mask) -> fp16   (llama_adkv.py:266-271)
 // ---------------------------------------------------------------------------------------------
+constexpr int SM_BLOCK = 256;
+
 __device__ __forceinline__ float block_reduce(float v, float *sm, bool is_max)
 {
 #pragma unroll
@@ -562,43 +657,78 @@ __device__ __forceinline__ float block_reduce(float v, float *sm, bool is_max)
     __syncthreads();
     float r = sm[0];
 #pragma unroll
-    for (int i = 1; i < BLOCK / 64; i++)
+    for (int i = 1; i < SM_BLOCK / 64; i++)
         r = is_max ? fmaxf(r, sm[i]) : r + sm[i];
     return r;
 }
 
-__global__ __launch_bounds__(BLOCK) void softmax_kernel(
+__global__ __launch_bounds__(SM_BLOCK) void softmax_kernel(
     const h1 *__restrict__ logits, h1 *__restrict__ weights, const float *__restrict__ mask,
     int n, int rows_per_mask_row, float scaling)
 {
-    __shared__ float sm[BLOCK / 64];
+    __shared__ float sm[SM_BLOCK / 64];
     const int row = blockIdx.x;
     const h1 *l = logits + (size_t)row * n;
     h1 *w = weights + (size_t)row * n;
     const float *mk = mask ? mask + (size_t)(row / rows_per_mask_row) * n : nullptr;
 
+    // rows up to SM_BLOCK*KEEP elements are read from memory once and kept in registers
+    constexpr int KEEP = 20;
+    float x[KEEP];
+    const bool fits = n <= SM_BLOCK * KEEP;
     float mx = -INFINITY;
-    for (int i = threadIdx.x; i < n; i += BLOCK) {
-        float x = (float)l[i] * scaling;
-        if (mk)
-            x += mk[i];
-        mx = fmaxf(mx, x);
+    if (fits) {
+#pragma unroll
+        for (int k = 0; k < KEEP; k++) {
+            const int i = threadIdx.x + k * SM_BLOCK;
+            x[k] = -INFINITY;
+            if (i < n) {
+                x[k] = (float)l[i] * scaling;
+                if (mk)
+                    x[k] += mk[i];
+            }
+            mx = fmaxf(mx, x[k]);
+        }
+    } else {
+        for (int i = threadIdx.x; i < n; i += SM_BLOCK) {
+            float v = (float)l[i] * scaling;
+            if (mk)
+                v += mk[i];
+            mx = fmaxf(mx, v);
+        }
     }
     mx = block_reduce(mx, sm, true);
     float sum = 0.0f;
-    for (int i = threadIdx.x; i < n; i += BLOCK) {
-        float x = (float)l[i] * scaling;
-        if (mk)
-            x += mk[i];
-        sum += __expf(x - mx);
+    if (fits) {
+#pragma unroll
+        for (int k = 0; k < KEEP; k++) {
+            x[k] = __expf(x[k] - mx);
+            sum += x[k];
+        }
+    } else {
+        for (int i = threadIdx.x; i < n; i += SM_BLOCK) {
+            float v = (float)l[i] * scaling;
+            if (mk)
+                v += mk[i];
+            sum += __expf(v - mx);
+        }
     }
     sum = block_reduce(sum, sm, false);
     const float inv = 1.0f / sum;
-    for (int i = threadIdx.x; i < n; i += BLOCK) {
-        float x = (float)l[i] * scaling;
-        if (mk)
-            x += mk[i];
-        w[i] = (h1)(__expf(x - mx) * inv);
+    if (fits) {
+#pragma unroll
+        for (int k = 0; k < KEEP; k++) {
+            const int i = threadIdx.x + k * SM_BLOCK;
+            if (i < n)
+                w[i] = (h1)(x[k] * inv);
+        }
+    } else {
+        for (int i = threadIdx.x; i < n; i += SM_BLOCK) {
+            float v = (float)l[i] * scaling;
+            if (mk)
+                v += mk[i];
+            w[i] = (h1)(__expf(v - mx) * inv);
+        }
     }
 }
 
@@ -632,27 +762,85 @@ static int check_common(int B, int H, int T, int D, int n_super_cap)
     return ADKV_OK;
 }
 
-static inline dim3 grid_for(int BH, int lph)
+static inline int lanes_per_head(int D) { return D == 128 ? 32 : 64; }
+
+// Waves a SIMD should hold for packed-f16 issue to run near full rate, and SIMDs on the device.
+constexpr int WAVES_PER_SIMD_TARGET = 4;
+constexpr int N_SIMD = 256 * 4;
+
+// Segment plan for a decode launch: as few segments as give every SIMD its target of waves.
+static Seg plan_segments(void *ckpt, int n_ckpt_cap, int ckpt_interval, int BH, int T, int D)
 {
-    return dim3((unsigned)(((int64_t)BH * lph + BLOCK - 1) / BLOCK));
+    Seg s;
+    s.ckpt = (h1 *)ckpt;
+    s.n_ckpt_cap = n_ckpt_cap;
+    s.ckpt_interval = ckpt ? ckpt_interval : 0;
+    s.seg_tokens = T > 0 ? T : 1;
+    s.nseg = 1;
+    if (!ckpt || ckpt_interval <= 0 || T <= ckpt_interval)
+        return s;
+    const int avail = (T + ckpt_interval - 1) / ckpt_interval;               // finest split
+    const long units_target = (long)N_SIMD * WAVES_PER_SIMD_TARGET * (64 / lanes_per_head(D));
+    long want = (units_target + BH - 1) / BH;
+    if (want < 1)
+        want = 1;
+    if (want > avail)
+        want = avail;
+    int m = (int)((avail + want - 1) / want);                                 // intervals per segment
+    // every segment start s*m*interval needs checkpoint s*m-1 < n_ckpt_cap
+    while (m < avail && ((avail - 1) / m) * m - 1 >= n_ckpt_cap)
+        m++;
+    if (m >= avail)
+        return s;
+    s.seg_tokens = m * ckpt_interval;
+    s.nseg = (T + s.seg_tokens - 1) / s.seg_tokens;
+    return s;
 }
 
-#define ADKV_DISPATCH_D(KERNEL, ...)                                                          \
-    switch (D) {                                                                              \
-    case 128:                                                                                 \
-        hipLaunchKernelGGL((KERNEL<128, 4>), grid_for(BH, 32), dim3(BLOCK), 0, st, __VA_ARGS__); \
-        break;                                                                                \
-    case 256:                                                                                 \
-        hipLaunchKernelGGL((KERNEL<256, 4>), grid_for(BH, 64), dim3(BLOCK), 0, st, __VA_ARGS__); \
-        break;                                                                                \
-    default:                                                                                  \
-        hipLaunchKernelGGL((KERNEL<512, 8>), grid_for(BH, 64), dim3(BLOCK), 0, st, __VA_ARGS__); \
-        break;                                                                                \
+template <typename F256, typename FBIG>
+static void launch_units(long threads, int big, F256 f256, FBIG fbig)
+{
+    // 16-wave workgroups share one lookup table and let a CU hold 4 waves per SIMD; small launches
+    // use 4-wave workgroups so that they still spread over the CUs
+    if (big > 256 && threads >= (long)big * 256)
+        fbig(dim3((unsigned)((threads + big - 1) / big)), dim3(big));
+    else
+        f256(dim3((unsigned)((threads + 255) / 256)), dim3(256));
+}
+
+#define ADKV_LAUNCH(KERNEL, DD, CC, BIG, ...)                                                   \
+    launch_units(                                                                               \
+        (long)BH * seg.nseg * (DD / CC), BIG,                                                   \
+        [&](dim3 g, dim3 b) { hipLaunchKernelGGL((KERNEL<DD, CC, 256>), g, b, 0, st, __VA_ARGS__); }, \
+        [&](dim3 g, dim3 b) { hipLaunchKernelGGL((KERNEL<DD, CC, BIG>), g, b, 0, st, __VA_ARGS__); })
+
+#define ADKV_DISPATCH_D(KERNEL, ...)                  \
+    switch (D) {                                      \
+    case 128:                                         \
+        ADKV_LAUNCH(KERNEL, 128, 4, 1024, __VA_ARGS__); \
+        break;                                        \
+    case 256:                                         \
+        ADKV_LAUNCH(KERNEL, 256, 4, 1024, __VA_ARGS__); \
+        break;                                        \
+    default:                                          \
+        ADKV_LAUNCH(KERNEL, 512, 8, 256, __VA_ARGS__); \
+        break;                                        \
     }
+
+static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval)
+{
+    if (!ckpt)
+        return ADKV_OK;
+    if (n_ckpt_cap <= 0 || ckpt_interval <= 0 || (ckpt_interval & 7))
+        return ADKV_E_SHAPE;
+    if ((uintptr_t)ckpt & 3)
+        return ADKV_E_ALIGN;
+    return ADKV_OK;
+}
 
 extern "C" {
 
-int adkv_abi_version(void) { return 1; }
+int adkv_abi_version(void) { return 2; }
 
 int adkv_last_hip_error(void) { return g_last_hip_error; }
 
@@ -666,16 +854,18 @@ const char *adkv_strerror(int code)
     case ADKV_E_CAPACITY: return "cache capacity too small";
     case ADKV_E_ALIGN: return "pointer not sufficiently aligned";
     case ADKV_E_UNSUPPORTED: return "unsupported configuration";
+    case ADKV_E_WORKSPACE: return "workspace too small";
     case ADKV_E_LAUNCH: return "HIP launch failed";
     default: return "unknown error";
     }
 }
 
-int adkv_encode_kv(void *cache, const void *kv_new,
-                   const void *zp, const void *sc, const void *alpha, const void *beta,
-                   const void *tgt,
-                   int B, int H, int T, int D, int n_super_cap,
-                   float, float, void *state_out, void *stream)
+int adkv_encode_kv_ex(void *cache, const void *kv_new,
+                      const void *zp, const void *sc, const void *alpha, const void *beta,
+                      const void *tgt,
+                      int B, int H, int T, int D, int n_super_cap,
+                      void *state_out, void *ckpt_out, int n_ckpt_cap, int ckpt_interval,
+                      void *stream)
 {
     if (!cache || !kv_new || !zp || !sc || !alpha || !beta || !tgt)
         return ADKV_E_NULL;
@@ -686,21 +876,40 @@ int adkv_encode_kv(void *cache, const void *kv_new,
         return ADKV_E_CAPACITY;
     if (((uintptr_t)cache & 15) || ((uintptr_t)kv_new & 3))
         return ADKV_E_ALIGN;
+    if ((rc = check_ckpt(ckpt_out, n_ckpt_cap, ckpt_interval)))
+        return rc;
     if (T == 0 && state_out == nullptr)
         return ADKV_OK;
     const int BH = B * H;
     hipStream_t st = (hipStream_t)stream;
+    Seg seg;
+    seg.ckpt = (h1 *)ckpt_out;
+    seg.n_ckpt_cap = n_ckpt_cap;
+    seg.ckpt_interval = ckpt_out ? ckpt_interval : 0;
+    seg.seg_tokens = T > 0 ? T : 1;
+    seg.nseg = 1;
     ADKV_DISPATCH_D(encode_kernel, (uint4 *)cache, (const h1 *)kv_new, (const h1 *)zp,
                     (const h1 *)sc, (const h1 *)alpha, (const h1 *)beta, (const h1 *)tgt, BH, H, T,
-                    n_super_cap, (h1 *)state_out);
+                    n_super_cap, (h1 *)state_out, seg);
     return check_launch();
 }
 
-int adkv_forward_qk(const void *q, void *k_cache, const void *k_new, void *logits,
-                    const void *zp, const void *sc, const void *alpha, const void *beta,
-                    const void *tgt,
-                    int B, int H, int T, int D, int n_super_cap,
-                    float, float, void *state_out, void *stream)
+int adkv_encode_kv(void *cache, const void *kv_new,
+                   const void *zp, const void *sc, const void *alpha, const void *beta,
+                   const void *tgt,
+                   int B, int H, int T, int D, int n_super_cap,
+                   float, float, void *state_out, void *stream)
+{
+    return adkv_encode_kv_ex(cache, kv_new, zp, sc, alpha, beta, tgt, B, H, T, D, n_super_cap,
+                             state_out, nullptr, 0, 0, stream);
+}
+
+int adkv_forward_qk_ex(const void *q, void *k_cache, const void *k_new, void *logits,
+                       const void *zp, const void *sc, const void *alpha, const void *beta,
+                       const void *tgt,
+                       int B, int H, int T, int D, int n_super_cap,
+                       void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
+                       void *stream)
 {
     if (!q || !k_cache || !k_new || !logits || !zp || !sc || !alpha || !beta || !tgt)
         return ADKV_E_NULL;
@@ -711,19 +920,42 @@ int adkv_forward_qk(const void *q, void *k_cache, const void *k_new, void *logit
         return ADKV_E_CAPACITY;
     if (((uintptr_t)k_cache & 15) || ((uintptr_t)q & 3) || ((uintptr_t)k_new & 3))
         return ADKV_E_ALIGN;
+    if ((rc = check_ckpt(ckpt, n_ckpt_cap, ckpt_interval)))
+        return rc;
     const int BH = B * H;
     hipStream_t st = (hipStream_t)stream;
+    const Seg seg = plan_segments(ckpt, n_ckpt_cap, ckpt_interval, BH, T, D);
     ADKV_DISPATCH_D(qk_kernel, (const h1 *)q, (uint4 *)k_cache, (const h1 *)k_new, (h1 *)logits,
                     (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha, (const h1 *)beta,
-                    (const h1 *)tgt, BH, H, T, n_super_cap, (h1 *)state_out);
+                    (const h1 *)tgt, BH, H, T, n_super_cap, (h1 *)state_out, seg);
     return check_launch();
 }
 
-int adkv_forward_ov(const void *attn, void *v_cache, const void *v_new, void *out,
+int adkv_forward_qk(const void *q, void *k_cache, const void *k_new, void *logits,
                     const void *zp, const void *sc, const void *alpha, const void *beta,
                     const void *tgt,
                     int B, int H, int T, int D, int n_super_cap,
                     float, float, void *state_out, void *stream)
+{
+    return adkv_forward_qk_ex(q, k_cache, k_new, logits, zp, sc, alpha, beta, tgt, B, H, T, D,
+                              n_super_cap, state_out, nullptr, 0, 0, stream);
+}
+
+int64_t adkv_forward_ov_workspace_bytes(int B, int H, int T, int D, int n_ckpt_cap, int ckpt_interval)
+{
+    if (B <= 0 || H <= 0 || T < 0 || n_ckpt_cap <= 0 || ckpt_interval <= 0)
+        return 0;
+    int dummy = 0;
+    const Seg seg = plan_segments(&dummy, n_ckpt_cap, ckpt_interval, B * H, T, D);
+    return seg.nseg > 1 ? (int64_t)seg.nseg * B * H * D * 4 : 0;
+}
+
+int adkv_forward_ov_ex(const void *attn, void *v_cache, const void *v_new, void *out,
+                       const void *zp, const void *sc, const void *alpha, const void *beta,
+                       const void *tgt,
+                       int B, int H, int T, int D, int n_super_cap,
+                       void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
+                       void *workspace, int64_t workspace_bytes, void *stream)
 {
     if (!attn || !v_cache || !v_new || !out || !zp || !sc || !alpha || !beta || !tgt)
         return ADKV_E_NULL;
@@ -734,12 +966,39 @@ int adkv_forward_ov(const void *attn, void *v_cache, const void *v_new, void *ou
         return ADKV_E_CAPACITY;
     if (((uintptr_t)v_cache & 15) || ((uintptr_t)out & 3) || ((uintptr_t)v_new & 3))
         return ADKV_E_ALIGN;
+    if ((rc = check_ckpt(ckpt, n_ckpt_cap, ckpt_interval)))
+        return rc;
     const int BH = B * H;
     hipStream_t st = (hipStream_t)stream;
+    const Seg seg = plan_segments(ckpt, n_ckpt_cap, ckpt_interval, BH, T, D);
+    if (seg.nseg > 1) {
+        if (!workspace || workspace_bytes < (int64_t)seg.nseg * BH * D * 4)
+            return ADKV_E_WORKSPACE;
+        if ((uintptr_t)workspace & 15)
+            return ADKV_E_ALIGN;
+    }
     ADKV_DISPATCH_D(ov_kernel, (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new, (h1 *)out,
-                    (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha, (const h1 *)beta,
-                    (const h1 *)tgt, BH, H, T, n_super_cap, (h1 *)state_out);
-    return check_launch();
+                    (float *)workspace, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,
+                    (const h1 *)beta, (const h1 *)tgt, BH, H, T, n_super_cap, (h1 *)state_out, seg);
+    if ((rc = check_launch()))
+        return rc;
+    if (seg.nseg > 1) {
+        const long n = (long)BH * D;
+        hipLaunchKernelGGL(ov_finalize_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                           (const float *)workspace, (h1 *)out, n, seg.nseg);
+        rc = check_launch();
+    }
+    return rc;
+}
+
+int adkv_forward_ov(const void *attn, void *v_cache, const void *v_new, void *out,
+                    const void *zp, const void *sc, const void *alpha, const void *beta,
+                    const void *tgt,
+                    int B, int H, int T, int D, int n_super_cap,
+                    float, float, void *state_out, void *stream)
+{
+    return adkv_forward_ov_ex(attn, v_cache, v_new, out, zp, sc, alpha, beta, tgt, B, H, T, D,
+                              n_super_cap, state_out, nullptr, 0, 0, nullptr, 0, stream);
 }
 
 int adkv_softmax(const void *logits, void *weights, const void *mask,
@@ -749,7 +1008,7 @@ int adkv_softmax(const void *logits, void *weights, const void *mask,
         return ADKV_E_NULL;
     if (rows <= 0 || n <= 0 || (mask && rows_per_mask_row <= 0))
         return ADKV_E_SHAPE;
-    hipLaunchKernelGGL(softmax_kernel, dim3((unsigned)rows), dim3(BLOCK), 0, (hipStream_t)stream,
+    hipLaunchKernelGGL(softmax_kernel, dim3((unsigned)rows), dim3(SM_BLOCK), 0, (hipStream_t)stream,
                        (const h1 *)logits, (h1 *)weights, (const float *)mask, n,
                        mask ? rows_per_mask_row : 1, scaling);
     return check_launch();

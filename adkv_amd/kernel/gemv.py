@@ -50,6 +50,18 @@ def _ptr(t: torch.Tensor | None) -> int | None:
     return None if t is None else t.data_ptr()
 
 
+def _ckpt_args(ckpt: torch.Tensor | None, ckpt_interval: int, B: int, nh: int, DIM: int):
+    """Validates a checkpoint tensor ``[B, nh, n_ckpt_cap, DIM, 2]`` fp16 -> (ptr, cap, interval)."""
+    if ckpt is None:
+        return None, 0, 0
+    _chk(ckpt.dtype == torch.float16 and ckpt.is_contiguous() and ckpt.dim() == 5
+         and ckpt.shape[0] == B and ckpt.shape[1] == nh and ckpt.shape[3] == DIM and ckpt.shape[4] == 2
+         and ckpt.shape[2] >= 1,
+         "ckpt must be contiguous fp16 [B, nh, n_ckpt_cap, DIM, 2]")
+    _chk(ckpt_interval > 0 and ckpt_interval % 8 == 0, "ckpt_interval must be a positive multiple of 8")
+    return ckpt.data_ptr(), ckpt.shape[2], int(ckpt_interval)
+
+
 def forward_qk(
     q: torch.Tensor,
     k_cache: torch.Tensor,
@@ -64,6 +76,8 @@ def forward_qk(
     scale_max: float,
     *,
     state_out: torch.Tensor | None = None,
+    ckpt: torch.Tensor | None = None,
+    ckpt_interval: int = 0,
 ) -> torch.Tensor:
     """Decode-phase QK^T over the nibble-packed ADKV cache (reference gemv.py:16-55).
 
@@ -79,6 +93,10 @@ def forward_qk(
         scale_min, scale_max: kept for API compatibility (unused by the fp16 recurrence).
         state_out: optional ``[B, nh, DIM, 2]`` float16, receives (zp, sc) after token ``T-1``
             (extension; not in the reference).
+        ckpt, ckpt_interval: optional state checkpoints of this cache, ``[B, nh, n, DIM, 2]`` float16
+            with entry ``j`` = state before token ``(j+1)*ckpt_interval`` (extension).  With them
+            the time axis is replayed in independent segments; entry ``T/ckpt_interval - 1`` is
+            written when token ``T`` opens a new interval.
 
     Returns ``[B, nh, T+1]`` float16 logits.
     """
@@ -103,12 +121,13 @@ def forward_qk(
     if state_out is not None:
         _chk(state_out.dtype == torch.float16 and state_out.is_contiguous()
              and state_out.numel() == B * nh * DIM * 2, "state_out must be contiguous fp16 [B,nh,DIM,2]")
+    cp, ccap, civ = _ckpt_args(ckpt, ckpt_interval, B, nh, DIM)
     with torch.cuda.device(dev):
-        rc = _lib.lib().adkv_forward_qk(
+        rc = _lib.lib().adkv_forward_qk_ex(
             q_flat.data_ptr(), k_cache.data_ptr(), k_new_flat.data_ptr(), o.data_ptr(),
             zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
-            B, nh, T, DIM, n_super_cap, float(scale_min), float(scale_max),
-            _ptr(state_out), _lib.current_stream_ptr(dev))
+            B, nh, T, DIM, n_super_cap, _ptr(state_out), cp, ccap, civ,
+            _lib.current_stream_ptr(dev))
     _lib.check(rc, "forward_qk")
     return o.reshape(B, nh, T + 1)
 
@@ -126,6 +145,8 @@ def forward_ov(
     scale_max: float,
     *,
     state_out: torch.Tensor | None = None,
+    ckpt: torch.Tensor | None = None,
+    ckpt_interval: int = 0,
 ) -> torch.Tensor:
     """Decode-phase OV over the nibble-packed ADKV cache (reference gemv.py:58-97).
 
@@ -158,12 +179,19 @@ def forward_ov(
     if state_out is not None:
         _chk(state_out.dtype == torch.float16 and state_out.is_contiguous()
              and state_out.numel() == B * nh * DIM * 2, "state_out must be contiguous fp16 [B,nh,DIM,2]")
+    cp, ccap, civ = _ckpt_args(ckpt, ckpt_interval, B, nh, DIM)
+    L = _lib.lib()
+    ws, ws_bytes = None, 0
+    if cp is not None:
+        ws_bytes = L.adkv_forward_ov_workspace_bytes(B, nh, T, DIM, ccap, civ)
+        if ws_bytes:
+            ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dev)
     with torch.cuda.device(dev):
-        rc = _lib.lib().adkv_forward_ov(
+        rc = L.adkv_forward_ov_ex(
             attn_flat.data_ptr(), v_cache.data_ptr(), v_new_flat.data_ptr(), o.data_ptr(),
             zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
-            B, nh, T, DIM, n_super_cap, float(scale_min), float(scale_max),
-            _ptr(state_out), _lib.current_stream_ptr(dev))
+            B, nh, T, DIM, n_super_cap, _ptr(state_out), cp, ccap, civ,
+            _ptr(ws), ws_bytes, _lib.current_stream_ptr(dev))
     _lib.check(rc, "forward_ov")
     return o.view(attn.shape[0], attn.shape[1], -1)
 
@@ -180,11 +208,14 @@ def encode_kv(
     scale_max: float,
     *,
     state_out: torch.Tensor | None = None,
+    ckpt: torch.Tensor | None = None,
+    ckpt_interval: int = 0,
 ) -> torch.Tensor:
     """Prefill: quantise tokens ``[0, T)`` into the uint4-tiled KV cache (reference gemv.py:100-132).
 
     Replays the ADKV filter from ``(kv_zp, kv_sc)``; token ``t`` goes to byte row ``t/2``, low
     nibble for even ``t`` and high nibble for odd ``t``.  Purely in place; returns ``kv_cache``.
+    ``ckpt`` (extension): receives the state before every token ``(j+1)*ckpt_interval <= T``.
     """
     _chk(kv_new.dtype == torch.float16, "kv_new must be float16")
     _chk(kv_cache.dtype == torch.uint8, "kv_cache must be uint8")
@@ -206,12 +237,13 @@ def encode_kv(
              and state_out.numel() == B * nh * DIM * 2, "state_out must be contiguous fp16 [B,nh,DIM,2]")
     if B * nh * T == 0 and state_out is None:
         return kv_cache
+    cp, ccap, civ = _ckpt_args(ckpt, ckpt_interval, B, nh, DIM)
     with torch.cuda.device(dev):
-        rc = _lib.lib().adkv_encode_kv(
+        rc = _lib.lib().adkv_encode_kv_ex(
             kv_cache.data_ptr(), kv_new_flat.data_ptr(),
             zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
-            B, nh, T, DIM, n_super_cap, float(scale_min), float(scale_max),
-            _ptr(state_out), _lib.current_stream_ptr(dev))
+            B, nh, T, DIM, n_super_cap, _ptr(state_out), cp, ccap, civ,
+            _lib.current_stream_ptr(dev))
     _lib.check(rc, "encode_kv")
     return kv_cache
 

@@ -40,6 +40,8 @@ def parse():
     ap.add_argument("--ctx", type=int, default=4096)
     ap.add_argument("--layer-buffers", type=int, default=4,
                     help="distinct K/V caches rotated through (defeats on-die cache reuse)")
+    ap.add_argument("--ckpt-interval", type=int, default=256,
+                    help="state checkpoint spacing in tokens (0 = none: one sequential replay per head)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-heads", type=int, default=0,
                     help="heads of one sequence timed on the host (0 = auto, about 10-30 s)")
@@ -97,19 +99,24 @@ def main():
     smin, smax = math.exp(-4.0), math.exp(4.0)
     NL = args.layer_buffers
 
-    kps, vps, kcs, vcs = [], [], [], []
+    S = args.ckpt_interval
+    ncap = T // S + 1 if S else 0
+    kps, vps, kcs, vcs, kks, vks = [], [], [], [], [], []
     for l in range(NL):
         kp = synth.make_params(H, D, seed=3, layer=l).to(dev)
         vp = synth.make_params(H, D, seed=4, layer=l).to(dev)
         kc = synth.alloc_cache(B, H, T + 8, D, dev)
         vc = synth.alloc_cache(B, H, T + 8, D, dev)
+        kk = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=dev) if S else None
+        vk = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=dev) if S else None
         x = synth.make_k(B, H, T, D, layer=l, dtype=torch.float16, device=dev)
-        gemv.encode_kv(kc, x, *kp.astuple(), smin, smax)
+        gemv.encode_kv(kc, x, *kp.astuple(), smin, smax, ckpt=kk, ckpt_interval=S)
         del x
         x = synth.make_v(B, H, T, D, layer=l, dtype=torch.float16, device=dev)
-        gemv.encode_kv(vc, x, *vp.astuple(), smin, smax)
+        gemv.encode_kv(vc, x, *vp.astuple(), smin, smax, ckpt=vk, ckpt_interval=S)
         del x
         kps.append(kp.astuple()); vps.append(vp.astuple()); kcs.append(kc); vcs.append(vc)
+        kks.append(kk); vks.append(vk)
     q = synth.make_q(B, H, D, device=dev)
     k_new = synth.make_k(B, H, 1, D, seed=11, dtype=torch.float16, device=dev, t0=T)
     v_new = synth.make_v(B, H, 1, D, seed=12, dtype=torch.float16, device=dev)
@@ -125,13 +132,13 @@ def main():
         if timed:
             e = [ev() for _ in range(4)]
             e[0].record()
-        logits = gemv.forward_qk(q, kcs[l], k_new, *kps[l], T, smin, smax)
+        logits = gemv.forward_qk(q, kcs[l], k_new, *kps[l], T, smin, smax, ckpt=kks[l], ckpt_interval=S)
         if timed:
             e[1].record()
         w = gemv.softmax_scale_mask(logits, scaling)
         if timed:
             e[2].record()
-        out = gemv.forward_ov(w, vcs[l], v_new, *vps[l], smin, smax)
+        out = gemv.forward_ov(w, vcs[l], v_new, *vps[l], smin, smax, ckpt=vks[l], ckpt_interval=S)
         if timed:
             e[3].record()
             marks.append(e)
@@ -171,8 +178,9 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": f"cfg2 Llama-2-7B-shaped ADKV decode attention: B={B} H={H} d={D} ctx={T} "
-                        f"4-bit K+V codes, step = forward_qk+softmax+forward_ov, {NL} rotating layer caches",
-            "batch": B, "heads": H, "head_dim": D, "ctx": T, "bits": 4,
+                        f"4-bit K+V codes, step = forward_qk+softmax+forward_ov, {NL} rotating layer caches, "
+                        f"state checkpoints every {S} tokens",
+            "batch": B, "heads": H, "head_dim": D, "ctx": T, "bits": 4, "ckpt_interval": S,
             "parallelism": "1 GPU",
         },
         "kernel_ms": {"forward_qk": qk_ms, "softmax": sm_ms, "forward_ov": ov_ms,

@@ -27,6 +27,7 @@ extern "C" {
 #define ADKV_E_CAPACITY (-4)   /* cache has too few supergroups */
 #define ADKV_E_ALIGN (-5)      /* pointer alignment requirement violated */
 #define ADKV_E_UNSUPPORTED (-6)
+#define ADKV_E_WORKSPACE (-7)  /* workspace missing or too small */
 #define ADKV_E_LAUNCH (-100)   /* HIP reported a launch error; see adkv_last_hip_error() */
 
 /* ABI version of this header; bumped on any signature change. */
@@ -83,6 +84,43 @@ int adkv_forward_ov(const void *attn, void *v_cache, const void *v_new, void *ou
  */
 int adkv_softmax(const void *logits, void *weights, const void *mask,
                  int rows, int n, int rows_per_mask_row, float scaling, void *stream);
+
+/*
+ * ---- Extensions with state checkpoints (no counterpart in the reference's code; its paper sketches
+ * them in App. I).  The fp16 recurrence rounds at every step, so a sequence can only be cut where
+ * the exact state is known.  A checkpoint tensor is fp16 [B, H, n_ckpt_cap, D, 2]; entry j holds
+ * (zp, sc) BEFORE token (j+1)*ckpt_interval (ckpt_interval a positive multiple of 8).  It belongs to
+ * one cache tensor and is maintained by these calls: the encoder writes every entry up to T, the
+ * decode calls write entry T/ckpt_interval-1 when the appended token T starts a new interval.
+ * Given checkpoints, the decode calls split the time axis into independently replayed segments so
+ * that small batches and long contexts still fill the GPU; results are bit-identical for codes and
+ * state, and equal up to fp32 summation order for logits/outputs.  Passing ckpt = NULL gives exactly
+ * the plain entry points above.
+ */
+int adkv_encode_kv_ex(void *cache, const void *kv_new,
+                      const void *zp, const void *sc, const void *alpha, const void *beta,
+                      const void *tgt,
+                      int B, int H, int T, int D, int n_super_cap,
+                      void *state_out, void *ckpt_out, int n_ckpt_cap, int ckpt_interval,
+                      void *stream);
+
+int adkv_forward_qk_ex(const void *q, void *k_cache, const void *k_new, void *logits,
+                       const void *zp, const void *sc, const void *alpha, const void *beta,
+                       const void *tgt,
+                       int B, int H, int T, int D, int n_super_cap,
+                       void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
+                       void *stream);
+
+/* Bytes of fp32 workspace adkv_forward_ov_ex needs for these sizes (0 when it runs one segment). */
+int64_t adkv_forward_ov_workspace_bytes(int B, int H, int T, int D, int n_ckpt_cap,
+                                        int ckpt_interval);
+
+int adkv_forward_ov_ex(const void *attn, void *v_cache, const void *v_new, void *out,
+                       const void *zp, const void *sc, const void *alpha, const void *beta,
+                       const void *tgt,
+                       int B, int H, int T, int D, int n_super_cap,
+                       void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
+                       void *workspace, int64_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

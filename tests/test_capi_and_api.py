@@ -51,6 +51,13 @@ def test_argument_validation_in_c_abi_needs_no_device():
     assert L.adkv_forward_qk(*qk) == -4          # slot 8 needs a second supergroup
     qk[12] = 96
     assert L.adkv_forward_qk(*qk) == -2
+    # checkpoint arguments: interval must be a positive multiple of 8; a multi-segment OV needs workspace
+    ex = [one] * 9 + [1, 1, 64, 128, 16, None, one, 8, 12, None]
+    assert L.adkv_forward_qk_ex(*ex) == -3
+    assert L.adkv_forward_ov_workspace_bytes(1, 1, 64, 128, 8, 16) == 4 * 1 * 1 * 128 * 4
+    ov = [one] * 9 + [1, 1, 64, 128, 16, None, one, 8, 16, None, 0, None]
+    assert L.adkv_forward_ov_ex(*ov) == -7
+    assert L.adkv_forward_ov_workspace_bytes(128, 32, 4096, 128, 17, 256) == 2 * 128 * 32 * 128 * 4
 
 
 def _p(nh, D, dtype=torch.float16):

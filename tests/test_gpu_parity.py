@@ -203,3 +203,102 @@ def test_full_size_invariants(gpu, oracle):
                                       _np16(x[b:b + 1, h:h + 1, T:]), *ph)
         goto = _np16(out[b:b + 1, h:h + 1]).astype(np.float64)
         assert np.max(np.abs(goto - ow)) <= 2e-3
+
+
+def _oracle_ckpts(oracle, cache_np, pn, T, S, ncap):
+    """Checkpoints the oracle way: entry j = replayed state after (j+1)*S tokens."""
+    B, H = cache_np.shape[:2]
+    D = cache_np.shape[3] * 4
+    ck = np.zeros((B, H, ncap, D, 2), np.uint16)
+    for j in range(ncap):
+        if (j + 1) * S <= T:
+            _, st = oracle.replay_f16(cache_np, *pn, (j + 1) * S, want_khat=False)
+            ck[:, :, j] = st
+    return ck
+
+
+@pytest.mark.parametrize("B,H,T,D,S", [
+    (1, 2, 100, 128, 16), (2, 3, 64, 128, 16), (1, 2, 63, 128, 8), (1, 1, 257, 128, 64),
+    (2, 2, 48, 256, 16), (1, 2, 40, 512, 8), (3, 2, 15, 128, 16), (1, 2, 1024, 128, 256),
+])
+def test_checkpointed_segments(gpu, oracle, B, H, T, D, S):
+    """Encoder checkpoints are the oracle's replayed states; decode over independently replayed
+    segments gives the same appended codes, final state and (up to fp32 summation order) the same
+    logits/outputs as one sequential replay; a checkpoint is recorded when T closes an interval."""
+    x, p = _inputs(B, H, T + 1, D, seed=3 * T + S)
+    pn = [_np16(t) for t in p.astuple()]
+    pg = [t.to(gpu) for t in p.astuple()]
+    xn = _np16(x)
+    ncap = T // S + 2
+    base = oracle.alloc_cache(B, H, T + 9, D)
+    oracle.encode_kv_f16(base, xn[:, :, :T], *pn)
+    ck_want = _oracle_ckpts(oracle, base, pn, T, S, ncap)
+
+    cache = synth.alloc_cache(B, H, T + 9, D, gpu)
+    ck = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=gpu)
+    gemv.encode_kv(cache, x[:, :, :T].contiguous().to(gpu), *pg, SMIN, SMAX, ckpt=ck, ckpt_interval=S)
+    torch.cuda.synchronize()
+    assert np.array_equal(cache.cpu().numpy(), base)
+    n_have = T // S
+    assert np.array_equal(_np16(ck).view(np.uint16)[:, :, :n_have], ck_want[:, :, :n_have])
+    assert not ck[:, :, n_have:].any()
+
+    g = torch.Generator().manual_seed(9)
+    q = torch.randn(B, H, 1, D, generator=g).half()
+    attn = torch.softmax(torch.randn(B, H, T + 1, generator=g) * 2, -1).half()
+    _, st_want = oracle.replay_f16(base, *pn, T, want_khat=False)
+
+    k_want = base.copy()
+    l_want, _ = oracle.forward_qk_f16(_np16(q), k_want, xn[:, :, T:T + 1], *pn, T)
+    kc, ckk = cache.clone(), ck.clone()
+    st = torch.zeros(B, H, D, 2, dtype=torch.float16, device=gpu)
+    logits = gemv.forward_qk(q.to(gpu), kc, x[:, :, T:T + 1].to(gpu), *pg, T, SMIN, SMAX,
+                             state_out=st, ckpt=ckk, ckpt_interval=S)
+    torch.cuda.synchronize()
+    assert np.array_equal(kc.cpu().numpy(), k_want)
+    assert np.array_equal(_np16(st).view(np.uint16), st_want)
+    assert np.all(np.abs(_np16(logits).astype(np.float64) - l_want) <= _ulp16(l_want) + 1e-3)
+    got_ck = _np16(ckk).view(np.uint16)
+    if T % S == 0:
+        assert np.array_equal(got_ck[:, :, T // S - 1], st_want), "closing checkpoint not recorded"
+    assert np.array_equal(got_ck[:, :, :n_have], ck_want[:, :, :n_have])
+
+    v_want = base.copy()
+    o_want, _ = oracle.forward_ov_f16(_np16(attn), v_want, xn[:, :, T:T + 1], *pn)
+    vc, ckv = cache.clone(), ck.clone()
+    st2 = torch.zeros_like(st)
+    out = gemv.forward_ov(attn.to(gpu), vc, x[:, :, T:T + 1].to(gpu), *pg, SMIN, SMAX,
+                          state_out=st2, ckpt=ckv, ckpt_interval=S)
+    torch.cuda.synchronize()
+    assert np.array_equal(vc.cpu().numpy(), v_want)
+    assert np.array_equal(_np16(st2).view(np.uint16), st_want)
+    assert np.all(np.abs(_np16(out).astype(np.float64) - o_want) <= _ulp16(o_want) + 1e-3)
+    if T % S == 0:
+        assert np.array_equal(_np16(ckv).view(np.uint16)[:, :, T // S - 1], st_want)
+
+
+def test_full_size_segmented_matches_sequential(gpu):
+    """Headline shape with checkpoints every 256 tokens: the segmented launch (16-wave workgroups)
+    appends the same codes and state as the sequential one and its logits/outputs agree."""
+    B, H, T, D, S = 128, 32, 4096, 128, 256
+    p = synth.make_params(H, D).to(gpu)
+    x = synth.make_k(B, H, T + 1, D, dtype=torch.float16, device=gpu)
+    cache = synth.alloc_cache(B, H, T + 8, D, gpu)
+    ck = torch.zeros(B, H, T // S + 1, D, 2, dtype=torch.float16, device=gpu)
+    gemv.encode_kv(cache, x[:, :, :T].contiguous(), *p.astuple(), SMIN, SMAX, ckpt=ck, ckpt_interval=S)
+    q = synth.make_q(B, H, D, device=gpu)
+    xn = x[:, :, T:].contiguous()
+    c1, c2 = cache.clone(), cache.clone()
+    s1 = torch.zeros(B, H, D, 2, dtype=torch.float16, device=gpu)
+    s2 = torch.zeros_like(s1)
+    l1 = gemv.forward_qk(q, c1, xn, *p.astuple(), T, SMIN, SMAX, state_out=s1)
+    l2 = gemv.forward_qk(q, c2, xn, *p.astuple(), T, SMIN, SMAX, state_out=s2, ckpt=ck, ckpt_interval=S)
+    assert torch.equal(c1, c2) and torch.equal(s1.view(torch.int16), s2.view(torch.int16))
+    assert torch.equal(l1, l2)          # per-token sums have the same order in both launches
+    assert torch.equal(ck[:, :, T // S - 1].view(torch.int16), s1.view(torch.int16))
+    w = gemv.softmax_scale_mask(l1, D ** -0.5)
+    c1, c2 = cache.clone(), cache.clone()
+    o1 = gemv.forward_ov(w, c1, xn, *p.astuple(), SMIN, SMAX)
+    o2 = gemv.forward_ov(w, c2, xn, *p.astuple(), SMIN, SMAX, ckpt=ck, ckpt_interval=S)
+    assert torch.equal(c1, c2)
+    assert torch.max(torch.abs(o1.float() - o2.float())) <= 1e-3
