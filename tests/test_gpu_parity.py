@@ -301,4 +301,6 @@ def test_full_size_segmented_matches_sequential(gpu):
     o1 = gemv.forward_ov(w, c1, xn, *p.astuple(), SMIN, SMAX)
     o2 = gemv.forward_ov(w, c2, xn, *p.astuple(), SMIN, SMAX, ckpt=ck, ckpt_interval=S)
     assert torch.equal(c1, c2)
-    assert torch.max(torch.abs(o1.float() - o2.float())) <= 1e-3
+    # fp32 partial sums are added in a different order: at most one fp16 ulp apart
+    d = torch.abs(o1.float() - o2.float())
+    assert torch.all(d <= 2.0 ** -10 * torch.clamp(o1.float().abs(), min=2.0 ** -4))
