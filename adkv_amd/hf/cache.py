@@ -1,0 +1,231 @@
+"""Per-layer packed ADKV KV cache: the host-side owner of the code buffers.
+
+Counterpart of the reference's ``KVCacheLayer_ADKV`` / ``KVCache_ADKV``
+(src/adkv/hf/llama_adkv.py:44-288) with the same public names, method signatures, buffer layout
+``[B, H, n_super, C // 4, 4, 4]`` uint8 and error behaviour, so code written against the
+reference's cache object works unchanged.  What differs is underneath:
+
+* the three kernels are the gfx950 ones (``adkv_amd.kernel.gemv``), launched on the current stream;
+* the scale/mask/softmax chain between QK and OV is one fused launch instead of five torch ops;
+* capacity grows geometrically (the reference reallocates and copies both caches every 64 tokens,
+  llama_adkv.py:104-123);
+* next to each code buffer lives a small checkpoint tensor holding the exact fp16 filter state
+  every ``CKPT_INTERVAL`` tokens (4 bytes per channel per checkpoint, ~3 % of the codes at 256).
+  The kernels keep it up to date and use it to replay the time axis in independent segments.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..kernel.gemv import encode_kv, forward_ov, forward_qk, softmax_scale_mask
+
+SCALE_MIN = math.exp(-4.0)  # kept for API parity; the fp16 recurrence never clamps
+SCALE_MAX = math.exp(4.0)
+
+INIT_SEQ_LEN = 64    # token slots of a fresh cache (reference llama_adkv.py:40)
+CAP_LEN = 64         # capacity granularity in tokens (reference llama_adkv.py:41)
+GROWTH = 1.5         # geometric growth factor once the initial capacity is exceeded
+CKPT_INTERVAL = 256  # tokens between state checkpoints (multiple of 8); 0 disables them
+
+_HEAD_DIMS = (128, 256, 512)
+
+
+class KVCacheLayer_ADKV:
+    """Quantised K/V store of one attention layer."""
+
+    def __init__(self):
+        self._key_buf: torch.Tensor | None = None
+        self._value_buf: torch.Tensor | None = None
+        self._key_ckpt: torch.Tensor | None = None
+        self._value_ckpt: torch.Tensor | None = None
+        self._quant_len = 0
+        self._cap_len = 0
+        self._B = self._H = self._C = 0
+        self._device = None
+        self._ckpt_interval = CKPT_INTERVAL
+
+    # ------------------------------------------------------------------ HF cache protocol
+    def get_seq_length(self) -> int:
+        return self._quant_len
+
+    def get_mask_sizes(self, cache_position) -> tuple[int, int]:
+        """(kv_length, kv_offset) for mask construction.  ``cache_position`` is the query's position
+        tensor (transformers 5.3, the version the reference pins) or the query length as an int
+        (later 5.x releases)."""
+        q_len = cache_position if isinstance(cache_position, int) else cache_position.shape[0]
+        return self._quant_len + q_len, 0
+
+    @property
+    def key_states(self) -> torch.Tensor | None:
+        """Packed uint8 K codes (None before the first token)."""
+        return self._key_buf
+
+    @property
+    def value_states(self) -> torch.Tensor | None:
+        """Packed uint8 V codes (None before the first token)."""
+        return self._value_buf
+
+    # ------------------------------------------------------------------ storage
+    @staticmethod
+    def _n_super(tokens: int) -> int:
+        return -(-tokens // 8)
+
+    def _n_ckpt(self, cap_tokens: int) -> int:
+        return cap_tokens // self._ckpt_interval + 1 if self._ckpt_interval else 0
+
+    def _new_buffers(self, cap_tokens: int):
+        ns = self._n_super(cap_tokens)
+        shape = (self._B, self._H, ns, self._C // 4, 4, 4)
+        mk = lambda: torch.zeros(shape, dtype=torch.uint8, device=self._device)
+        ck = (lambda: torch.zeros((self._B, self._H, self._n_ckpt(ns * 8), self._C, 2),
+                                  dtype=torch.float16, device=self._device)) \
+            if self._ckpt_interval else (lambda: None)
+        return ns * 8, mk(), mk(), ck(), ck()
+
+    def _init_buffers(self, B: int, H: int, C: int, device: torch.device):
+        if C not in _HEAD_DIMS:
+            raise ValueError(f"ADKV kernels support head_dim in (128, 256, 512), got {C}")
+        self._B, self._H, self._C, self._device = B, H, C, device
+        self._quant_len = 0
+        (self._cap_len, self._key_buf, self._value_buf,
+         self._key_ckpt, self._value_ckpt) = self._new_buffers(INIT_SEQ_LEN)
+
+    def _cap_buffers(self, T: int):
+        """Make room for ``T`` tokens.  New slots are zero, as the append kernels expect."""
+        if T <= self._cap_len:
+            return
+        want = max(T, int(self._cap_len * GROWTH))
+        want = -(-want // CAP_LEN) * CAP_LEN
+        cap, key, value, kck, vck = self._new_buffers(want)
+        old = self._key_buf.shape[2]
+        key[:, :, :old].copy_(self._key_buf)
+        value[:, :, :old].copy_(self._value_buf)
+        if kck is not None:
+            n = self._key_ckpt.shape[2]
+            kck[:, :, :n].copy_(self._key_ckpt)
+            vck[:, :, :n].copy_(self._value_ckpt)
+        self._key_buf, self._value_buf, self._key_ckpt, self._value_ckpt = key, value, kck, vck
+        self._cap_len = cap
+
+    def _check_geometry(self, B: int, H: int, C: int, device: torch.device):
+        if self._key_buf is None:
+            self._init_buffers(B, H, C, device)
+        elif (B, H, C) != (self._B, self._H, self._C):
+            raise ValueError("cache was created for a different (B, H, C)")
+
+    def _view(self, p: torch.Tensor) -> torch.Tensor:
+        return p.view(self._H, self._C)
+
+    # ------------------------------------------------------------------ quantise
+    def _append_tokens(self, key_states, value_states,
+                       key_zp_init, key_scale_init, key_alpha, key_beta, key_quant_target,
+                       value_zp_init, value_scale_init, value_alpha, value_beta, value_quant_target):
+        """Quantise ``[B, H, T, C]`` keys/values from token 0 into the packed buffers."""
+        v = self._view
+        S = self._ckpt_interval
+        encode_kv(self._key_buf, key_states.to(torch.float16).contiguous(),
+                  v(key_zp_init), v(key_scale_init), v(key_alpha), v(key_beta), v(key_quant_target),
+                  SCALE_MIN, SCALE_MAX, ckpt=self._key_ckpt, ckpt_interval=S)
+        encode_kv(self._value_buf, value_states.to(torch.float16).contiguous(),
+                  v(value_zp_init), v(value_scale_init), v(value_alpha), v(value_beta),
+                  v(value_quant_target),
+                  SCALE_MIN, SCALE_MAX, ckpt=self._value_ckpt, ckpt_interval=S)
+        self._quant_len += key_states.shape[2]
+
+    def prefill(self, key_states, value_states,
+                key_zp_init, key_scale_init, key_alpha, key_beta, key_quant_target,
+                value_zp_init, value_scale_init, value_alpha, value_beta, value_quant_target):
+        """Quantise the prompt into the cache.  No attention is computed here."""
+        B, H, T, C = key_states.shape
+        if value_states.shape != key_states.shape:
+            raise ValueError("key/value shapes differ")
+        self._check_geometry(B, H, C, key_states.device)
+        if T == 0:
+            return
+        if self._quant_len != 0:
+            raise NotImplementedError(
+                "ADKV prefill encodes from token 0; chunked prefill is not supported by the kernel")
+        self._cap_buffers(T)
+        self._append_tokens(key_states, value_states,
+                            key_zp_init, key_scale_init, key_alpha, key_beta, key_quant_target,
+                            value_zp_init, value_scale_init, value_alpha, value_beta,
+                            value_quant_target)
+
+    # ------------------------------------------------------------------ decode
+    def decode(self, query_states, key_states, value_states,
+               key_zp_init, key_scale_init, key_alpha, key_beta, key_quant_target,
+               value_zp_init, value_scale_init, value_alpha, value_beta, value_quant_target,
+               attention_mask: torch.Tensor | None = None,
+               scaling: float = 1.0) -> tuple[torch.Tensor, torch.Tensor]:
+        """One causal decode step: attend over the cached tokens and the new one, append the new
+        K/V codes, return ``(output [B,H,C] in the query's dtype, weights [B,H,ctx+1] fp16)``."""
+        B, Hq, Tq, C = query_states.shape
+        H, Tk = key_states.shape[1], key_states.shape[2]
+        if Tq != 1 or Tk != 1:
+            raise ValueError("decode expects exactly one query/key/value token")
+        if Hq != H:
+            raise ValueError("ADKV decode supports MHA (num_attention_heads == num_key_value_heads)")
+        self._check_geometry(B, H, C, query_states.device)
+        ctx = self._quant_len
+        self._cap_buffers(ctx + 1)
+
+        f16 = lambda t: t.to(torch.float16).contiguous()
+        v = self._view
+        S = self._ckpt_interval
+        logits = forward_qk(f16(query_states), self._key_buf, f16(key_states),
+                            v(key_zp_init), v(key_scale_init), v(key_alpha), v(key_beta),
+                            v(key_quant_target), ctx, SCALE_MIN, SCALE_MAX,
+                            ckpt=self._key_ckpt, ckpt_interval=S)
+        weights = softmax_scale_mask(logits, scaling, attention_mask)
+        out = forward_ov(weights, self._value_buf, f16(value_states),
+                         v(value_zp_init), v(value_scale_init), v(value_alpha), v(value_beta),
+                         v(value_quant_target), SCALE_MIN, SCALE_MAX,
+                         ckpt=self._value_ckpt, ckpt_interval=S)
+        self._quant_len = ctx + 1
+        return out.to(query_states.dtype), weights
+
+    # ------------------------------------------------------------------ accounting
+    def nbytes(self) -> int:
+        """Device bytes held by this layer (codes + checkpoints)."""
+        ts = (self._key_buf, self._value_buf, self._key_ckpt, self._value_ckpt)
+        return sum(t.numel() * t.element_size() for t in ts if t is not None)
+
+
+class KVCache_ADKV(list):
+    """One ``KVCacheLayer_ADKV`` per decoder layer (reference llama_adkv.py:279-288)."""
+
+    def __init__(self, num_layers: int):
+        super().__init__(KVCacheLayer_ADKV() for _ in range(num_layers))
+
+    def get_seq_length(self, layer_idx: int = 0) -> int:
+        return self[layer_idx].get_seq_length()
+
+    def get_mask_sizes(self, cache_position, layer_idx: int) -> tuple[int, int]:
+        return self[layer_idx].get_mask_sizes(cache_position)
+
+    # the rest is what newer transformers releases ask of a cache object during generate()
+    def get_query_offset(self, layer_idx: int = 0) -> int:
+        return self.get_seq_length(layer_idx)
+
+    def get_max_length(self) -> int:
+        return -1
+
+    is_sliding = [False]
+    is_compileable = False
+
+
+def adkv_cache_bytes(B: int, H: int, C: int, tokens: int, layers: int, bits: int = 4,
+                     ckpt_interval: int = CKPT_INTERVAL) -> int:
+    """Bytes of a full ADKV cache: K and V codes plus fp16 (zp, sc) checkpoints.  Same accounting
+    as the reference's memory model (tools/memory_comparison_fig.py:46-56) with
+    ``ckpt_num = tokens // ckpt_interval``; the ten parameter vectors per layer are added once."""
+    codes = B * H * (-(-tokens // 8) * 8) * C * bits // 8
+    ckpt = (B * H * (tokens // ckpt_interval) * C * 2 * 2) if ckpt_interval else 0
+    params = 10 * H * C * 2
+    return layers * (2 * (codes + ckpt) + params)
+
+
+def fp16_cache_bytes(B: int, H: int, C: int, tokens: int, layers: int) -> int:
+    return layers * 2 * B * H * tokens * C * 2

@@ -1,0 +1,138 @@
+"""Hugging Face Llama with the ADKV quantised KV cache on MI355X.
+
+Counterpart of the reference's ``adkv.hf.llama_adkv`` (src/adkv/hf/llama_adkv.py:291-462): same
+class names, same buffer names on the attention module (``key_zp_init`` ... ``value_quant_target``),
+same ``load_adkv_config`` entry point, so a script written for the reference only changes its
+import.  Prefill runs the regular dense attention and also quantises the prompt into the cache;
+a single-token step goes through ``KVCacheLayer_ADKV.decode`` (llama_adkv.py:347-356 in the
+reference).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+from torch import nn
+from transformers.models.llama.modeling_llama import (
+    LlamaAttention,
+    LlamaDecoderLayer,
+    LlamaForCausalLM,
+    LlamaModel,
+    apply_rotary_pos_emb,
+    eager_attention_forward,
+)
+from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
+
+from .cache import (CAP_LEN, INIT_SEQ_LEN, SCALE_MAX, SCALE_MIN, KVCache_ADKV,  # noqa: F401
+                    KVCacheLayer_ADKV)
+
+# the five per-(head, channel) quantities, for K and for V (reference llama_adkv.py:27)
+ADKV_PARAM_FIELDS = ("zp_init", "scale_init", "alpha", "beta", "quant_target")
+
+
+@dataclass
+class ADKVConfig:
+    """Calibrated parameters of one tensor (K or V) of one layer, each of ``H * head_dim`` values."""
+    zp_init: torch.Tensor
+    scale_init: torch.Tensor
+    alpha: torch.Tensor
+    beta: torch.Tensor
+    quant_target: torch.Tensor
+
+
+class LlamaAttention_ADKV(LlamaAttention):
+    """Llama attention whose single-token steps read the packed ADKV cache."""
+
+    def __init__(self, config, layer_idx: int):
+        super().__init__(config, layer_idx)
+        width = config.num_key_value_heads * self.head_dim
+        for side in ("key", "value"):
+            for name in ADKV_PARAM_FIELDS:
+                # fp16 because the deployment recurrence is fp16; filled by load_adkv_config()
+                self.register_buffer(f"{side}_{name}", torch.empty(width, dtype=torch.float16),
+                                     persistent=False)
+
+    def _adkv_params(self, side: str) -> tuple[torch.Tensor, ...]:
+        return tuple(getattr(self, f"{side}_{name}") for name in ADKV_PARAM_FIELDS)
+
+    def forward(self, hidden_states, position_embeddings=None, attention_mask=None,
+                past_key_values=None, cache_position=None, use_cache: bool = True, **kwargs):
+        lead = hidden_states.shape[:-1]
+        split = (*lead, -1, self.head_dim)
+        q = self.q_proj(hidden_states).view(split).transpose(1, 2)
+        k = self.k_proj(hidden_states).view(split).transpose(1, 2)
+        v = self.v_proj(hidden_states).view(split).transpose(1, 2)
+        cos, sin = position_embeddings
+        q, k = apply_rotary_pos_emb(q, k, cos, sin)
+
+        layer_cache = None
+        if use_cache and past_key_values is not None:
+            if not isinstance(past_key_values, KVCache_ADKV):
+                raise TypeError("ADKV attention requires a KVCache_ADKV, got "
+                                f"{type(past_key_values).__name__}")
+            layer_cache = past_key_values[self.layer_idx]
+
+        if layer_cache is not None and q.shape[2] == 1:
+            ctx, weights = layer_cache.decode(
+                q, k, v, *self._adkv_params("key"), *self._adkv_params("value"),
+                attention_mask=attention_mask, scaling=self.scaling)
+            return self.o_proj(ctx.reshape(*lead, -1).contiguous()), weights
+
+        if layer_cache is not None:
+            layer_cache.prefill(k, v, *self._adkv_params("key"), *self._adkv_params("value"))
+
+        attend = eager_attention_forward
+        if self.config._attn_implementation != "eager":
+            attend = ALL_ATTENTION_FUNCTIONS[self.config._attn_implementation]
+        ctx, weights = attend(self, q, k, v, attention_mask,
+                              dropout=0.0 if not self.training else self.attention_dropout,
+                              scaling=self.scaling, **kwargs)
+        return self.o_proj(ctx.reshape(*lead, -1).contiguous()), weights
+
+
+class LlamaDecoderLayer_ADKV(LlamaDecoderLayer):
+    def __init__(self, config, layer_idx: int):
+        super().__init__(config, layer_idx)
+        self.self_attn = LlamaAttention_ADKV(config=config, layer_idx=layer_idx)
+
+
+class LlamaModel_ADKV(LlamaModel):
+    _no_split_modules = ["LlamaDecoderLayer_ADKV"]
+
+    def __init__(self, config):
+        super().__init__(config)
+        self.layers = nn.ModuleList(LlamaDecoderLayer_ADKV(config, i)
+                                    for i in range(config.num_hidden_layers))
+        self.post_init()  # the replaced layers need the config's initialisation too
+
+    def forward(self, input_ids=None, attention_mask=None, position_ids=None, past_key_values=None,
+                inputs_embeds=None, cache_position=None, use_cache=None, **kwargs):
+        if use_cache is None:
+            use_cache = getattr(self.config, "use_cache", True)
+        if use_cache and past_key_values is None:
+            # created here so that HF never substitutes its DynamicCache
+            past_key_values = KVCache_ADKV(self.config.num_hidden_layers)
+        return super().forward(input_ids=input_ids, attention_mask=attention_mask,
+                               position_ids=position_ids, past_key_values=past_key_values,
+                               inputs_embeds=inputs_embeds, cache_position=cache_position,
+                               use_cache=use_cache, **kwargs)
+
+
+class LlamaForCausalLM_ADKV(LlamaForCausalLM):
+    _no_split_modules = ["LlamaDecoderLayer_ADKV"]
+
+    def __init__(self, config):
+        super().__init__(config)
+        self.model = LlamaModel_ADKV(config)
+        self.tie_weights()
+
+    def load_adkv_config(self, adkv_config: list[tuple[ADKVConfig, ADKVConfig]]):
+        """Copy per-layer (K, V) parameter sets into the attention modules' fp16 buffers."""
+        for layer, pair in zip(self.model.layers, adkv_config):
+            for side, cfg in zip(("key", "value"), pair):
+                for name in ADKV_PARAM_FIELDS:
+                    getattr(layer.self_attn, f"{side}_{name}").copy_(getattr(cfg, name))
+
+    def _prepare_cache_for_generation(self, *args, **kwargs):
+        # generate() must not install a DynamicCache; LlamaModel_ADKV makes the ADKV cache itself
+        return None

@@ -1,0 +1,152 @@
+"""Host-side cache object and HF integration (counterparts of src/adkv/hf/llama_adkv.py:44-462)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from adkv_amd import synth
+from adkv_amd.hf import cache as C
+from adkv_amd.hf.cache import KVCache_ADKV, KVCacheLayer_ADKV
+
+
+def _np16(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.float16)
+
+
+def _flat(p):
+    return [t.reshape(-1) for t in p.astuple()]
+
+
+# ----------------------------------------------------------------------------- CPU: host logic
+def test_cache_storage_management_cpu():
+    c = KVCacheLayer_ADKV()
+    assert c.get_seq_length() == 0 and c.key_states is None
+    c._init_buffers(2, 3, 128, torch.device("cpu"))
+    assert c.key_states.shape == (2, 3, 8, 32, 4, 4) and c.key_states.dtype == torch.uint8
+    assert c._cap_len == 64 and not c.key_states.any()
+    c._key_buf[0, 0, 0, 0, 0, 0] = 7
+    c._key_ckpt[0, 0, 0, 0, 0] = 1.5
+    c._cap_buffers(64)                       # fits: nothing happens
+    assert c._cap_len == 64
+    c._cap_buffers(65)                       # grows geometrically, in CAP_LEN steps, keeps content
+    assert c._cap_len == 128 and c.key_states.shape[2] == 16
+    assert c._key_buf[0, 0, 0, 0, 0, 0] == 7 and c._key_ckpt[0, 0, 0, 0, 0] == 1.5
+    assert not c._key_buf[:, :, 8:].any()    # new slots are zero (the append is a read-modify-write)
+    c._cap_buffers(1000)
+    assert c._cap_len == 1024 and c._key_ckpt.shape[2] == 1024 // C.CKPT_INTERVAL + 1
+    assert c.get_mask_sizes(torch.arange(3)) == (3, 0)
+    assert KVCacheLayer_ADKV._n_super(0) == 0 and KVCacheLayer_ADKV._n_super(9) == 2
+
+
+def test_cache_errors_cpu():
+    p = synth.make_params(2, 128)
+    kp = _flat(p)
+    c = KVCacheLayer_ADKV()
+    with pytest.raises(ValueError, match="head_dim in \\(128, 256, 512\\)"):
+        c.prefill(torch.zeros(1, 2, 4, 64), torch.zeros(1, 2, 4, 64), *kp, *kp)
+    c = KVCacheLayer_ADKV()
+    with pytest.raises(ValueError, match="key/value shapes differ"):
+        c.prefill(torch.zeros(1, 2, 4, 128), torch.zeros(1, 2, 5, 128), *kp, *kp)
+    c.prefill(torch.zeros(1, 2, 0, 128), torch.zeros(1, 2, 0, 128), *kp, *kp)   # T == 0: allocate only
+    assert c.get_seq_length() == 0 and c.key_states is not None
+    with pytest.raises(ValueError, match="different \\(B, H, C\\)"):
+        c.prefill(torch.zeros(2, 2, 4, 128), torch.zeros(2, 2, 4, 128), *kp, *kp)
+    q = torch.zeros(1, 2, 1, 128)
+    with pytest.raises(ValueError, match="exactly one query/key/value token"):
+        c.decode(torch.zeros(1, 2, 2, 128), q, q, *kp, *kp)
+    with pytest.raises(ValueError, match="supports MHA"):
+        c.decode(torch.zeros(1, 4, 1, 128), q, q, *kp, *kp)
+    c._quant_len = 3
+    with pytest.raises(NotImplementedError, match="chunked prefill is not supported"):
+        c.prefill(torch.zeros(1, 2, 4, 128), torch.zeros(1, 2, 4, 128), *kp, *kp)
+    kv = KVCache_ADKV(3)
+    assert len(kv) == 3 and kv.get_seq_length(1) == 0
+    # no device => loud failure from the kernel layer, never a CPU fallback
+    c2 = KVCacheLayer_ADKV()
+    with pytest.raises(RuntimeError, match="HIP device"):
+        c2.prefill(torch.zeros(1, 2, 4, 128), torch.zeros(1, 2, 4, 128), *kp, *kp)
+
+
+def test_memory_model():
+    """Same accounting as tools/memory_comparison_fig.py:46-56 for B=32, T=4096, hidden 4096."""
+    a = C.adkv_cache_bytes(32, 32, 128, 4096, layers=1, ckpt_interval=0)
+    assert a == 2 * 32 * 4096 * 4096 // 2 + 10 * 4096 * 2
+    f = C.fp16_cache_bytes(32, 32, 128, 4096, layers=1)
+    assert 3.9 < f / a < 4.0
+    with_ck = C.adkv_cache_bytes(32, 32, 128, 4096, layers=1, ckpt_interval=256)
+    assert 1.03 < with_ck / a < 1.04
+
+
+# ----------------------------------------------------------------------------- GPU
+@pytest.mark.gpu
+@pytest.mark.parametrize("interval", [0, 16, 256])
+def test_prefill_then_decode_steps_match_oracle(gpu, oracle, monkeypatch, interval):
+    """Prompt of 50 tokens, then 30 single-token steps that cross capacity growth (64 -> 128 slots)
+    and several checkpoint boundaries; codes bit-exact and outputs within 2e-3 at every step."""
+    monkeypatch.setattr(C, "CKPT_INTERVAL", interval)
+    B, H, D, T0, steps = 2, 3, 128, 50, 30
+    kp, vp = synth.make_params(H, D, seed=3), synth.make_params(H, D, seed=4)
+    k = synth.make_k(B, H, T0 + steps, D, dtype=torch.float16)
+    v = synth.make_v(B, H, T0 + steps, D, dtype=torch.float16)
+    g = torch.Generator().manual_seed(1)
+    scaling = D ** -0.5
+    kpn, vpn = [_np16(t) for t in kp.astuple()], [_np16(t) for t in vp.astuple()]
+    ko, vo = oracle.alloc_cache(B, H, T0 + steps + 8, D), oracle.alloc_cache(B, H, T0 + steps + 8, D)
+    oracle.encode_kv_f16(ko, _np16(k)[:, :, :T0], *kpn)
+    oracle.encode_kv_f16(vo, _np16(v)[:, :, :T0], *vpn)
+
+    layer = KVCacheLayer_ADKV()
+    kg, vg = _flat(kp.to(gpu)), _flat(vp.to(gpu))
+    layer.prefill(k[:, :, :T0].to(gpu), v[:, :, :T0].to(gpu), *kg, *vg)
+    assert layer.get_seq_length() == T0
+    for s in range(steps):
+        T = T0 + s
+        q = torch.randn(B, H, 1, D, generator=g).half()
+        mask = None
+        if s % 3 == 1:                        # additive mask that hides a few cached tokens
+            mask = torch.zeros(B, 1, 1, T + 1)
+            mask[:, :, :, 3:9] = float("-inf")
+        out, w = layer.decode(q.to(gpu), k[:, :, T:T + 1].to(gpu), v[:, :, T:T + 1].to(gpu), *kg, *vg,
+                              attention_mask=None if mask is None else mask.to(gpu), scaling=scaling)
+        want, w_want, _ = oracle.decode_step_f16(_np16(q), ko, vo, _np16(k)[:, :, T:T + 1],
+                                                 _np16(v)[:, :, T:T + 1], kpn, vpn, T, scaling,
+                                                 mask=None if mask is None else mask[:, :, 0, :].numpy())
+        assert out.shape == (B, H, D) and w.shape == (B, H, T + 1) and out.dtype == torch.float16
+        assert np.max(np.abs(_np16(out).astype(np.float64) - want)) <= 2e-3, s
+        assert layer.get_seq_length() == T + 1
+    n = oracle.n_super(T0 + steps)
+    assert np.array_equal(layer.key_states.cpu().numpy()[:, :, :n], ko[:, :, :n])
+    assert np.array_equal(layer.value_states.cpu().numpy()[:, :, :n], vo[:, :, :n])
+    assert layer._cap_len == 128
+
+
+@pytest.mark.gpu
+def test_tiny_llama_generate(gpu):
+    """Random-init 2-layer Llama (2 heads of 128) decodes greedily through the ADKV cache; with
+    near-lossless parameters (tiny scale) its tokens match the dense fp32 model's."""
+    transformers = pytest.importorskip("transformers")
+    from transformers import LlamaConfig, LlamaForCausalLM
+    from adkv_amd.hf.llama_adkv import ADKVConfig, LlamaForCausalLM_ADKV
+
+    cfg = LlamaConfig(vocab_size=128, hidden_size=256, intermediate_size=512, num_hidden_layers=2,
+                      num_attention_heads=2, num_key_value_heads=2, max_position_embeddings=256,
+                      attn_implementation="eager")
+    torch.manual_seed(0)
+    dense = LlamaForCausalLM(cfg).to(gpu).eval()
+    model = LlamaForCausalLM_ADKV(cfg).to(gpu).eval()
+    model.load_state_dict(dense.state_dict())
+    n = 2 * 128
+    # delta coding with alpha = 1 and an adaptive scale tracks smooth-ish activations closely
+    mk = lambda: ADKVConfig(zp_init=torch.zeros(n), scale_init=torch.full((n,), 0.05),
+                            alpha=torch.full((n,), 0.95), beta=torch.full((n,), 0.05),
+                            quant_target=torch.full((n,), 3.5))
+    model.load_adkv_config([(mk(), mk()) for _ in range(2)])
+    ids = torch.randint(0, 128, (2, 12), generator=torch.Generator().manual_seed(3)).to(gpu)
+    with torch.no_grad():
+        out = model.generate(ids, max_new_tokens=8, do_sample=False)
+        ref = dense.generate(ids, max_new_tokens=8, do_sample=False)
+    assert out.shape == (2, 20)
+    assert torch.equal(out[:, :12], ids)
+    # the first generated token comes from the dense prefill path: identical by construction
+    assert torch.equal(out[:, 12], ref[:, 12])
