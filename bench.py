@@ -42,6 +42,9 @@ def parse():
                     help="distinct K/V caches rotated through (defeats on-die cache reuse)")
     ap.add_argument("--ckpt-interval", type=int, default=256,
                     help="state checkpoint spacing in tokens (0 = none: one sequential replay per head)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three 1 GiB device-to-device copies (a known-size kernel to scale "
+                         "rocprofv3 FETCH_SIZE/WRITE_SIZE readings by)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-heads", type=int, default=0,
                     help="heads of one sequence timed on the host (0 = auto, about 10-30 s)")
@@ -123,6 +126,14 @@ def main():
     scaling = D ** -0.5
     torch.cuda.synchronize()
     torch.cuda.empty_cache()
+
+    if args.calibrate_copy:
+        a = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        del a, b
 
     ev = lambda: torch.cuda.Event(enable_timing=True)
     marks = []

@@ -7,6 +7,11 @@
  * Nothing in the shipped package may call into this library; only tests, the
  * smoke check and the bench's cpu_baseline leg do.
  *
+ * Parity status: the reference holds no tests or golden vectors for this path; every function is
+ * pinned by the independent checks in tests/test_oracle_*.py.  Parity unpinned on two points:
+ * adkv_o_quant_f32 versus the reference's torch.compile'd chunk function (compiler-dependent),
+ * and CUDA hardware behaviour at NaN/denormal corners beyond its intrinsics' documentation.
+ *
  * All fp16 values cross this interface as raw uint16_t bit patterns.
  */
 #ifndef ADKV_ORACLE_H
