@@ -198,13 +198,15 @@ def main():
                       "step_device_median": dev_ms},
         "step_code_GBps": 2 * code_bytes / (ms_step * 1e-3) / 1e9,
         "roofline": {
-            "kernel": "qk_kernel<128,4>",
+            "kernel": "qk_kernel",
             "bound": "hbm",
             "achieved": achieved,
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": None,
+            # HBM bytes per QK launch from rocprofv3 FETCH_SIZE/WRITE_SIZE scaled by a 1 GiB copy
+            # (profiles/decode_cfg2_pmc_traffic.md); measured for the default workload only
+            "traffic": 1.1227e9 if (B, H, D, T, S) == (128, 32, 128, 4096, 256) else None,
         },
     }
     if not args.no_cpu_baseline:
