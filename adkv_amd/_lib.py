@@ -13,7 +13,7 @@ import torch  # noqa: F401  (loads libamdhip64 first)
 
 _DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_DIR, "libadkv_hip.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _vp, _i, _f = C.c_void_p, C.c_int, C.c_float
 
@@ -27,6 +27,7 @@ PROTOTYPES = {
     "adkv_forward_ov": (_i, [_vp] * 9 + [_i] * 5 + [_f, _f, _vp, _vp]),
     "adkv_softmax": (_i, [_vp] * 3 + [_i] * 3 + [_f, _vp]),
     "adkv_encode_kv_ex": (_i, [_vp] * 7 + [_i] * 5 + [_vp, _vp, _i, _i, _vp]),
+    "adkv_append_kv": (_i, [_vp] * 7 + [_i] * 6 + [_vp, _vp, _i, _i, _vp]),
     "adkv_forward_qk_ex": (_i, [_vp] * 9 + [_i] * 5 + [_vp, _vp, _i, _i, _vp]),
     "adkv_forward_ov_workspace_bytes": (C.c_int64, [_i] * 6),
     "adkv_forward_ov_ex": (_i, [_vp] * 9 + [_i] * 5 + [_vp, _vp, _i, _i, _vp, C.c_int64, _vp]),

@@ -124,6 +124,18 @@ __device__ __forceinline__ int quantize(h1 x, h1 zp, h1 sc)
     return (int)r;
 }
 
+// The encoder's form of quantize(): same value, fewer instructions.  x - zp as one fp32 fma with
+// fp16 operands (exactly the rounded fp32 difference), IEEE divide, round-half-even, then the
+// hardware float->int conversion, which saturates and maps NaN to 0 as CUDA's __float2int_rn does.
+__device__ __forceinline__ int quantize_enc(h1 x, h1 zp, h1 sc)
+{
+    const float d = __builtin_fmaf((float)x, 1.0f, -(float)zp);
+    const float r = __builtin_rintf(d / (float)sc);
+    int q;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(q) : "v"(r));
+    return q < -8 ? -8 : (q > 7 ? 7 : q);
+}
+
 __device__ __forceinline__ h2 codes_to_h2(int q0, int q1) { return (h2){(h1)q0, (h1)q1}; }
 
 // Quantise one new token's channel pair with the current state and patch its two nibbles into the

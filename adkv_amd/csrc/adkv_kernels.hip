@@ -19,6 +19,8 @@
 
 #include "../../include/adkv_hip.h"
 
+#include <stdlib.h>
+
 #pragma clang fp contract(off)
 
 namespace adkv {
@@ -121,6 +123,16 @@ __device__ __forceinline__ void load_state(const h1 *src, Pair *st)
     }
 }
 
+// store_state for any channel count, including a single channel held in both halves of a pair
+template <int CPL>
+__device__ __forceinline__ void store_state_n(h1 *dst, const Pair *st)
+{
+    if (CPL >= 2)
+        store_state<CPL>(dst, st);
+    else
+        *reinterpret_cast<h2 *>(dst) = (h2){st[0].zp.x, st[0].sc.x};
+}
+
 // Which (head, segment) this lane works on.  Units beyond the end are clamped to the last one and
 // flagged inactive: they compute but never store.
 template <int D, int CPL, int BLK>
@@ -160,69 +172,179 @@ __device__ __forceinline__ void init_pairs(Pair *st, const h1 *zp, const h1 *sc,
 // ---------------------------------------------------------------------------------------------
 // encode_kv  (gemv.cu:168-308)
 // ---------------------------------------------------------------------------------------------
-template <int D, int CPL, int BLK>
+// The state at token t depends on every code before it, so the encoder is one serial chain per
+// channel and nothing but B*H*D is parallel.  A lane owns CPL consecutive channels (1, 2 or 4: the
+// launcher picks the widest that still gives every SIMD work, because a wave that is alone on its
+// SIMD issues an instruction only every ~5 ns whatever it is).  Input rows for the next two
+// supergroups are in flight while the current one is quantised.  The eight codes of a channel are
+// summed as signed q << 4t and biased once by 0x8888... instead of being masked in one by one.
+constexpr int ENC_PF = 3; // supergroup input buffers in rotation
+
+template <int CPL, int BLK>
 __global__ __launch_bounds__(BLK) void encode_kernel(
-    uint4 *__restrict__ cache, const h1 *__restrict__ kv_new,
+    uint32_t *__restrict__ cache, const h1 *__restrict__ kv_new,
     const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
     const h1 *__restrict__ be, const h1 *__restrict__ tg,
-    int BH, int H, int T, int n_super_cap, h1 *__restrict__ state_out, Seg sa)
+    int BH, int H, int T0, int T, int D, int n_super_cap, const h1 *__restrict__ state_in,
+    h1 *__restrict__ state_out, Seg sa)
 {
-    using G = Geo<D, CPL>;
-    const Unit<D, CPL, BLK> un(BH, 1);
-    const int bx = un.bx, c0 = un.c0;
-    const bool active = un.active;
+    // Quantises tokens [T0, T) of a stream whose first T0 tokens are already in the cache; kv_new
+    // holds the T - T0 new rows; state_in is the state after token T0-1 (ignored when T0 == 0).
+    constexpr int NP = CPL >= 2 ? CPL / 2 : 1;
+    const long total = (long)BH * D;
+    long ci = ((long)blockIdx.x * BLK + threadIdx.x) * CPL;
+    const bool active = ci < total;
+    if (!active)
+        ci = total - CPL;
+    const int bx = (int)(ci / D), c0 = (int)(ci % D);
     const int h = bx % H;
 
-    Pair st[G::NP];
-    init_pairs<D, CPL>(st, zp, sc, al, be, tg, h, bx, c0, 0, sa);
+    Pair st[NP];
+    if (CPL >= 2) {
+#pragma unroll
+        for (int p = 0; p < NP; p++)
+            load_pair(st[p], zp, sc, al, be, tg, h * D + c0 + 2 * p);
+    } else {
+        const int pi = h * D + c0;
+        st[0].zp = splat(zp[pi]);
+        st[0].sc = splat(sc[pi]);
+        st[0].al = splat(al[pi]);
+        st[0].be = splat(be[pi]);
+        st[0].omt = splat((h1)1.0f) - st[0].be * splat(tg[pi]);
+    }
+    if (T0 > 0) {
+        const h1 *si = state_in + ((size_t)bx * D + c0) * 2;
+        if (CPL >= 2) {
+            load_state<CPL>(si, st);
+        } else {
+            st[0].zp = splat(si[0]);
+            st[0].sc = splat(si[1]);
+        }
+    }
 
-    uint4 *cb = cache + (size_t)bx * n_super_cap * G::VPS + un.lh * G::NV;
-    const h1 *xb = kv_new + (size_t)bx * T * D + c0;
-    const int n_super = (T + 7) / 8;
+    uint32_t *cw = cache + (size_t)bx * n_super_cap * D + c0;
+    const h1 *xb = kv_new + (size_t)bx * (T - T0) * D + c0; // rows of tokens T0.. of this head
 
-    for (int sg = 0; sg < n_super; sg++) {
+    auto load_tok = [&](int t, h2 *x) {
+        if (CPL >= 2) {
+#pragma unroll
+            for (int p = 0; p < NP; p++)
+                x[p] = *reinterpret_cast<const h2 *>(xb + (size_t)(t - T0) * D + 2 * p);
+        } else {
+            x[0] = splat(xb[(size_t)(t - T0) * D]);
+        }
+    };
+    auto step = [&](const h2 *x, int tt, uint32_t *w) {
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            const int q0 = quantize_enc(x[p].x, st[p].zp.x, st[p].sc.x);
+            w[CPL >= 2 ? 2 * p : 0] += (uint32_t)q0 << (4 * tt);
+            int q1 = q0;
+            if (CPL >= 2) {
+                q1 = quantize_enc(x[p].y, st[p].zp.y, st[p].sc.y);
+                w[2 * p + 1] += (uint32_t)q1 << (4 * tt);
+            }
+            const h2 q = (h2){(h1)(short)q0, (h1)(short)q1};
+            update_pair(st[p], q, q * st[p].sc);
+        }
+    };
+    // bias adds 8 to the nibbles written now; keep selects nibbles of earlier tokens to preserve
+    auto store_sg = [&](int sg, const uint32_t *w, uint32_t bias, uint32_t keep) {
+        if (!active)
+            return;
+        uint32_t *dst = cw + (size_t)sg * D;
+        uint32_t o[CPL];
+#pragma unroll
+        for (int c = 0; c < CPL; c++)
+            o[c] = w[c] + bias;
+        if (keep) {
+#pragma unroll
+            for (int c = 0; c < CPL; c++)
+                o[c] = (o[c] & ~keep) | (dst[c] & keep);
+        }
+        if (CPL == 4)
+            *reinterpret_cast<uint4 *>(dst) = make_uint4(o[0], o[1], o[2], o[3]);
+        else if (CPL == 2)
+            *reinterpret_cast<uint2 *>(dst) = make_uint2(o[0], o[1]);
+        else
+            dst[0] = o[0];
+        // state before token (j+1)*interval
+        const int tend = sg * 8 + 8;
+        if (sa.ckpt != nullptr && tend <= T && tend % sa.ckpt_interval == 0) {
+            const int j = tend / sa.ckpt_interval - 1;
+            if (j < sa.n_ckpt_cap)
+                store_state_n<CPL>(sa.ckpt + (((size_t)bx * sa.n_ckpt_cap + j) * D + c0) * 2, st);
+        }
+    };
+
+    auto nib_mask = [](int k) { return k >= 8 ? 0xFFFFFFFFu : ((1u << (4 * k)) - 1u); };
+
+    // a stream that resumes inside a supergroup first completes it (nibbles below T0 are kept)
+    int t = T0;
+    if ((t & 7) && t < T) {
+        const int lo = t & 7, sg = t >> 3;
         uint32_t w[CPL];
 #pragma unroll
         for (int c = 0; c < CPL; c++)
             w[c] = 0u;
-        // issue the supergroup's loads first, then run the serial chain over them
-        h2 x[8][G::NP];
-#pragma unroll
-        for (int tt = 0; tt < 8; tt++) {
-            const int t = sg * 8 + tt;
-            if (t < T) {
-#pragma unroll
-                for (int p = 0; p < G::NP; p++)
-                    x[tt][p] = *reinterpret_cast<const h2 *>(xb + (size_t)t * D + 2 * p);
-            }
+        for (; t < T && (t >> 3) == sg; t++) {
+            h2 x[NP];
+            load_tok(t, x);
+            step(x, t & 7, w);
         }
+        const int hi = (t >> 3) == sg ? (t & 7) : 8;
+        store_sg(sg, w, 0x88888888u & nib_mask(hi) & ~nib_mask(lo), nib_mask(lo));
+    }
+
+    // full supergroups: no per-token conditions, inputs ENC_PF-1 supergroups ahead
+    const int sgb = t >> 3;                     // first full supergroup
+    const int nfull = (T - t) >> 3;
+    h2 xbuf[ENC_PF][8][NP];
 #pragma unroll
-        for (int tt = 0; tt < 8; tt++) {
-            const int t = sg * 8 + tt;
-            if (t < T) {
+    for (int i = 0; i < ENC_PF - 1; i++)
+        if (i < nfull) {
 #pragma unroll
-                for (int p = 0; p < G::NP; p++) {
-                    const h2 q = append_pair(w[2 * p], w[2 * p + 1], tt, x[tt][p], st[p]);
-                    update_pair(st[p], q, q * st[p].sc);
+            for (int tt = 0; tt < 8; tt++)
+                load_tok((sgb + i) * 8 + tt, xbuf[i][tt]);
+        }
+    for (int sg0 = 0; sg0 < nfull; sg0 += ENC_PF) {
+#pragma unroll
+        for (int i = 0; i < ENC_PF; i++) {
+            const int sg = sg0 + i;
+            if (sg < nfull) {
+                if (sg + ENC_PF - 1 < nfull) {
+#pragma unroll
+                    for (int tt = 0; tt < 8; tt++)
+                        load_tok((sgb + sg + ENC_PF - 1) * 8 + tt, xbuf[(i + ENC_PF - 1) % ENC_PF][tt]);
                 }
-            }
-        }
-        if (active) {
+                uint32_t w[CPL];
 #pragma unroll
-            for (int v = 0; v < G::NV; v++)
-                cb[(size_t)sg * G::VPS + v] =
-                    make_uint4(w[4 * v], w[4 * v + 1], w[4 * v + 2], w[4 * v + 3]);
-            // state before token (j+1)*interval
-            const int tend = sg * 8 + 8;
-            if (sa.ckpt != nullptr && tend <= T && tend % sa.ckpt_interval == 0) {
-                const int j = tend / sa.ckpt_interval - 1;
-                if (j < sa.n_ckpt_cap)
-                    store_state<CPL>(sa.ckpt + (((size_t)bx * sa.n_ckpt_cap + j) * D + c0) * 2, st);
+                for (int c = 0; c < CPL; c++)
+                    w[c] = 0u;
+#pragma unroll
+                for (int tt = 0; tt < 8; tt++)
+                    step(xbuf[i][tt], tt, w);
+                store_sg(sgb + sg, w, 0x88888888u, 0u); // code = q + 8
             }
         }
     }
+    // ragged last supergroup: codes of the tokens present, zero nibbles after them
+    t += nfull * 8;
+    if (t < T) {
+        const int ntail = T - t;
+        uint32_t w[CPL];
+#pragma unroll
+        for (int c = 0; c < CPL; c++)
+            w[c] = 0u;
+        for (int tt = 0; tt < ntail; tt++) {
+            h2 x[NP];
+            load_tok(t + tt, x);
+            step(x, tt, w);
+        }
+        store_sg(t >> 3, w, 0x88888888u & nib_mask(ntail), 0u);
+    }
     if (state_out != nullptr && active)
-        store_state<CPL>(state_out + ((size_t)bx * D + c0) * 2, st);
+        store_state_n<CPL>(state_out + ((size_t)bx * D + c0) * 2, st);
 }
 
 // Shared tail of the two decode kernels: quantise the new token with the state after token T-1,
@@ -840,7 +962,7 @@ static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval)
 
 extern "C" {
 
-int adkv_abi_version(void) { return 2; }
+int adkv_abi_version(void) { return 3; }
 
 int adkv_last_hip_error(void) { return g_last_hip_error; }
 
@@ -860,25 +982,29 @@ const char *adkv_strerror(int code)
     }
 }
 
-int adkv_encode_kv_ex(void *cache, const void *kv_new,
-                      const void *zp, const void *sc, const void *alpha, const void *beta,
-                      const void *tgt,
-                      int B, int H, int T, int D, int n_super_cap,
-                      void *state_out, void *ckpt_out, int n_ckpt_cap, int ckpt_interval,
-                      void *stream)
+static int encode_common(void *cache, const void *kv_new,
+                         const void *zp, const void *sc, const void *alpha, const void *beta,
+                         const void *tgt,
+                         int B, int H, int T0, int T, int D, int n_super_cap,
+                         const void *state_in, void *state_out, void *ckpt_out, int n_ckpt_cap,
+                         int ckpt_interval, void *stream)
 {
     if (!cache || !kv_new || !zp || !sc || !alpha || !beta || !tgt)
         return ADKV_E_NULL;
     int rc = check_common(B, H, T, D, n_super_cap);
     if (rc)
         return rc;
+    if (T0 < 0 || T0 > T)
+        return ADKV_E_SHAPE;
+    if (T0 > 0 && !state_in)
+        return ADKV_E_NULL;
     if ((T + 7) / 8 > n_super_cap)
         return ADKV_E_CAPACITY;
     if (((uintptr_t)cache & 15) || ((uintptr_t)kv_new & 3))
         return ADKV_E_ALIGN;
     if ((rc = check_ckpt(ckpt_out, n_ckpt_cap, ckpt_interval)))
         return rc;
-    if (T == 0 && state_out == nullptr)
+    if (T == T0 && (state_out == nullptr || state_out == state_in))
         return ADKV_OK;
     const int BH = B * H;
     hipStream_t st = (hipStream_t)stream;
@@ -888,10 +1014,58 @@ int adkv_encode_kv_ex(void *cache, const void *kv_new,
     seg.ckpt_interval = ckpt_out ? ckpt_interval : 0;
     seg.seg_tokens = T > 0 ? T : 1;
     seg.nseg = 1;
-    ADKV_DISPATCH_D(encode_kernel, (uint4 *)cache, (const h1 *)kv_new, (const h1 *)zp,
-                    (const h1 *)sc, (const h1 *)alpha, (const h1 *)beta, (const h1 *)tgt, BH, H, T,
-                    n_super_cap, (h1 *)state_out, seg);
+    // widest lane that still leaves every SIMD with about two waves
+    const long channels = (long)BH * D;
+    int cpl = 4;
+    while (cpl > 1 && channels / (64L * cpl) < 2L * N_SIMD)
+        cpl >>= 1;
+    if (const char *e = getenv("ADKV_ENCODE_CPL")) {
+        const int v = atoi(e);
+        if (v == 1 || v == 2 || v == 4)
+            cpl = v;
+    }
+    const long lanes = channels / cpl;
+    const dim3 grid((unsigned)((lanes + 255) / 256)), block(256);
+#define ADKV_ENC(C)                                                                              \
+    hipLaunchKernelGGL((encode_kernel<C, 256>), grid, block, 0, st, (uint32_t *)cache,           \
+                       (const h1 *)kv_new, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,    \
+                       (const h1 *)beta, (const h1 *)tgt, BH, H, T0, T, D, n_super_cap,          \
+                       (const h1 *)state_in, (h1 *)state_out, seg)
+    if (cpl == 4)
+        ADKV_ENC(4);
+    else if (cpl == 2)
+        ADKV_ENC(2);
+    else
+        ADKV_ENC(1);
+#undef ADKV_ENC
     return check_launch();
+}
+
+int adkv_encode_kv_ex(void *cache, const void *kv_new,
+                      const void *zp, const void *sc, const void *alpha, const void *beta,
+                      const void *tgt,
+                      int B, int H, int T, int D, int n_super_cap,
+                      void *state_out, void *ckpt_out, int n_ckpt_cap, int ckpt_interval,
+                      void *stream)
+{
+    return encode_common(cache, kv_new, zp, sc, alpha, beta, tgt, B, H, 0, T, D, n_super_cap,
+                         nullptr, state_out, ckpt_out, n_ckpt_cap, ckpt_interval, stream);
+}
+
+int adkv_append_kv(void *cache, const void *kv_new,
+                   const void *zp, const void *sc, const void *alpha, const void *beta,
+                   const void *tgt,
+                   int B, int H, int T0, int n_new, int D, int n_super_cap,
+                   void *state_io, void *ckpt, int n_ckpt_cap, int ckpt_interval, void *stream)
+{
+    if (!state_io)
+        return ADKV_E_NULL;
+    if (n_new < 0)
+        return ADKV_E_SHAPE;
+    if (n_new == 0)
+        return ADKV_OK; // nothing to quantise; state_io already is the answer
+    return encode_common(cache, kv_new, zp, sc, alpha, beta, tgt, B, H, T0, T0 + n_new, D,
+                         n_super_cap, state_io, state_io, ckpt, n_ckpt_cap, ckpt_interval, stream);
 }
 
 int adkv_encode_kv(void *cache, const void *kv_new,

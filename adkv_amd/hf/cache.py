@@ -11,7 +11,9 @@ reference's cache object works unchanged.  What differs is underneath:
   llama_adkv.py:104-123);
 * next to each code buffer lives a small checkpoint tensor holding the exact fp16 filter state
   every ``CKPT_INTERVAL`` tokens (4 bytes per channel per checkpoint, ~3 % of the codes at 256).
-  The kernels keep it up to date and use it to replay the time axis in independent segments.
+  The kernels keep it up to date and use it to replay the time axis in independent segments;
+* the filter state after the last prompt token is carried, so a prompt may be prefilled in chunks
+  (the reference refuses: llama_adkv.py:195-197).
 """
 from __future__ import annotations
 
@@ -19,7 +21,7 @@ import math
 
 import torch
 
-from ..kernel.gemv import encode_kv, forward_ov, forward_qk, softmax_scale_mask
+from ..kernel.gemv import append_kv, forward_ov, forward_qk, softmax_scale_mask
 
 SCALE_MIN = math.exp(-4.0)  # kept for API parity; the fp16 recurrence never clamps
 SCALE_MAX = math.exp(4.0)
@@ -40,6 +42,11 @@ class KVCacheLayer_ADKV:
         self._value_buf: torch.Tensor | None = None
         self._key_ckpt: torch.Tensor | None = None
         self._value_ckpt: torch.Tensor | None = None
+        # (zp, sc) after the last quantised token, [B, H, C, 2] fp16; lets a prompt arrive in chunks.
+        # A decode step appends inside the attention kernels and leaves these stale.
+        self._key_state: torch.Tensor | None = None
+        self._value_state: torch.Tensor | None = None
+        self._state_valid = False
         self._quant_len = 0
         self._cap_len = 0
         self._B = self._H = self._C = 0
@@ -91,6 +98,8 @@ class KVCacheLayer_ADKV:
         self._quant_len = 0
         (self._cap_len, self._key_buf, self._value_buf,
          self._key_ckpt, self._value_ckpt) = self._new_buffers(INIT_SEQ_LEN)
+        mk = lambda: torch.zeros((B, H, C, 2), dtype=torch.float16, device=device)
+        self._key_state, self._value_state, self._state_valid = mk(), mk(), True
 
     def _cap_buffers(self, T: int):
         """Make room for ``T`` tokens.  New slots are zero, as the append kernels expect."""
@@ -122,16 +131,16 @@ class KVCacheLayer_ADKV:
     def _append_tokens(self, key_states, value_states,
                        key_zp_init, key_scale_init, key_alpha, key_beta, key_quant_target,
                        value_zp_init, value_scale_init, value_alpha, value_beta, value_quant_target):
-        """Quantise ``[B, H, T, C]`` keys/values from token 0 into the packed buffers."""
+        """Quantise ``[B, H, T, C]`` keys/values as tokens ``quant_len ..`` of the stream."""
         v = self._view
         S = self._ckpt_interval
-        encode_kv(self._key_buf, key_states.to(torch.float16).contiguous(),
+        append_kv(self._key_buf, key_states.to(torch.float16).contiguous(),
                   v(key_zp_init), v(key_scale_init), v(key_alpha), v(key_beta), v(key_quant_target),
-                  SCALE_MIN, SCALE_MAX, ckpt=self._key_ckpt, ckpt_interval=S)
-        encode_kv(self._value_buf, value_states.to(torch.float16).contiguous(),
+                  self._quant_len, self._key_state, ckpt=self._key_ckpt, ckpt_interval=S)
+        append_kv(self._value_buf, value_states.to(torch.float16).contiguous(),
                   v(value_zp_init), v(value_scale_init), v(value_alpha), v(value_beta),
                   v(value_quant_target),
-                  SCALE_MIN, SCALE_MAX, ckpt=self._value_ckpt, ckpt_interval=S)
+                  self._quant_len, self._value_state, ckpt=self._value_ckpt, ckpt_interval=S)
         self._quant_len += key_states.shape[2]
 
     def prefill(self, key_states, value_states,
@@ -144,10 +153,13 @@ class KVCacheLayer_ADKV:
         self._check_geometry(B, H, C, key_states.device)
         if T == 0:
             return
-        if self._quant_len != 0:
+        if self._quant_len != 0 and not self._state_valid:
+            # The reference refuses every second prefill (llama_adkv.py:195-197).  Here a prompt may
+            # arrive in chunks because the filter state is carried; only after single-token decode
+            # steps, which append inside the attention kernels, is that state gone.
             raise NotImplementedError(
                 "ADKV prefill encodes from token 0; chunked prefill is not supported by the kernel")
-        self._cap_buffers(T)
+        self._cap_buffers(self._quant_len + T)
         self._append_tokens(key_states, value_states,
                             key_zp_init, key_scale_init, key_alpha, key_beta, key_quant_target,
                             value_zp_init, value_scale_init, value_alpha, value_beta,
@@ -184,6 +196,7 @@ class KVCacheLayer_ADKV:
                          v(value_quant_target), SCALE_MIN, SCALE_MAX,
                          ckpt=self._value_ckpt, ckpt_interval=S)
         self._quant_len = ctx + 1
+        self._state_valid = False
         return out.to(query_states.dtype), weights
 
     # ------------------------------------------------------------------ accounting

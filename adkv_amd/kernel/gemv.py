@@ -248,6 +248,57 @@ def encode_kv(
     return kv_cache
 
 
+def append_kv(
+    kv_cache: torch.Tensor,
+    kv_new: torch.Tensor,
+    kv_zp: torch.Tensor,
+    kv_sc: torch.Tensor,
+    kv_alpha: torch.Tensor,
+    kv_beta: torch.Tensor,
+    kv_t: torch.Tensor,
+    T0: int,
+    state: torch.Tensor,
+    *,
+    ckpt: torch.Tensor | None = None,
+    ckpt_interval: int = 0,
+) -> torch.Tensor:
+    """Streaming append (extension; the reference can only append inside forward_qk/forward_ov,
+    after an O(T) replay): quantise ``kv_new [B, nh, n, DIM]`` as tokens ``T0 .. T0+n-1``.
+
+    ``state`` ``[B, nh, DIM, 2]`` float16 carries (zp, sc): the state after token ``T0-1`` on entry
+    (ignored when ``T0 == 0``), the state after the last new token on return.  The cache ends up
+    byte-identical to ``encode_kv`` over all ``T0+n`` tokens.  Returns ``kv_cache``.
+    """
+    _chk(kv_new.dtype == torch.float16, "kv_new must be float16")
+    _chk(kv_cache.dtype == torch.uint8, "kv_cache must be uint8")
+    _chk(kv_cache.is_contiguous(), "kv_cache must be contiguous (written in place)")
+    B, nh, n, DIM = kv_new.shape
+    zp, sc, al, be, tg = _params((kv_zp, kv_sc, kv_alpha, kv_beta, kv_t),
+                                 ("kv_zp", "kv_sc", "kv_alpha", "kv_beta", "kv_t"), nh, DIM)
+    n_super_cap = kv_cache.shape[2]
+    _chk(kv_cache.shape[3] * _TILE == DIM, "kv_cache channel groups do not match kv_new head dim")
+    _chk(T0 >= 0, "T0 must be non-negative")
+    need = (T0 + n + 7) // 8
+    _chk(need <= n_super_cap,
+         f"kv_cache capacity too small: need {need} supergroups for {T0 + n} tokens, have {n_super_cap}")
+    _chk(DIM in _DIMS, "DIM must be 128, 256 or 512")
+    _chk(state.dtype == torch.float16 and state.is_contiguous() and state.numel() == B * nh * DIM * 2,
+         "state must be contiguous fp16 [B,nh,DIM,2]")
+    dev = _need_device(kv_cache, kv_new, zp, sc, al, be, tg, state)
+    cp, ccap, civ = _ckpt_args(ckpt, ckpt_interval, B, nh, DIM)
+    if n == 0:
+        return kv_cache
+    x = kv_new.contiguous()
+    with torch.cuda.device(dev):
+        rc = _lib.lib().adkv_append_kv(
+            kv_cache.data_ptr(), x.data_ptr(),
+            zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
+            B, nh, T0, n, DIM, n_super_cap, state.data_ptr(), cp, ccap, civ,
+            _lib.current_stream_ptr(dev))
+    _lib.check(rc, "append_kv")
+    return kv_cache
+
+
 def softmax_scale_mask(logits: torch.Tensor, scaling: float,
                        mask: torch.Tensor | None = None) -> torch.Tensor:
     """``softmax(logits.float()*scaling + mask) -> fp16`` in one launch.

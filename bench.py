@@ -34,6 +34,9 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=40)
     ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--workload", choices=["decode", "encode"], default="decode",
+                    help="decode = headline decode attention (cfg2); encode = streaming quantiser (cfg3: "
+                         "B=8 ctx=32768 prefill, then 256 single-token appends)")
     ap.add_argument("--batch", type=int, default=128)
     ap.add_argument("--heads", type=int, default=32)
     ap.add_argument("--dim", type=int, default=128)
@@ -85,12 +88,102 @@ def cpu_baseline(args, T, D):
     }
 
 
+def encode_main(args):
+    """cfg3: one step = prefill-quantise B x ctx tokens of K (one launch); afterwards 256 timed
+    single-token appends.  tokens quantised / s = B*ctx / t_prefill."""
+    import numpy as np
+    import torch
+    from adkv_amd import synth
+    from adkv_amd.kernel import gemv
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    B = 8 if args.batch == 128 else args.batch
+    T = 32768 if args.ctx == 4096 else args.ctx
+    H, D, S = args.heads, args.dim, (args.ckpt_interval or 256)
+    n_app = 256
+    p = synth.make_params(H, D).to(dev)
+    x = synth.make_k(B, H, T + n_app, D, dtype=torch.float16, device=dev)
+    xp = x[:, :, :T].contiguous()
+    cache = synth.alloc_cache(B, H, T + n_app + 8, D, dev)
+    ck = torch.zeros(B, H, (T + n_app) // S + 1, D, 2, dtype=torch.float16, device=dev)
+    state = torch.zeros(B, H, D, 2, dtype=torch.float16, device=dev)
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+
+    def prefill():
+        gemv.append_kv(cache, xp, *p.astuple(), 0, state, ckpt=ck, ckpt_interval=S)
+
+    for _ in range(args.warmup):
+        prefill()
+    torch.cuda.synchronize()
+    marks = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        e0, e1 = ev(), ev()
+        e0.record(); prefill(); e1.record()
+        marks.append((e0, e1))
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_step = wall * 1e3 / args.steps
+    k_ms = sum(a.elapsed_time(b) for a, b in marks) / len(marks)
+
+    toks = [x[:, :, T + i:T + i + 1].contiguous() for i in range(n_app)]
+    torch.cuda.synchronize()
+    a0, a1 = ev(), ev()
+    a0.record()
+    for i in range(n_app):
+        gemv.append_kv(cache, toks[i], *p.astuple(), T + i, state, ckpt=ck, ckpt_interval=S)
+    a1.record(); torch.cuda.synchronize()
+    append_us = a0.elapsed_time(a1) * 1e3 / n_app
+
+    # bit-exactness of the codes: two sampled heads against the oracle, whole stream
+    from oracle import oracle as O
+    np16 = lambda t: t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.float16)
+    exact = True
+    for (b, h) in [(0, 0), (B - 1, H - 1)]:
+        want = O.alloc_cache(1, 1, T + n_app + 8, D)
+        O.encode_kv_f16(want, np16(x[b:b + 1, h:h + 1]), *[np16(t)[h:h + 1] for t in p.astuple()])
+        exact &= bool(np.array_equal(cache[b:b + 1, h:h + 1].cpu().numpy(), want))
+
+    bytes_launch = B * H * T * D * 2.5
+    achieved = bytes_launch / (k_ms * 1e-3) / 1e9
+    res = {
+        "metric": "streaming quantiser tokens quantised/sec (B*ctx / prefill time, one K tensor)",
+        "value": B * T / (ms_step * 1e-3), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": f"cfg3 streaming quantise: prefill B={B} H={H} d={D} ctx={T} fp16 -> 4-bit codes, "
+                               f"then {n_app} single-token appends with carried state",
+                   "batch": B, "heads": H, "head_dim": D, "ctx": T, "bits": 4, "ckpt_interval": S},
+        "append_us_per_token_step": append_us,
+        "codes_bit_exact_vs_oracle": exact,
+        "roofline": {"kernel": "encode_kernel", "bound": "hbm", "achieved": achieved,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
+                     "traffic": None},
+    }
+    if not args.no_cpu_baseline:
+        hs, Ts = 2, 4096
+        xs = np16(x[:1, :hs, :Ts])
+        c = O.alloc_cache(1, hs, Ts, D)
+        t0 = time.perf_counter()
+        O.encode_kv_f16(c, xs, *[np16(t)[:hs] for t in p.astuple()])
+        dt = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": Ts / (dt * H / hs), "unit": "tokens/s", "cores": 1, "kind": "port",
+                               "sample": f"C oracle encode, 1 sequence x {hs} of {H} heads x {Ts} tokens "
+                                         f"in {dt:.2f} s; scaled linearly to {H} heads"}
+    print(json.dumps(res))
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (the path shards over batch/heads with no "
               "exchange; nothing multi-GPU is built). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
+
+    if args.workload == "encode":
+        return encode_main(args)
 
     import torch
     from adkv_amd import synth

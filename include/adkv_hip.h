@@ -104,6 +104,21 @@ int adkv_encode_kv_ex(void *cache, const void *kv_new,
                       void *state_out, void *ckpt_out, int n_ckpt_cap, int ckpt_interval,
                       void *stream);
 
+/*
+ * Streaming append: quantise n_new further tokens of a stream whose first T0 tokens are already
+ * in the cache, kv_new fp16 [B,H,n_new,D].  state_io fp16 [B,H,D,2] holds the state after token
+ * T0-1 on entry (ignored when T0 == 0) and after token T0+n_new-1 on return, so appending costs
+ * O(n_new) instead of the O(T0) replay that forward_qk/forward_ov pay to recover the state
+ * (src/adkv/kernel/gemv.cu:744-764).  Byte-identical to one adkv_encode_kv over all T0+n_new tokens;
+ * also lifts the reference's "prefill encodes from token 0" restriction
+ * (src/adkv/hf/llama_adkv.py:195-197).  Checkpoint entries crossed by the new tokens are written.
+ */
+int adkv_append_kv(void *cache, const void *kv_new,
+                   const void *zp, const void *sc, const void *alpha, const void *beta,
+                   const void *tgt,
+                   int B, int H, int T0, int n_new, int D, int n_super_cap,
+                   void *state_io, void *ckpt, int n_ckpt_cap, int ckpt_interval, void *stream);
+
 int adkv_forward_qk_ex(const void *q, void *k_cache, const void *k_new, void *logits,
                        const void *zp, const void *sc, const void *alpha, const void *beta,
                        const void *tgt,

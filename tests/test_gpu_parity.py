@@ -304,3 +304,36 @@ def test_full_size_segmented_matches_sequential(gpu):
     # fp32 partial sums are added in a different order: at most one fp16 ulp apart
     d = torch.abs(o1.float() - o2.float())
     assert torch.all(d <= 2.0 ** -10 * torch.clamp(o1.float().abs(), min=2.0 ** -4))
+
+
+@pytest.mark.parametrize("B,H,D,cuts", [
+    (2, 3, 128, [0, 5, 6, 8, 19, 40, 41, 64, 100]),     # resumes inside, at and across supergroups
+    (1, 2, 256, [0, 16, 17, 33]),
+    (1, 1, 512, [0, 3, 24]),
+    (2, 2, 128, [3, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18]),  # token by token
+])
+def test_streaming_append_equals_one_shot_encode(gpu, oracle, B, H, D, cuts):
+    """append_kv over any split of the stream == encode_kv over the whole stream: cache bytes,
+    carried state and checkpoints (interval 16) are identical."""
+    T, S = cuts[-1], 16
+    x, p = _inputs(B, H, T, D, seed=T + D)
+    pn = [_np16(t) for t in p.astuple()]
+    pg = [t.to(gpu) for t in p.astuple()]
+    want = oracle.alloc_cache(B, H, T + 8, D)
+    st_want = oracle.encode_kv_f16(want, _np16(x), *pn)
+    ncap = T // S + 1
+    ck_want = _oracle_ckpts(oracle, want, pn, T, S, ncap)
+
+    cache = synth.alloc_cache(B, H, T + 8, D, gpu)
+    ck = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=gpu)
+    state = torch.zeros(B, H, D, 2, dtype=torch.float16, device=gpu)
+    xg = x.to(gpu)
+    t0 = 0
+    for t1 in cuts:
+        r = gemv.append_kv(cache, xg[:, :, t0:t1].contiguous(), *pg, t0, state, ckpt=ck, ckpt_interval=S)
+        assert r is cache
+        t0 = t1
+    torch.cuda.synchronize()
+    assert np.array_equal(cache.cpu().numpy(), want)
+    assert np.array_equal(_np16(state).view(np.uint16), st_want)
+    assert np.array_equal(_np16(ck).view(np.uint16)[:, :, :T // S], ck_want[:, :, :T // S])

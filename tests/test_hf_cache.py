@@ -57,7 +57,7 @@ def test_cache_errors_cpu():
         c.decode(torch.zeros(1, 2, 2, 128), q, q, *kp, *kp)
     with pytest.raises(ValueError, match="supports MHA"):
         c.decode(torch.zeros(1, 4, 1, 128), q, q, *kp, *kp)
-    c._quant_len = 3
+    c._quant_len, c._state_valid = 3, False      # as after decode steps: the carried state is gone
     with pytest.raises(NotImplementedError, match="chunked prefill is not supported"):
         c.prefill(torch.zeros(1, 2, 4, 128), torch.zeros(1, 2, 4, 128), *kp, *kp)
     kv = KVCache_ADKV(3)
@@ -98,7 +98,9 @@ def test_prefill_then_decode_steps_match_oracle(gpu, oracle, monkeypatch, interv
 
     layer = KVCacheLayer_ADKV()
     kg, vg = _flat(kp.to(gpu)), _flat(vp.to(gpu))
-    layer.prefill(k[:, :, :T0].to(gpu), v[:, :, :T0].to(gpu), *kg, *vg)
+    # the prompt arrives in two chunks (cut inside a supergroup)
+    layer.prefill(k[:, :, :21].to(gpu), v[:, :, :21].to(gpu), *kg, *vg)
+    layer.prefill(k[:, :, 21:T0].to(gpu), v[:, :, 21:T0].to(gpu), *kg, *vg)
     assert layer.get_seq_length() == T0
     for s in range(steps):
         T = T0 + s
