@@ -31,6 +31,8 @@ PROTOTYPES = {
     "adkv_forward_qk_ex": (_i, [_vp] * 9 + [_i] * 5 + [_vp, _vp, _i, _i, _vp]),
     "adkv_forward_ov_workspace_bytes": (C.c_int64, [_i] * 6),
     "adkv_forward_ov_ex": (_i, [_vp] * 9 + [_i] * 5 + [_vp, _vp, _i, _i, _vp, C.c_int64, _vp]),
+    "adkv_fp16_decode_workspace_bytes": (C.c_int64, [_i] * 3),
+    "adkv_fp16_decode": (_i, [_vp] * 5 + [C.c_int64] + [_i] * 4 + [_f, _vp]),
 }
 
 _lib = None

@@ -6,7 +6,8 @@ import subprocess
 import sys
 
 _DIR = os.path.dirname(os.path.abspath(__file__))
-SOURCES = [os.path.join(_DIR, "csrc", "adkv_kernels.hip")]
+SOURCES = [os.path.join(_DIR, "csrc", "adkv_kernels.hip"),
+           os.path.join(_DIR, "csrc", "fp16_baseline.hip")]
 HEADERS = [os.path.join(_DIR, "csrc", "adkv_device.h"),
            os.path.join(_DIR, "..", "include", "adkv_hip.h")]
 LIB_PATH = os.path.join(_DIR, "libadkv_hip.so")

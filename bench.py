@@ -49,6 +49,8 @@ def parse():
                     help="also run three 1 GiB device-to-device copies (a known-size kernel to scale "
                          "rocprofv3 FETCH_SIZE/WRITE_SIZE readings by)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-fp16-comparator", action="store_true",
+                    help="skip timing the fp16-KV decode kernel beside the ADKV step")
     ap.add_argument("--cpu-sample-heads", type=int, default=0,
                     help="heads of one sequence timed on the host (0 = auto, about 10-30 s)")
     return ap.parse_args()
@@ -86,6 +88,33 @@ def cpu_baseline(args, T, D):
         "sample": f"C oracle, 1 sequence x {hs} of {H} heads x ctx {T}, one layer-step = {dt:.2f} s; "
                   f"scaled linearly to {H} heads",
     }
+
+
+def fp16_comparator(args, dev, adkv_ms):
+    """The same decode-attention step over an uncompressed fp16 K/V cache (split-K flash decoding,
+    adkv_fp16_decode), timed like the ADKV step.  Reported beside the headline value, never as it."""
+    import torch
+    from adkv_amd import synth
+    from adkv_amd.kernel.fp16_baseline import fp16_decode_attention
+
+    B, H, D, T = args.batch, args.heads, args.dim, args.ctx
+    K = synth.make_k(B, H, T, D, layer=0, dtype=torch.float16, device=dev)
+    V = synth.make_v(B, H, T, D, layer=0, dtype=torch.float16, device=dev)
+    q = synth.make_q(B, H, D, device=dev)
+    ws = torch.empty(B * H * (-(-T // 512)) * (D + 2) * 4, dtype=torch.uint8, device=dev)
+    for _ in range(max(2, args.warmup)):
+        fp16_decode_attention(q, K, V, D ** -0.5, ws)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        fp16_decode_attention(q, K, V, D ** -0.5, ws)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    kv_bytes = 2.0 * B * H * T * D * 2
+    return {"kernel": "adkv_fp16_decode (fp16 K/V, split-K flash decoding)", "ms_per_step": ms,
+            "tokens_per_s": B / (N_LAYERS_MODEL * ms * 1e-3),
+            "kv_GBps": kv_bytes / (ms * 1e-3) / 1e9, "hbm_frac": kv_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "adkv_speedup": ms / adkv_ms}
 
 
 def encode_main(args):
@@ -302,6 +331,8 @@ def main():
             "traffic": 1.1227e9 if (B, H, D, T, S) == (128, 32, 128, 4096, 256) else None,
         },
     }
+    if not args.no_fp16_comparator and D == 128:
+        res["fp16_kv_comparator"] = fp16_comparator(args, dev, ms_step)
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(args, T, D)
     print(json.dumps(res))

@@ -137,6 +137,15 @@ int adkv_forward_ov_ex(const void *attn, void *v_cache, const void *v_new, void 
                        void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
                        void *workspace, int64_t workspace_bytes, void *stream);
 
+/* ---- comparator, not part of the drop-in boundary ----
+ * fp16-KV single-query attention (split-K flash decoding), standing in for the uncompressed fp16
+ * cache that ADKV's memory and latency claims are made against (tools/memory_comparison_fig.py:46-56
+ * models its bytes; the reference ships no kernel for it).  q [B,H,128], K/V [B,H,T,128], out [B,H,128], all fp16;
+ * out = softmax(scaling * q.K^T) V.  D must be 128. */
+int64_t adkv_fp16_decode_workspace_bytes(int B, int H, int T);
+int adkv_fp16_decode(const void *q, const void *K, const void *V, void *out, void *workspace,
+                     int64_t workspace_bytes, int B, int H, int T, int D, float scaling, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

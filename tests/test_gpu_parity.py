@@ -337,3 +337,35 @@ def test_streaming_append_equals_one_shot_encode(gpu, oracle, B, H, D, cuts):
     assert np.array_equal(cache.cpu().numpy(), want)
     assert np.array_equal(_np16(state).view(np.uint16), st_want)
     assert np.array_equal(_np16(ck).view(np.uint16)[:, :, :T // S], ck_want[:, :, :T // S])
+
+
+# ------------------------------------------------------------------ fp16-KV comparator kernel
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,H,T", [(1, 2, 1), (2, 3, 17), (2, 4, 512), (1, 4, 513), (2, 2, 1500)])
+def test_fp16_comparator_matches_fp32_attention(gpu, B, H, T):
+    """The uncompressed-cache comparator is ordinary attention: check it against fp32 torch math
+    (tolerance 2e-3 absolute on outputs of magnitude <= 1, the bar used for the ADKV outputs)."""
+    import torch
+    from adkv_amd.kernel.fp16_baseline import fp16_decode_attention
+
+    g = torch.Generator().manual_seed(100 + T)
+    q = torch.randn(B, H, 128, generator=g).half().cuda()
+    K = torch.randn(B, H, T, 128, generator=g).half().cuda()
+    V = torch.randn(B, H, T, 128, generator=g).half().cuda()
+    scaling = 128 ** -0.5
+    out = fp16_decode_attention(q, K, V, scaling)
+    torch.cuda.synchronize()
+    w = torch.softmax(torch.einsum("bhd,bhtd->bht", q.float(), K.float()) * scaling, dim=-1)
+    ref = torch.einsum("bht,bhtd->bhd", w, V.float())
+    assert (out.float() - ref).abs().max().item() <= 2e-3
+
+
+@pytest.mark.gpu
+def test_fp16_comparator_rejects_other_head_dims(gpu):
+    import torch
+    from adkv_amd.kernel.fp16_baseline import fp16_decode_attention
+
+    q = torch.zeros(1, 1, 256, dtype=torch.float16, device="cuda")
+    K = torch.zeros(1, 1, 8, 256, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError):
+        fp16_decode_attention(q, K, K, 1.0)
