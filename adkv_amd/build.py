@@ -7,6 +7,7 @@ import sys
 
 _DIR = os.path.dirname(os.path.abspath(__file__))
 SOURCES = [os.path.join(_DIR, "csrc", "adkv_kernels.hip"),
+           os.path.join(_DIR, "csrc", "adkv_fp32.hip"),
            os.path.join(_DIR, "csrc", "fp16_baseline.hip")]
 HEADERS = [os.path.join(_DIR, "csrc", "adkv_device.h"),
            os.path.join(_DIR, "..", "include", "adkv_hip.h")]

@@ -962,7 +962,7 @@ static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval)
 
 extern "C" {
 
-int adkv_abi_version(void) { return 3; }
+int adkv_abi_version(void) { return 4; }
 
 int adkv_last_hip_error(void) { return g_last_hip_error; }
 
@@ -1186,6 +1186,50 @@ int adkv_softmax(const void *logits, void *weights, const void *mask,
                        (const h1 *)logits, (h1 *)weights, (const float *)mask, n,
                        mask ? rows_per_mask_row : 1, scaling);
     return check_launch();
+}
+
+static int64_t pad256(int64_t n) { return (n + 255) & ~(int64_t)255; }
+
+int64_t adkv_decode_fused_workspace_bytes(int B, int H, int T, int D, int n_ckpt_cap, int ckpt_interval)
+{
+    if (B <= 0 || H <= 0 || T < 0)
+        return 0;
+    const int64_t row = pad256((int64_t)B * H * (T + 1) * 2);
+    return 2 * row + adkv_forward_ov_workspace_bytes(B, H, T, D, n_ckpt_cap, ckpt_interval);
+}
+
+int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k_new, const void *v_new,
+                      const void *const *k_params, const void *const *v_params,
+                      const void *mask, int rows_per_mask_row, float scaling,
+                      void *out, void *weights_out,
+                      int B, int H, int T, int D, int n_super_cap,
+                      void *k_ckpt, void *v_ckpt, int n_ckpt_cap, int ckpt_interval,
+                      void *workspace, int64_t workspace_bytes, void *stream)
+{
+    if (!k_params || !v_params || !workspace)
+        return workspace ? ADKV_E_NULL : ADKV_E_WORKSPACE;
+    if (B <= 0 || H <= 0 || T < 0)
+        return ADKV_E_SHAPE;
+    if (workspace_bytes < adkv_decode_fused_workspace_bytes(B, H, T, D, n_ckpt_cap, ckpt_interval))
+        return ADKV_E_WORKSPACE;
+    if ((uintptr_t)workspace & 255)
+        return ADKV_E_ALIGN;
+    const int64_t row = pad256((int64_t)B * H * (T + 1) * 2);
+    char *ws = (char *)workspace;
+    void *logits = ws;
+    void *weights = weights_out ? weights_out : (void *)(ws + row);
+    int rc = adkv_forward_qk_ex(q, k_cache, k_new, logits, k_params[0], k_params[1], k_params[2],
+                                k_params[3], k_params[4], B, H, T, D, n_super_cap, nullptr,
+                                k_ckpt, n_ckpt_cap, ckpt_interval, stream);
+    if (rc)
+        return rc;
+    rc = adkv_softmax(logits, weights, mask, B * H, T + 1, rows_per_mask_row, scaling, stream);
+    if (rc)
+        return rc;
+    return adkv_forward_ov_ex(weights, v_cache, v_new, out, v_params[0], v_params[1], v_params[2],
+                              v_params[3], v_params[4], B, H, T, D, n_super_cap, nullptr,
+                              v_ckpt, n_ckpt_cap, ckpt_interval, ws + 2 * row,
+                              workspace_bytes - 2 * row, stream);
 }
 
 } // extern "C"

@@ -21,7 +21,7 @@ import math
 
 import torch
 
-from ..kernel.gemv import append_kv, forward_ov, forward_qk, softmax_scale_mask
+from ..kernel.gemv import append_kv, decode_fused, decode_fused_workspace_bytes
 
 SCALE_MIN = math.exp(-4.0)  # kept for API parity; the fp16 recurrence never clamps
 SCALE_MAX = math.exp(4.0)
@@ -32,6 +32,19 @@ GROWTH = 1.5         # geometric growth factor once the initial capacity is exce
 CKPT_INTERVAL = 256  # tokens between state checkpoints (multiple of 8); 0 disables them
 
 _HEAD_DIMS = (128, 256, 512)
+
+# Scratch for the fused decode call (logits + partial sums), one per (device, stream): every layer's
+# step on a stream runs after the previous one, so they can share it.
+_workspaces: dict[tuple, torch.Tensor] = {}
+
+
+def _workspace(dev: torch.device, need: int) -> torch.Tensor:
+    key = (dev.index, torch.cuda.current_stream(dev).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.empty(max(need, 1) * 5 // 4, dtype=torch.uint8, device=dev)
+        _workspaces[key] = ws
+    return ws
 
 
 class KVCacheLayer_ADKV:
@@ -186,15 +199,16 @@ class KVCacheLayer_ADKV:
         f16 = lambda t: t.to(torch.float16).contiguous()
         v = self._view
         S = self._ckpt_interval
-        logits = forward_qk(f16(query_states), self._key_buf, f16(key_states),
-                            v(key_zp_init), v(key_scale_init), v(key_alpha), v(key_beta),
-                            v(key_quant_target), ctx, SCALE_MIN, SCALE_MAX,
-                            ckpt=self._key_ckpt, ckpt_interval=S)
-        weights = softmax_scale_mask(logits, scaling, attention_mask)
-        out = forward_ov(weights, self._value_buf, f16(value_states),
-                         v(value_zp_init), v(value_scale_init), v(value_alpha), v(value_beta),
-                         v(value_quant_target), SCALE_MIN, SCALE_MAX,
-                         ckpt=self._value_ckpt, ckpt_interval=S)
+        dev = query_states.device
+        ncap = self._key_ckpt.shape[2] if S else 0
+        ws = _workspace(dev, decode_fused_workspace_bytes(B, H, ctx, C, ncap, S))
+        out, weights = decode_fused(
+            f16(query_states), self._key_buf, self._value_buf, f16(key_states), f16(value_states),
+            (v(key_zp_init), v(key_scale_init), v(key_alpha), v(key_beta), v(key_quant_target)),
+            (v(value_zp_init), v(value_scale_init), v(value_alpha), v(value_beta),
+             v(value_quant_target)),
+            ctx, scaling, attention_mask,
+            k_ckpt=self._key_ckpt, v_ckpt=self._value_ckpt, ckpt_interval=S, workspace=ws)
         self._quant_len = ctx + 1
         self._state_valid = False
         return out.to(query_states.dtype), weights

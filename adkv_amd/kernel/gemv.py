@@ -327,3 +327,85 @@ def softmax_scale_mask(logits: torch.Tensor, scaling: float,
                                      float(scaling), _lib.current_stream_ptr(dev))
     _lib.check(rc, "softmax_scale_mask")
     return out
+
+
+def decode_fused(
+    q: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    k_new: torch.Tensor,
+    v_new: torch.Tensor,
+    k_params,
+    v_params,
+    T: int,
+    scaling: float,
+    mask: torch.Tensor | None = None,
+    *,
+    k_ckpt: torch.Tensor | None = None,
+    v_ckpt: torch.Tensor | None = None,
+    ckpt_interval: int = 0,
+    workspace: torch.Tensor | None = None,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """One decode-attention step of a layer through a single library call.
+
+    The body of the reference's ``KVCacheLayer_ADKV.decode`` (src/adkv/hf/llama_adkv.py:245-276):
+    ``forward_qk`` -> ``softmax(logits*scaling + mask)`` -> ``forward_ov``, with ``k_new`` / ``v_new``
+    appended at slot ``T`` of both caches.  ``k_params`` / ``v_params`` are the five ``[nh, DIM]``
+    fp16 tensors ``(zp, sc, alpha, beta, quant_target)``.  Returns ``(out [B,nh,DIM] fp16,
+    weights [B,nh,T+1] fp16)``.  ``workspace`` (uint8, 256-byte aligned, sized by
+    ``decode_fused_workspace_bytes``) may be passed to avoid the per-call allocation.
+    """
+    for t, n in ((q, "q"), (k_new, "k_new"), (v_new, "v_new")):
+        _chk(t.dtype == torch.float16, f"{n} must be float16")
+    for t, n in ((k_cache, "k_cache"), (v_cache, "v_cache")):
+        _chk(t.dtype == torch.uint8, f"{n} must be uint8")
+        _chk(t.is_contiguous(), f"{n} must be contiguous (appended in place)")
+    _chk(k_cache.shape == v_cache.shape, "k_cache and v_cache shapes differ")
+    B, nh = q.shape[0], q.shape[1]
+    n_super_cap, DIM = k_cache.shape[2], k_cache.shape[3] * _TILE
+    kp = _params(k_params, ("k_zp", "k_sc", "k_alpha", "k_beta", "k_t"), nh, DIM)
+    vp = _params(v_params, ("v_zp", "v_sc", "v_alpha", "v_beta", "v_t"), nh, DIM)
+    _chk(DIM == q.shape[-1], "q head dimension does not match k_cache")
+    _chk(T >= 0, "T must be non-negative")
+    _chk((T >> 1) // _TILE < n_super_cap, f"k_cache has no free supergroup to append token {T}")
+    _chk(DIM in _DIMS, "DIM must be 128, 256 or 512")
+    dev = _need_device(q, k_cache, v_cache, k_new, v_new, *kp, *vp)
+    n = T + 1
+    rpm, mptr, mk = 1, None, None
+    if mask is not None:
+        mk = mask[:, :, 0, :] if mask.dim() == 4 else mask
+        _chk(mk.dim() == 3 and mk.shape[0] == B and mk.shape[2] == n and mk.shape[1] in (1, nh),
+             "mask must broadcast to [B, nh, n]")
+        rpm = nh if mk.shape[1] == 1 else 1
+        mk = mk.to(device=dev, dtype=torch.float32).contiguous()
+        mptr = mk.data_ptr()
+    kcp, ccap, civ = _ckpt_args(k_ckpt, ckpt_interval, B, nh, DIM)
+    vcp, vcap, _ = _ckpt_args(v_ckpt, ckpt_interval, B, nh, DIM)
+    _chk((k_ckpt is None) == (v_ckpt is None) and ccap == vcap,
+         "k_ckpt and v_ckpt must both be given, with the same capacity, or both omitted")
+    L = _lib.lib()
+    need = L.adkv_decode_fused_workspace_bytes(B, nh, T, DIM, ccap, civ)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    _chk(workspace.dtype == torch.uint8 and workspace.is_cuda and workspace.numel() >= need,
+         "workspace too small")
+    qf = q.contiguous()
+    knf = k_new.reshape(B * nh, DIM).contiguous()
+    vnf = v_new.reshape(B * nh, DIM).contiguous()
+    out = torch.empty((B, nh, DIM), dtype=torch.float16, device=dev)
+    weights = torch.empty((B, nh, n), dtype=torch.float16, device=dev)
+    arr = _lib.C.c_void_p * 5
+    with torch.cuda.device(dev):
+        rc = L.adkv_decode_fused(
+            qf.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), knf.data_ptr(), vnf.data_ptr(),
+            arr(*[t.data_ptr() for t in kp]), arr(*[t.data_ptr() for t in vp]),
+            mptr, rpm, float(scaling), out.data_ptr(), weights.data_ptr(),
+            B, nh, T, DIM, n_super_cap, kcp, vcp, ccap, civ,
+            workspace.data_ptr(), workspace.numel(), _lib.current_stream_ptr(dev))
+    _lib.check(rc, "decode_fused")
+    return out, weights
+
+
+def decode_fused_workspace_bytes(B: int, nh: int, T: int, DIM: int, n_ckpt_cap: int = 0,
+                                 ckpt_interval: int = 0) -> int:
+    return int(_lib.lib().adkv_decode_fused_workspace_bytes(B, nh, T, DIM, n_ckpt_cap, ckpt_interval))

@@ -137,6 +137,52 @@ int adkv_forward_ov_ex(const void *attn, void *v_cache, const void *v_new, void 
                        void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
                        void *workspace, int64_t workspace_bytes, void *stream);
 
+/*
+ * One decode-attention step of one layer in a single call: forward_qk -> scale/mask/softmax ->
+ * forward_ov, appending k_new / v_new at slot T of both caches.  Replaces the body of
+ * KVCacheLayer_ADKV.decode (src/adkv/hf/llama_adkv.py:245-276).
+ * k_params / v_params: host arrays of five device pointers {zp, sc, alpha, beta, tgt}, each
+ * fp16 [H, D].  mask: optional fp32 additive mask as in adkv_softmax.  out: fp16 [B, H, D].
+ * weights_out: optional fp16 [B, H, T+1] (the attention weights the reference returns); when
+ * NULL they live in the workspace.  Checkpoint tensors as in the _ex entry points (NULL = none).
+ * workspace: >= adkv_decode_fused_workspace_bytes(...) bytes, 256-byte aligned.
+ */
+int64_t adkv_decode_fused_workspace_bytes(int B, int H, int T, int D, int n_ckpt_cap,
+                                          int ckpt_interval);
+int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k_new,
+                      const void *v_new, const void *const *k_params, const void *const *v_params,
+                      const void *mask, int rows_per_mask_row, float scaling,
+                      void *out, void *weights_out,
+                      int B, int H, int T, int D, int n_super_cap,
+                      void *k_ckpt, void *v_ckpt, int n_ckpt_cap, int ckpt_interval,
+                      void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
+ * fp32 ("train / eval") form of the recurrence: fake-quantise a token stream with the state kept
+ * in fp32 and every operation separately rounded.  Replaces the forward pass of
+ * _adkv_chunk_forward + IntQuantSTE (src/adkv/train/train_model.py:8-22,61-81) and the Triton
+ * kernel _adkv_quant_kernel (src/adkv/hf/llama_adkv_eval.py:34-118, one call per K and per V).
+ *   x         [B, T, C] of x_dtype (ADKV_DT_*), element strides stride_b / stride_t, channel
+ *             stride 1;  xhat: same layout, may alias x (in-place, as the eval cache does) or NULL
+ *   codes     optional int8 [B, T, C] contiguous, the integer q per element
+ *   zp_state, sc_state   optional fp32 [B, C]: read as the starting state unless zp_init/sc_init
+ *             are given, and always written with the state after the last token
+ *   zp_init, sc_init     optional fp32 [C]: starting state broadcast over the batch
+ *   alpha, beta, tgt     fp32 [C]
+ *   zp_seq, sc_seq       optional fp32 [B, T, C] contiguous: the state BEFORE each token
+ *             (train_model.py:66-68)
+ *   lower_limit/upper_limit   integer code range (train_model.py:96-97), sc_min/sc_max the
+ *             clamp of the scale (train_model.py:98-99).
+ */
+#define ADKV_DT_F32 0
+#define ADKV_DT_F16 1
+#define ADKV_DT_BF16 2
+int adkv_quant_f32(const void *x, void *xhat, void *codes, void *zp_state, void *sc_state,
+                   const void *zp_init, const void *sc_init, const void *alpha,
+                   const void *beta, const void *tgt, void *zp_seq, void *sc_seq,
+                   int B, int T, int C, int64_t stride_b, int64_t stride_t, int x_dtype,
+                   int lower_limit, int upper_limit, float sc_min, float sc_max, void *stream);
+
 /* ---- comparator, not part of the drop-in boundary ----
  * fp16-KV single-query attention (split-K flash decoding), standing in for the uncompressed fp16
  * cache that ADKV's memory and latency claims are made against (tools/memory_comparison_fig.py:46-56

@@ -369,3 +369,50 @@ def test_fp16_comparator_rejects_other_head_dims(gpu):
     K = torch.zeros(1, 1, 8, 256, dtype=torch.float16, device="cuda")
     with pytest.raises(RuntimeError):
         fp16_decode_attention(q, K, K, 1.0)
+
+
+# ------------------------------------------------------------------ single-call decode step
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,H,T,D,S,masked", [
+    (2, 4, 257, 128, 0, False), (2, 3, 530, 128, 64, True), (1, 2, 100, 256, 16, False),
+    (1, 2, 0, 128, 0, False)])
+def test_decode_fused_equals_three_calls(gpu, B, H, T, D, S, masked):
+    """adkv_decode_fused is the three entry points chained inside the library: outputs, weights,
+    appended codes and checkpoints must equal the separate calls bit for bit."""
+    kp = [t.to(gpu) for t in synth.make_params(H, D, seed=3).astuple()]
+    vp = [t.to(gpu) for t in synth.make_params(H, D, seed=4).astuple()]
+    k = synth.make_k(B, H, T + 1, D, dtype=torch.float16).to(gpu)
+    v = synth.make_v(B, H, T + 1, D, dtype=torch.float16).to(gpu)
+    q = synth.make_q(B, H, D).to(gpu)
+    scaling = D ** -0.5
+    ncap = (T + 8) // S + 1 if S else 0
+    mask = None
+    if masked:
+        mask = torch.zeros(B, 1, 1, T + 1)
+        mask[:, :, :, :5] = torch.finfo(torch.float32).min
+        mask = mask.to(gpu)
+
+    def fresh():
+        kc, vc = synth.alloc_cache(B, H, T + 8, D, gpu), synth.alloc_cache(B, H, T + 8, D, gpu)
+        kk = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=gpu) if S else None
+        vk = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=gpu) if S else None
+        if T:
+            gemv.encode_kv(kc, k[:, :, :T].contiguous(), *kp, SMIN, SMAX, ckpt=kk, ckpt_interval=S)
+            gemv.encode_kv(vc, v[:, :, :T].contiguous(), *vp, SMIN, SMAX, ckpt=vk, ckpt_interval=S)
+        return kc, vc, kk, vk
+
+    kc, vc, kk, vk = fresh()
+    logits = gemv.forward_qk(q, kc, k[:, :, T:], *kp, T, SMIN, SMAX, ckpt=kk, ckpt_interval=S)
+    w = gemv.softmax_scale_mask(logits, scaling, mask)
+    out = gemv.forward_ov(w, vc, v[:, :, T:], *vp, SMIN, SMAX, ckpt=vk, ckpt_interval=S)
+
+    kc2, vc2, kk2, vk2 = fresh()
+    out2, w2 = gemv.decode_fused(q, kc2, vc2, k[:, :, T:], v[:, :, T:], kp, vp, T, scaling, mask,
+                                 k_ckpt=kk2, v_ckpt=vk2, ckpt_interval=S)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
+    assert torch.equal(w.view(torch.int16), w2.view(torch.int16))
+    assert torch.equal(kc, kc2) and torch.equal(vc, vc2)
+    if S:
+        assert torch.equal(kk.view(torch.int16), kk2.view(torch.int16))
+        assert torch.equal(vk.view(torch.int16), vk2.view(torch.int16))
