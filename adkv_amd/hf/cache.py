@@ -213,6 +213,55 @@ class KVCacheLayer_ADKV:
         self._state_valid = False
         return out.to(query_states.dtype), weights
 
+    # ------------------------------------------------------------------ save / restore
+    def state_dict(self) -> dict:
+        """Everything needed to continue decoding elsewhere: the used part of the code buffers, the
+        state checkpoints that go with them and, while it is still valid, the carried filter state.
+        Plain tensors and ints, so ``torch.save`` / ``torch.load(weights_only=True)`` round-trip it."""
+        if self._key_buf is None:
+            return {"quant_len": 0}
+        ns = self._n_super(self._quant_len)
+        nck = self._quant_len // self._ckpt_interval if self._ckpt_interval else 0
+        sd = {"quant_len": self._quant_len, "ckpt_interval": self._ckpt_interval,
+              "geometry": (self._B, self._H, self._C),
+              "key_codes": self._key_buf[:, :, :ns].contiguous(),
+              "value_codes": self._value_buf[:, :, :ns].contiguous()}
+        if self._ckpt_interval:
+            sd["key_ckpt"] = self._key_ckpt[:, :, :nck].contiguous()
+            sd["value_ckpt"] = self._value_ckpt[:, :, :nck].contiguous()
+        if self._state_valid:
+            sd["key_state"], sd["value_state"] = self._key_state.clone(), self._value_state.clone()
+        return sd
+
+    def load_state_dict(self, sd: dict, device=None) -> None:
+        """Rebuild the layer from ``state_dict()`` output on ``device`` (default: where the saved
+        tensors live).  Slots past the saved tokens are zero, as the append kernels expect."""
+        if sd.get("quant_len", 0) == 0 and "key_codes" not in sd:
+            self.__init__()
+            return
+        B, H, C = sd["geometry"]
+        dev = torch.device(device) if device is not None else sd["key_codes"].device
+        T = int(sd["quant_len"])
+        self._ckpt_interval = int(sd["ckpt_interval"])
+        self._init_buffers(B, H, C, dev)
+        self._cap_buffers(T)
+        ns = self._n_super(T)
+        if tuple(sd["key_codes"].shape) != (B, H, ns, C // 4, 4, 4):
+            raise ValueError("saved code tensor does not match its geometry")
+        self._key_buf[:, :, :ns].copy_(sd["key_codes"])
+        self._value_buf[:, :, :ns].copy_(sd["value_codes"])
+        if self._ckpt_interval:
+            nck = T // self._ckpt_interval
+            if sd["key_ckpt"].shape[2] != nck:
+                raise ValueError("saved checkpoints do not cover the saved tokens")
+            self._key_ckpt[:, :, :nck].copy_(sd["key_ckpt"])
+            self._value_ckpt[:, :, :nck].copy_(sd["value_ckpt"])
+        self._quant_len = T
+        self._state_valid = "key_state" in sd
+        if self._state_valid:
+            self._key_state.copy_(sd["key_state"])
+            self._value_state.copy_(sd["value_state"])
+
     # ------------------------------------------------------------------ accounting
     def nbytes(self) -> int:
         """Device bytes held by this layer (codes + checkpoints)."""
@@ -241,6 +290,19 @@ class KVCache_ADKV(list):
 
     is_sliding = [False]
     is_compileable = False
+
+    def save(self, path) -> None:
+        """Write all layers to one file (tensors moved to the CPU)."""
+        cpu = lambda v: v.cpu() if isinstance(v, torch.Tensor) else v
+        torch.save([{k: cpu(v) for k, v in layer.state_dict().items()} for layer in self], path)
+
+    @classmethod
+    def load(cls, path, device) -> "KVCache_ADKV":
+        layers = torch.load(path, map_location="cpu", weights_only=True)
+        cache = cls(len(layers))
+        for layer, sd in zip(cache, layers):
+            layer.load_state_dict(sd, device)
+        return cache
 
 
 def adkv_cache_bytes(B: int, H: int, C: int, tokens: int, layers: int, bits: int = 4,

@@ -152,3 +152,50 @@ def test_tiny_llama_generate(gpu):
     assert torch.equal(out[:, :12], ids)
     # the first generated token comes from the dense prefill path: identical by construction
     assert torch.equal(out[:, 12], ref[:, 12])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("interval", [0, 16])
+def test_cache_save_and_restore_continues_identically(gpu, tmp_path, monkeypatch, interval):
+    """A cache saved after prefill + decode steps and restored from the file continues exactly like
+    the original: same outputs, same codes, same checkpoints; a cache saved right after prefill
+    also keeps its carried state and accepts another prompt chunk."""
+    monkeypatch.setattr(C, "CKPT_INTERVAL", interval)
+    B, H, D, T0 = 2, 2, 128, 41
+    kp, vp = synth.make_params(H, D, seed=3), synth.make_params(H, D, seed=4)
+    kg, vg = _flat(kp.to(gpu)), _flat(vp.to(gpu))
+    k = synth.make_k(B, H, T0 + 40, D, dtype=torch.float16).to(gpu)
+    v = synth.make_v(B, H, T0 + 40, D, dtype=torch.float16).to(gpu)
+    q = torch.randn(B, H, 1, D, generator=torch.Generator().manual_seed(5)).half().to(gpu)
+
+    def step(layer, t):
+        return layer.decode(q, k[:, :, t:t + 1], v[:, :, t:t + 1], *kg, *vg, scaling=D ** -0.5)
+
+    cache = KVCache_ADKV(1)
+    cache[0].prefill(k[:, :, :T0], v[:, :, :T0], *kg, *vg)
+    cache.save(tmp_path / "prefill.pt")
+    for t in range(T0, T0 + 3):
+        step(cache[0], t)
+    cache.save(tmp_path / "decoded.pt")
+
+    again = KVCache_ADKV.load(tmp_path / "decoded.pt", gpu)
+    assert again[0].get_seq_length() == T0 + 3 and not again[0]._state_valid
+    for t in range(T0 + 3, T0 + 30):              # crosses capacity growth in both
+        o1, w1 = step(cache[0], t)
+        o2, w2 = step(again[0], t)
+        assert torch.equal(o1.view(torch.int16), o2.view(torch.int16))
+        assert torch.equal(w1.view(torch.int16), w2.view(torch.int16))
+    n = C.KVCacheLayer_ADKV._n_super(T0 + 30)
+    assert torch.equal(cache[0].key_states[:, :, :n], again[0].key_states[:, :, :n])
+    assert torch.equal(cache[0].value_states[:, :, :n], again[0].value_states[:, :, :n])
+    with pytest.raises(NotImplementedError):
+        again[0].prefill(k[:, :, :4], v[:, :, :4], *kg, *vg)
+
+    # restored right after prefill: the carried state survives, so a second chunk is accepted
+    chunked = KVCache_ADKV.load(tmp_path / "prefill.pt", gpu)
+    chunked[0].prefill(k[:, :, T0:T0 + 9], v[:, :, T0:T0 + 9], *kg, *vg)
+    whole = KVCacheLayer_ADKV()
+    whole.prefill(k[:, :, :T0 + 9], v[:, :, :T0 + 9], *kg, *vg)
+    n = C.KVCacheLayer_ADKV._n_super(T0 + 9)
+    assert torch.equal(chunked[0].key_states[:, :, :n], whole.key_states[:, :, :n])
+    assert torch.equal(chunked[0].value_states[:, :, :n], whole.value_states[:, :, :n])
