@@ -1,0 +1,412 @@
+// Decode kernels for head dim 128 that put the contraction on the matrix cores, for GQ >= 1 query
+// heads per KV head.  Included inside namespace adkv by adkv_kernels.hip.
+//
+// The fp16 replay of the filter state (the dominant cost) is the same per-lane arithmetic as in
+// qk_kernel / ov_kernel and runs once per KV head; only what happens to the dequantised value
+// differs.  v_mfma_f32_4x4x4_16B_f16 multiplies sixteen independent 4x4 blocks per instruction:
+// lane 4b+r supplies row r of A and column r of B of block b (four fp16 each) and receives column
+// r of D (four fp32, one per row).
+//
+//   QK:  D[token][head] += A[token][4 channels] * B[4 channels][head]
+//        The dequantised keys of one supergroup (8 tokens x 2 heads x 128 channels) go through a
+//        wave-private LDS tile; a block is (KV head, 4 tokens, a quarter of the channels), eight
+//        instructions walk the quarter, two DPP rotations add the quarters.  No cross-lane
+//        reduction of per-lane partial dot products is left.
+//   OV:  D[head][channel] += A[head][4 tokens] * B[4 tokens][channel]
+//        B is the lane's own channel over four consecutive tokens (two v_perm_b32 per channel pair
+//        repack token-major pairs), A the attention weights of the block's heads: every lane gets
+//        the outputs of all GQ heads for its own channels, with no data leaving the lane.
+#pragma once
+
+typedef float f4v __attribute__((ext_vector_type(4)));
+typedef _Float16 h4v __attribute__((ext_vector_type(4)));
+
+constexpr int GQA_D = 128;
+constexpr int GQA_CPL = 4;
+constexpr int TILE_ROW64 = 65;               // 8-byte words per token row: 2 heads x 32 lanes + 1 pad
+constexpr int TILE_WORDS64 = 8 * TILE_ROW64; // per wave
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF,
+                                                                  0xF, false));
+}
+
+__device__ __forceinline__ h4v as_h4(uint32_t lo, uint32_t hi)
+{
+    return __builtin_bit_cast(h4v, make_uint2(lo, hi));
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward_qk with GQ query heads per KV head
+// ---------------------------------------------------------------------------------------------
+template <int GQ, int BLK>
+__global__ __launch_bounds__(BLK) void qk_gqa_kernel(
+    const h1 *__restrict__ q, uint4 *__restrict__ cache, const h1 *__restrict__ k_new,
+    h1 *__restrict__ out,
+    const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
+    const h1 *__restrict__ be, const h1 *__restrict__ tg,
+    int BH, int H, int T, int n_super_cap, h1 *__restrict__ state_out, Seg sa)
+{
+    constexpr int D = GQA_D, CPL = GQA_CPL;
+    constexpr int NB = (GQ + 3) / 4; // column sets of four heads
+    using G = Geo<D, CPL>;
+    __shared__ uint2 smem[LUT_WORDS64 + (BLK / 64) * TILE_WORDS64];
+    const uint2 *lut = smem;
+    lut_fill(smem, threadIdx.x, BLK);
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63;
+    const uint32_t lane_copy = (uint32_t)(lane & (LUT_COPIES - 1)) * 8u;
+    uint2 *tile = smem + LUT_WORDS64 + (threadIdx.x >> 6) * TILE_WORDS64;
+
+    const Unit<D, CPL, BLK> un(BH, sa.nseg);
+    const int bx = un.bx, lh = un.lh, c0 = un.c0;
+    const bool active = un.active;
+    const bool last = un.seg == sa.nseg - 1;
+    const int h = bx % H;
+
+    Pair st[G::NP];
+    init_pairs<D, CPL>(st, zp, sc, al, be, tg, h, bx, c0, un.seg, sa);
+
+    // matrix-core roles of this lane: block (hh, tg4, qd), row/column r
+    const int r = lane & 3, qd = (lane >> 2) & 3, tg4 = (lane >> 4) & 1;
+    // B operands: q of head r (+4 per column set), channels of quarter qd, four per instruction
+    uint2 qb[NB][8];
+#pragma unroll
+    for (int n = 0; n < NB; n++) {
+        const int g = 4 * n + r;
+        const uint2 *src = reinterpret_cast<const uint2 *>(q + ((size_t)bx * GQ + (g < GQ ? g : 0)) * D) + qd * 8;
+#pragma unroll
+        for (int m = 0; m < 8; m++)
+            qb[n][m] = (g < GQ) ? src[m] : make_uint2(0u, 0u);
+    }
+    const uint2 *arow = tile + (tg4 * 4 + r) * TILE_ROW64 + (lane >> 5) * 32 + qd * 8;
+
+    const int t0 = un.seg * sa.seg_tokens;
+    const int t1 = last ? T : t0 + sa.seg_tokens;
+    uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV;
+    const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;
+    const int nfull = (t1 - t0) >> 3;
+
+    // logits of the tile's tokens: read the A operands, run the instructions, add the quarters,
+    // lane (.., qd, r) stores token tg4*4+qd of head r
+    auto emit_read = [&](uint2 *a) {
+#pragma unroll
+        for (int m = 0; m < 8; m++)
+            a[m] = arow[m];
+    };
+    auto emit_finish = [&](const uint2 *a, int sg, int ntok) {
+#pragma unroll
+        for (int n = 0; n < NB; n++) {
+            f4v d = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int m = 0; m < 8; m++)
+                d = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(a[m].x, a[m].y), as_h4(qb[n][m].x, qb[n][m].y),
+                                                       d, 0, 0, 0);
+            float s[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                float v = d[i];
+                v += dpp_mov<0x128>(v); // row_ror:8
+                v += dpp_mov<0x124>(v); // row_ror:4
+                s[i] = v;
+            }
+            const float mine = qd == 0 ? s[0] : qd == 1 ? s[1] : qd == 2 ? s[2] : s[3];
+            const int tok = tg4 * 4 + qd, g = 4 * n + r;
+            if (active && g < GQ && tok < ntok)
+                out[((size_t)bx * GQ + g) * (T + 1) + t0 + sg * 8 + tok] = (h1)mine;
+        }
+    };
+
+    auto token = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2]) {
+        uint32_t kh[G::NP];
+#pragma unroll
+        for (int p = 0; p < G::NP; p++) {
+            Pair &s = st[p];
+            const h2 qs = as_h2(e[p][t].x) * s.sc;
+            kh[p] = as_u32(qs + s.zp);
+            update_pair_abs(s, as_h2(e[p][t].y), qs);
+        }
+        tile[t * TILE_ROW64 + lane] = make_uint2(kh[0], kh[1]);
+#pragma unroll
+        for (int p = 0; p < G::NP; p++)
+            e[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    uint4 buf[PF][G::NV];
+    uint2 lk[G::NP][8];
+    uint32_t nb[G::NP][2];
+    uint2 areg[8];
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+#pragma unroll
+        for (int v = 0; v < G::NV; v++)
+            buf[i][v] = (i < nfull) ? cb[(size_t)i * G::VPS + v] : make_uint4(0, 0, 0, 0);
+    }
+    if (nfull > 0) {
+        pair_bytes_of<D, CPL>(buf[0], nb);
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+#pragma unroll
+            for (int p = 0; p < G::NP; p++)
+                lk[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+    }
+    for (int sg0 = 0; sg0 < nfull; sg0 += PF) {
+#pragma unroll
+        for (int i = 0; i < PF; i++) {
+            const int sg = sg0 + i;
+            if (sg < nfull) {
+                pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
+                if (sg + PF < nfull) {
+#pragma unroll
+                    for (int v = 0; v < G::NV; v++)
+                        buf[i][v] = cb[(size_t)(sg + PF) * G::VPS + v];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int t = 0; t < 3; t++)
+                    token(t, lk, nb);
+                // the tile reads of supergroup sg-1 were issued before these three tokens
+                // overwrote its first rows (LDS operations of a wave execute in order)
+                if (sg > 0)
+                    emit_finish(areg, sg - 1, 8);
+#pragma unroll
+                for (int t = 3; t < 8; t++)
+                    token(t, lk, nb);
+                emit_read(areg);
+            }
+        }
+    }
+    if (nfull > 0)
+        emit_finish(areg, nfull - 1, 8);
+    if (!last)
+        return;
+
+    // ragged tail (T % 8 tokens, gemv.cu:648-654) and the appended token share one more tile
+    const int ntail = (t1 - t0) & 7;
+    if (ntail) {
+        const uint4 u = cb[(size_t)nfull * G::VPS];
+        const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+        for (int tt = 0; tt < ntail; tt++) {
+            uint32_t kh[2];
+#pragma unroll
+            for (int pp = 0; pp < 2; pp++) {
+                Pair &s = st[pp];
+                const uint32_t na = (w[2 * pp] >> (4 * tt)) & 0xFu;
+                const uint32_t nbb = (w[2 * pp + 1] >> (4 * tt)) & 0xFu;
+                const h2 qc = codes_to_h2((int)na - 8, (int)nbb - 8);
+                const h2 qs = qc * s.sc;
+                kh[pp] = as_u32(qs + s.zp);
+                update_pair(s, qc, qs);
+            }
+            tile[tt * TILE_ROW64 + lane] = make_uint2(kh[0], kh[1]);
+        }
+    }
+    if (active)
+        publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
+    h2 deq[G::NP];
+    append_new_token<D, CPL>(cbh, T, k_new + (size_t)bx * D + c0, st, deq, active);
+    tile[ntail * TILE_ROW64 + lane] = make_uint2(as_u32(deq[0]), as_u32(deq[1]));
+    emit_read(areg);
+    emit_finish(areg, nfull, ntail + 1);
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward_ov with GQ query heads per KV head
+// ---------------------------------------------------------------------------------------------
+template <int GQ, int BLK>
+__global__ __launch_bounds__(BLK) void ov_gqa_kernel(
+    const h1 *__restrict__ attn, uint4 *__restrict__ cache, const h1 *__restrict__ v_new,
+    h1 *__restrict__ out, float *__restrict__ partial,
+    const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
+    const h1 *__restrict__ be, const h1 *__restrict__ tg,
+    int BH, int H, int T, int n_super_cap, h1 *__restrict__ state_out, Seg sa)
+{
+    constexpr int D = GQA_D, CPL = GQA_CPL;
+    constexpr int NB = (GQ + 3) / 4;
+    using G = Geo<D, CPL>;
+    __shared__ uint2 lut[LUT_WORDS64];
+    lut_fill(lut, threadIdx.x, BLK);
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const uint32_t lane_copy = (uint32_t)(lane & (LUT_COPIES - 1)) * 8u;
+
+    const Unit<D, CPL, BLK> un(BH, sa.nseg);
+    const int bx = un.bx, lh = un.lh, c0 = un.c0;
+    const bool active = un.active;
+    const bool last = un.seg == sa.nseg - 1;
+    const int h = bx % H;
+    const int r = lane & 3;
+
+    Pair st[G::NP];
+    init_pairs<D, CPL>(st, zp, sc, al, be, tg, h, bx, c0, un.seg, sa);
+    f4v acc[NB][CPL]; // [column set][channel of this lane], element i = head 4n+i
+#pragma unroll
+    for (int n = 0; n < NB; n++)
+#pragma unroll
+        for (int c = 0; c < CPL; c++)
+            acc[n][c] = (f4v){0.0f, 0.0f, 0.0f, 0.0f};
+
+    const int t0 = un.seg * sa.seg_tokens;
+    const int t1 = last ? T : t0 + sa.seg_tokens;
+    uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV;
+    const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;
+    const int nfull = (t1 - t0) >> 3;
+    // A operand rows: the weights of head r (+4 per column set) of this lane's KV head
+    const h1 *wb[NB];
+    bool wok[NB];
+#pragma unroll
+    for (int n = 0; n < NB; n++) {
+        wok[n] = 4 * n + r < GQ;
+        wb[n] = attn + ((size_t)bx * GQ + (wok[n] ? 4 * n + r : 0)) * (T + 1) + t0;
+    }
+    auto load_w = [&](int n, int sg) {
+        uint4 v;
+        __builtin_memcpy(&v, wb[n] + (size_t)sg * 8, 16); // rows are only 2-byte aligned
+        return wok[n] ? v : make_uint4(0u, 0u, 0u, 0u);
+    };
+
+    // four tokens of dequantised values, token-major pairs -> per-channel h4 -> four instructions
+    auto contract = [&](const uint32_t (*kh)[4], const uint4 *wv, int half) {
+        uint32_t b[CPL][2];
+#pragma unroll
+        for (int p = 0; p < G::NP; p++) {
+            b[2 * p][0] = __builtin_amdgcn_perm(kh[p][1], kh[p][0], 0x05040100u);
+            b[2 * p][1] = __builtin_amdgcn_perm(kh[p][3], kh[p][2], 0x05040100u);
+            b[2 * p + 1][0] = __builtin_amdgcn_perm(kh[p][1], kh[p][0], 0x07060302u);
+            b[2 * p + 1][1] = __builtin_amdgcn_perm(kh[p][3], kh[p][2], 0x07060302u);
+        }
+#pragma unroll
+        for (int n = 0; n < NB; n++) {
+            const h4v a = half ? as_h4(wv[n].z, wv[n].w) : as_h4(wv[n].x, wv[n].y);
+#pragma unroll
+            for (int c = 0; c < CPL; c++)
+                acc[n][c] = __builtin_amdgcn_mfma_f32_4x4x4f16(a, as_h4(b[c][0], b[c][1]), acc[n][c], 0, 0, 0);
+        }
+    };
+    uint32_t kh[G::NP][4];
+    auto token = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2]) {
+#pragma unroll
+        for (int p = 0; p < G::NP; p++) {
+            Pair &s = st[p];
+            const h2 qs = as_h2(e[p][t].x) * s.sc;
+            kh[p][t & 3] = as_u32(qs + s.zp);
+            update_pair_abs(s, as_h2(e[p][t].y), qs);
+        }
+#pragma unroll
+        for (int p = 0; p < G::NP; p++)
+            e[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    uint4 buf[PF][G::NV];
+    uint4 wbuf[PF][NB];
+    uint2 lk[G::NP][8];
+    uint32_t nb[G::NP][2];
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+#pragma unroll
+        for (int v = 0; v < G::NV; v++)
+            buf[i][v] = (i < nfull) ? cb[(size_t)i * G::VPS + v] : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int n = 0; n < NB; n++)
+            wbuf[i][n] = (i < nfull) ? load_w(n, i) : make_uint4(0, 0, 0, 0);
+    }
+    if (nfull > 0) {
+        pair_bytes_of<D, CPL>(buf[0], nb);
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+#pragma unroll
+            for (int p = 0; p < G::NP; p++)
+                lk[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+    }
+    for (int sg0 = 0; sg0 < nfull; sg0 += PF) {
+#pragma unroll
+        for (int i = 0; i < PF; i++) {
+            const int sg = sg0 + i;
+            if (sg < nfull) {
+                pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
+                uint4 wcur[NB];
+#pragma unroll
+                for (int n = 0; n < NB; n++)
+                    wcur[n] = wbuf[i][n];
+                if (sg + PF < nfull) {
+#pragma unroll
+                    for (int v = 0; v < G::NV; v++)
+                        buf[i][v] = cb[(size_t)(sg + PF) * G::VPS + v];
+#pragma unroll
+                    for (int n = 0; n < NB; n++)
+                        wbuf[i][n] = load_w(n, sg + PF);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+                    token(t, lk, nb);
+                contract(kh, wcur, 0);
+#pragma unroll
+                for (int t = 4; t < 8; t++)
+                    token(t, lk, nb);
+                contract(kh, wcur, 1);
+            }
+        }
+    }
+
+    if (last) {
+        // ragged tail, then the appended token: a handful of tokens, plain fp32 multiply-adds
+        auto add_token = [&](const h2 *vd, int t) {
+#pragma unroll
+            for (int g = 0; g < GQ; g++) {
+                const float wt = (float)attn[((size_t)bx * GQ + g) * (T + 1) + t];
+#pragma unroll
+                for (int p = 0; p < G::NP; p++) {
+                    acc[g >> 2][2 * p][g & 3] = __builtin_fmaf(wt, (float)vd[p].x, acc[g >> 2][2 * p][g & 3]);
+                    acc[g >> 2][2 * p + 1][g & 3] =
+                        __builtin_fmaf(wt, (float)vd[p].y, acc[g >> 2][2 * p + 1][g & 3]);
+                }
+            }
+        };
+        const int ntail = (t1 - t0) & 7;
+        if (ntail) {
+            const uint4 u = cb[(size_t)nfull * G::VPS];
+            const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+            for (int tt = 0; tt < ntail; tt++) {
+                h2 vd[2];
+#pragma unroll
+                for (int pp = 0; pp < 2; pp++) {
+                    Pair &s = st[pp];
+                    const uint32_t na = (w[2 * pp] >> (4 * tt)) & 0xFu;
+                    const uint32_t nbb = (w[2 * pp + 1] >> (4 * tt)) & 0xFu;
+                    const h2 qc = codes_to_h2((int)na - 8, (int)nbb - 8);
+                    const h2 qs = qc * s.sc;
+                    vd[pp] = qs + s.zp;
+                    update_pair(s, qc, qs);
+                }
+                add_token(vd, t0 + nfull * 8 + tt);
+            }
+        }
+        if (active)
+            publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
+        h2 deq[G::NP];
+        append_new_token<D, CPL>(cbh, T, v_new + (size_t)bx * D + c0, st, deq, active);
+        add_token(deq, T);
+    }
+    if (!active)
+        return;
+#pragma unroll
+    for (int g = 0; g < GQ; g++) {
+        const size_t row = (size_t)bx * GQ + g;
+        const float o0 = acc[g >> 2][0][g & 3], o1 = acc[g >> 2][1][g & 3];
+        const float o2 = acc[g >> 2][2][g & 3], o3 = acc[g >> 2][3][g & 3];
+        if (sa.nseg == 1) {
+            h2 *o = reinterpret_cast<h2 *>(out + row * D + c0);
+            o[0] = (h2){(h1)o0, (h1)o1};
+            o[1] = (h2){(h1)o2, (h1)o3};
+        } else {
+            *reinterpret_cast<float4 *>(partial + ((size_t)un.seg * BH * GQ + row) * D + c0) =
+                make_float4(o0, o1, o2, o3);
+        }
+    }
+}

@@ -29,6 +29,9 @@ namespace adkv {
 #define ADKV_PF 4
 #endif
 constexpr int PF = ADKV_PF; // supergroups in flight per lane
+#ifndef ADKV_MFMA_DEFAULT
+#define ADKV_MFMA_DEFAULT 0
+#endif
 
 template <int D, int CPL>
 struct Geo {
@@ -764,6 +767,7 @@ __global__ __launch_bounds__(256) void ov_finalize_kernel(const float *__restric
 // softmax(float(logits)*scaling + mask) -> fp16   (llama_adkv.py:266-271)
 // ---------------------------------------------------------------------------------------------
 constexpr int SM_BLOCK = 256;
+constexpr int SM_KEEP_FWD = 20;
 
 __device__ __forceinline__ float block_reduce(float v, float *sm, bool is_max)
 {
@@ -795,7 +799,7 @@ __global__ __launch_bounds__(SM_BLOCK) void softmax_kernel(
     const float *mk = mask ? mask + (size_t)(row / rows_per_mask_row) * n : nullptr;
 
     // rows up to SM_BLOCK*KEEP elements are read from memory once and kept in registers
-    constexpr int KEEP = 20;
+    constexpr int KEEP = SM_KEEP_FWD;
     float x[KEEP];
     const bool fits = n <= SM_BLOCK * KEEP;
     float mx = -INFINITY;
@@ -854,6 +858,81 @@ __global__ __launch_bounds__(SM_BLOCK) void softmax_kernel(
     }
 }
 
+// Rows longer than one workgroup can hold in registers are cut into chunks of SM_CHUNK elements,
+// one workgroup each: the first pass leaves (max, sum of exp(x - max)) per chunk, the second
+// combines a row's chunks and normalises.  Each logit is read twice and nothing depends on the
+// order in which workgroups run.
+constexpr int SM_KEEP = SM_KEEP_FWD;
+constexpr int SM_CHUNK = SM_BLOCK * SM_KEEP;
+
+__device__ __forceinline__ void softmax_load_chunk(const h1 *l, const float *mk, int n, int base,
+                                                   float scaling, float *x, float &mx)
+{
+    mx = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < SM_KEEP; k++) {
+        const int i = base + threadIdx.x + k * SM_BLOCK;
+        x[k] = -INFINITY;
+        if (i < n) {
+            x[k] = (float)l[i] * scaling;
+            if (mk)
+                x[k] += mk[i];
+        }
+        mx = fmaxf(mx, x[k]);
+    }
+}
+
+__global__ __launch_bounds__(SM_BLOCK) void softmax_part_kernel(
+    const h1 *__restrict__ logits, const float *__restrict__ mask, float2 *__restrict__ part,
+    int n, int nchunk, int rows_per_mask_row, float scaling)
+{
+    __shared__ float sm[SM_BLOCK / 64];
+    const int row = blockIdx.y, ck = blockIdx.x;
+    const h1 *l = logits + (size_t)row * n;
+    const float *mk = mask ? mask + (size_t)(row / rows_per_mask_row) * n : nullptr;
+    float x[SM_KEEP], mx;
+    softmax_load_chunk(l, mk, n, ck * SM_CHUNK, scaling, x, mx);
+    mx = block_reduce(mx, sm, true);
+    float sum = 0.0f;
+    if (mx > -INFINITY) {
+#pragma unroll
+        for (int k = 0; k < SM_KEEP; k++)
+            sum += __expf(x[k] - mx);
+    }
+    sum = block_reduce(sum, sm, false);
+    if (threadIdx.x == 0)
+        part[(size_t)row * nchunk + ck] = make_float2(mx, sum);
+}
+
+__global__ __launch_bounds__(SM_BLOCK) void softmax_norm_kernel(
+    const h1 *__restrict__ logits, h1 *__restrict__ weights, const float *__restrict__ mask,
+    const float2 *__restrict__ part, int n, int nchunk, int rows_per_mask_row, float scaling)
+{
+    const int row = blockIdx.y, ck = blockIdx.x;
+    const h1 *l = logits + (size_t)row * n;
+    h1 *w = weights + (size_t)row * n;
+    const float *mk = mask ? mask + (size_t)(row / rows_per_mask_row) * n : nullptr;
+    const float2 *pr = part + (size_t)row * nchunk;
+    float M = -INFINITY;
+    for (int k = 0; k < nchunk; k++)
+        M = fmaxf(M, pr[k].x);
+    float Z = 0.0f;
+    for (int k = 0; k < nchunk; k++) {
+        const float2 p = pr[k];
+        if (p.x > -INFINITY)
+            Z += p.y * __expf(p.x - M);
+    }
+    const float inv = 1.0f / Z;
+    float x[SM_KEEP], mx;
+    softmax_load_chunk(l, mk, n, ck * SM_CHUNK, scaling, x, mx);
+#pragma unroll
+    for (int k = 0; k < SM_KEEP; k++) {
+        const int i = ck * SM_CHUNK + threadIdx.x + k * SM_BLOCK;
+        if (i < n)
+            w[i] = (h1)(__expf(x[k] - M) * inv);
+    }
+}
+
 } // namespace adkv
 
 // ---------------------------------------------------------------------------------------------
@@ -887,6 +966,8 @@ static int check_common(int B, int H, int T, int D, int n_super_cap)
 static inline int lanes_per_head(int D) { return D == 128 ? 32 : 64; }
 
 // Waves a SIMD should hold for packed-f16 issue to run near full rate, and SIMDs on the device.
+#include "adkv_gqa_kernels.h"
+
 constexpr int WAVES_PER_SIMD_TARGET = 4;
 constexpr int N_SIMD = 256 * 4;
 
@@ -949,6 +1030,41 @@ static void launch_units(long threads, int big, F256 f256, FBIG fbig)
         break;                                        \
     }
 
+// Matrix-core kernels (head dim 128): 16-wave workgroups for big launches, 8-wave ones otherwise
+// (their LDS tile leaves room for one workgroup per CU either way).
+#define ADKV_LAUNCH_GQA(KERNEL, GQV, ...)                                                          \
+    do {                                                                                            \
+        const long threads = (long)BH * seg.nseg * 32;                                              \
+        if (threads >= 1024L * 256)                                                                 \
+            hipLaunchKernelGGL((KERNEL<GQV, 1024>), dim3((unsigned)((threads + 1023) / 1024)),      \
+                               dim3(1024), 0, st, __VA_ARGS__);                                     \
+        else                                                                                        \
+            hipLaunchKernelGGL((KERNEL<GQV, 512>), dim3((unsigned)((threads + 511) / 512)),         \
+                               dim3(512), 0, st, __VA_ARGS__);                                      \
+    } while (0)
+
+#define ADKV_DISPATCH_GQ(KERNEL, ...)                                                              \
+    switch (GQ) {                                                                                   \
+    case 1: ADKV_LAUNCH_GQA(KERNEL, 1, __VA_ARGS__); break;                                         \
+    case 2: ADKV_LAUNCH_GQA(KERNEL, 2, __VA_ARGS__); break;                                         \
+    case 4: ADKV_LAUNCH_GQA(KERNEL, 4, __VA_ARGS__); break;                                         \
+    case 8: ADKV_LAUNCH_GQA(KERNEL, 8, __VA_ARGS__); break;                                         \
+    default: return ADKV_E_UNSUPPORTED;                                                             \
+    }
+
+// Whether single-query-head launches (GQ == 1, head dim 128) also take the matrix-core kernels:
+// the built-in choice, overridden by ADKV_MFMA=0/1 in the environment, overridden by
+// adkv_set_mha_kernel().
+static int g_mha_kernel = -1;
+static bool mfma_for_mha()
+{
+    if (g_mha_kernel < 0) {
+        const char *e = getenv("ADKV_MFMA");
+        g_mha_kernel = (e ? atoi(e) : ADKV_MFMA_DEFAULT) != 0;
+    }
+    return g_mha_kernel != 0;
+}
+
 static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval)
 {
     if (!ckpt)
@@ -962,7 +1078,9 @@ static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval)
 
 extern "C" {
 
-int adkv_abi_version(void) { return 4; }
+int adkv_abi_version(void) { return 5; }
+
+void adkv_set_mha_kernel(int use_matrix_cores) { g_mha_kernel = use_matrix_cores; }
 
 int adkv_last_hip_error(void) { return g_last_hip_error; }
 
@@ -1078,6 +1196,45 @@ int adkv_encode_kv(void *cache, const void *kv_new,
                              state_out, nullptr, 0, 0, stream);
 }
 
+int adkv_forward_qk_gqa(const void *q, void *k_cache, const void *k_new, void *logits,
+                        const void *zp, const void *sc, const void *alpha, const void *beta,
+                        const void *tgt,
+                        int B, int Hq, int H, int T, int D, int n_super_cap,
+                        void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
+                        void *stream)
+{
+    if (!q || !k_cache || !k_new || !logits || !zp || !sc || !alpha || !beta || !tgt)
+        return ADKV_E_NULL;
+    int rc = check_common(B, H, T, D, n_super_cap);
+    if (rc)
+        return rc;
+    if (Hq <= 0 || Hq % H)
+        return ADKV_E_SHAPE;
+    const int GQ = Hq / H;
+    if (GQ > 1 && D != 128)
+        return ADKV_E_UNSUPPORTED;
+    if ((T >> 3) >= n_super_cap)
+        return ADKV_E_CAPACITY;
+    if (((uintptr_t)k_cache & 15) || ((uintptr_t)q & 7) || ((uintptr_t)k_new & 3))
+        return ADKV_E_ALIGN;
+    if ((rc = check_ckpt(ckpt, n_ckpt_cap, ckpt_interval)))
+        return rc;
+    const int BH = B * H;
+    hipStream_t st = (hipStream_t)stream;
+    const Seg seg = plan_segments(ckpt, n_ckpt_cap, ckpt_interval, BH, T, D);
+    if (D == 128 && (GQ > 1 || mfma_for_mha())) {
+        ADKV_DISPATCH_GQ(qk_gqa_kernel, (const h1 *)q, (uint4 *)k_cache, (const h1 *)k_new,
+                         (h1 *)logits, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,
+                         (const h1 *)beta, (const h1 *)tgt, BH, H, T, n_super_cap, (h1 *)state_out,
+                         seg);
+        return check_launch();
+    }
+    ADKV_DISPATCH_D(qk_kernel, (const h1 *)q, (uint4 *)k_cache, (const h1 *)k_new, (h1 *)logits,
+                    (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha, (const h1 *)beta,
+                    (const h1 *)tgt, BH, H, T, n_super_cap, (h1 *)state_out, seg);
+    return check_launch();
+}
+
 int adkv_forward_qk_ex(const void *q, void *k_cache, const void *k_new, void *logits,
                        const void *zp, const void *sc, const void *alpha, const void *beta,
                        const void *tgt,
@@ -1085,24 +1242,8 @@ int adkv_forward_qk_ex(const void *q, void *k_cache, const void *k_new, void *lo
                        void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
                        void *stream)
 {
-    if (!q || !k_cache || !k_new || !logits || !zp || !sc || !alpha || !beta || !tgt)
-        return ADKV_E_NULL;
-    int rc = check_common(B, H, T, D, n_super_cap);
-    if (rc)
-        return rc;
-    if ((T >> 3) >= n_super_cap)
-        return ADKV_E_CAPACITY;
-    if (((uintptr_t)k_cache & 15) || ((uintptr_t)q & 3) || ((uintptr_t)k_new & 3))
-        return ADKV_E_ALIGN;
-    if ((rc = check_ckpt(ckpt, n_ckpt_cap, ckpt_interval)))
-        return rc;
-    const int BH = B * H;
-    hipStream_t st = (hipStream_t)stream;
-    const Seg seg = plan_segments(ckpt, n_ckpt_cap, ckpt_interval, BH, T, D);
-    ADKV_DISPATCH_D(qk_kernel, (const h1 *)q, (uint4 *)k_cache, (const h1 *)k_new, (h1 *)logits,
-                    (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha, (const h1 *)beta,
-                    (const h1 *)tgt, BH, H, T, n_super_cap, (h1 *)state_out, seg);
-    return check_launch();
+    return adkv_forward_qk_gqa(q, k_cache, k_new, logits, zp, sc, alpha, beta, tgt, B, H, H, T, D,
+                               n_super_cap, state_out, ckpt, n_ckpt_cap, ckpt_interval, stream);
 }
 
 int adkv_forward_qk(const void *q, void *k_cache, const void *k_new, void *logits,
@@ -1124,18 +1265,23 @@ int64_t adkv_forward_ov_workspace_bytes(int B, int H, int T, int D, int n_ckpt_c
     return seg.nseg > 1 ? (int64_t)seg.nseg * B * H * D * 4 : 0;
 }
 
-int adkv_forward_ov_ex(const void *attn, void *v_cache, const void *v_new, void *out,
-                       const void *zp, const void *sc, const void *alpha, const void *beta,
-                       const void *tgt,
-                       int B, int H, int T, int D, int n_super_cap,
-                       void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
-                       void *workspace, int64_t workspace_bytes, void *stream)
+int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void *out,
+                        const void *zp, const void *sc, const void *alpha, const void *beta,
+                        const void *tgt,
+                        int B, int Hq, int H, int T, int D, int n_super_cap,
+                        void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
+                        void *workspace, int64_t workspace_bytes, void *stream)
 {
     if (!attn || !v_cache || !v_new || !out || !zp || !sc || !alpha || !beta || !tgt)
         return ADKV_E_NULL;
     int rc = check_common(B, H, T, D, n_super_cap);
     if (rc)
         return rc;
+    if (Hq <= 0 || Hq % H)
+        return ADKV_E_SHAPE;
+    const int GQ = Hq / H;
+    if (GQ > 1 && D != 128)
+        return ADKV_E_UNSUPPORTED;
     if ((T >> 3) >= n_super_cap)
         return ADKV_E_CAPACITY;
     if (((uintptr_t)v_cache & 15) || ((uintptr_t)out & 3) || ((uintptr_t)v_new & 3))
@@ -1146,23 +1292,43 @@ int adkv_forward_ov_ex(const void *attn, void *v_cache, const void *v_new, void 
     hipStream_t st = (hipStream_t)stream;
     const Seg seg = plan_segments(ckpt, n_ckpt_cap, ckpt_interval, BH, T, D);
     if (seg.nseg > 1) {
-        if (!workspace || workspace_bytes < (int64_t)seg.nseg * BH * D * 4)
+        if (!workspace || workspace_bytes < (int64_t)seg.nseg * BH * GQ * D * 4)
             return ADKV_E_WORKSPACE;
         if ((uintptr_t)workspace & 15)
             return ADKV_E_ALIGN;
     }
-    ADKV_DISPATCH_D(ov_kernel, (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new, (h1 *)out,
-                    (float *)workspace, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,
-                    (const h1 *)beta, (const h1 *)tgt, BH, H, T, n_super_cap, (h1 *)state_out, seg);
+    if (D == 128 && (GQ > 1 || mfma_for_mha())) {
+        ADKV_DISPATCH_GQ(ov_gqa_kernel, (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new,
+                         (h1 *)out, (float *)workspace, (const h1 *)zp, (const h1 *)sc,
+                         (const h1 *)alpha, (const h1 *)beta, (const h1 *)tgt, BH, H, T, n_super_cap,
+                         (h1 *)state_out, seg);
+    } else {
+        ADKV_DISPATCH_D(ov_kernel, (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new, (h1 *)out,
+                        (float *)workspace, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,
+                        (const h1 *)beta, (const h1 *)tgt, BH, H, T, n_super_cap, (h1 *)state_out,
+                        seg);
+    }
     if ((rc = check_launch()))
         return rc;
     if (seg.nseg > 1) {
-        const long n = (long)BH * D;
+        const long n = (long)BH * GQ * D;
         hipLaunchKernelGGL(ov_finalize_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
                            (const float *)workspace, (h1 *)out, n, seg.nseg);
         rc = check_launch();
     }
     return rc;
+}
+
+int adkv_forward_ov_ex(const void *attn, void *v_cache, const void *v_new, void *out,
+                       const void *zp, const void *sc, const void *alpha, const void *beta,
+                       const void *tgt,
+                       int B, int H, int T, int D, int n_super_cap,
+                       void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
+                       void *workspace, int64_t workspace_bytes, void *stream)
+{
+    return adkv_forward_ov_gqa(attn, v_cache, v_new, out, zp, sc, alpha, beta, tgt, B, H, H, T, D,
+                               n_super_cap, state_out, ckpt, n_ckpt_cap, ckpt_interval, workspace,
+                               workspace_bytes, stream);
 }
 
 int adkv_forward_ov(const void *attn, void *v_cache, const void *v_new, void *out,
@@ -1175,61 +1341,105 @@ int adkv_forward_ov(const void *attn, void *v_cache, const void *v_new, void *ou
                               n_super_cap, state_out, nullptr, 0, 0, nullptr, 0, stream);
 }
 
-int adkv_softmax(const void *logits, void *weights, const void *mask,
-                 int rows, int n, int rows_per_mask_row, float scaling, void *stream)
+int64_t adkv_softmax_workspace_bytes(int rows, int n)
+{
+    if (rows <= 0 || n <= SM_CHUNK)
+        return 0;
+    return (int64_t)rows * ((n + SM_CHUNK - 1) / SM_CHUNK) * 8;
+}
+
+int adkv_softmax_ex(const void *logits, void *weights, const void *mask,
+                    int rows, int n, int rows_per_mask_row, float scaling,
+                    void *workspace, int64_t workspace_bytes, void *stream)
 {
     if (!logits || !weights)
         return ADKV_E_NULL;
     if (rows <= 0 || n <= 0 || (mask && rows_per_mask_row <= 0))
         return ADKV_E_SHAPE;
-    hipLaunchKernelGGL(softmax_kernel, dim3((unsigned)rows), dim3(SM_BLOCK), 0, (hipStream_t)stream,
-                       (const h1 *)logits, (h1 *)weights, (const float *)mask, n,
+    const int64_t need = adkv_softmax_workspace_bytes(rows, n);
+    if (need == 0 || !workspace || rows > 65535) {
+        // one workgroup per row; rows that do not fit in its registers are read three times
+        hipLaunchKernelGGL(softmax_kernel, dim3((unsigned)rows), dim3(SM_BLOCK), 0, (hipStream_t)stream,
+                           (const h1 *)logits, (h1 *)weights, (const float *)mask, n,
+                           mask ? rows_per_mask_row : 1, scaling);
+        return check_launch();
+    }
+    if (workspace_bytes < need)
+        return ADKV_E_WORKSPACE;
+    if ((uintptr_t)workspace & 7)
+        return ADKV_E_ALIGN;
+    const int nchunk = (n + SM_CHUNK - 1) / SM_CHUNK;
+    const dim3 grid((unsigned)nchunk, (unsigned)rows);
+    hipLaunchKernelGGL(softmax_part_kernel, grid, dim3(SM_BLOCK), 0, (hipStream_t)stream,
+                       (const h1 *)logits, (const float *)mask, (float2 *)workspace, n, nchunk,
                        mask ? rows_per_mask_row : 1, scaling);
+    hipLaunchKernelGGL(softmax_norm_kernel, grid, dim3(SM_BLOCK), 0, (hipStream_t)stream,
+                       (const h1 *)logits, (h1 *)weights, (const float *)mask,
+                       (const float2 *)workspace, n, nchunk, mask ? rows_per_mask_row : 1, scaling);
     return check_launch();
+}
+
+int adkv_softmax(const void *logits, void *weights, const void *mask,
+                 int rows, int n, int rows_per_mask_row, float scaling, void *stream)
+{
+    return adkv_softmax_ex(logits, weights, mask, rows, n, rows_per_mask_row, scaling, nullptr, 0,
+                           stream);
 }
 
 static int64_t pad256(int64_t n) { return (n + 255) & ~(int64_t)255; }
 
-int64_t adkv_decode_fused_workspace_bytes(int B, int H, int T, int D, int n_ckpt_cap, int ckpt_interval)
+int64_t adkv_forward_ov_gqa_workspace_bytes(int B, int Hq, int H, int T, int D, int n_ckpt_cap,
+                                            int ckpt_interval)
 {
-    if (B <= 0 || H <= 0 || T < 0)
+    if (H <= 0 || Hq <= 0 || Hq % H)
         return 0;
-    const int64_t row = pad256((int64_t)B * H * (T + 1) * 2);
-    return 2 * row + adkv_forward_ov_workspace_bytes(B, H, T, D, n_ckpt_cap, ckpt_interval);
+    return adkv_forward_ov_workspace_bytes(B, H, T, D, n_ckpt_cap, ckpt_interval) * (Hq / H);
+}
+
+int64_t adkv_decode_fused_workspace_bytes(int B, int Hq, int H, int T, int D, int n_ckpt_cap,
+                                          int ckpt_interval)
+{
+    if (B <= 0 || H <= 0 || Hq <= 0 || T < 0)
+        return 0;
+    const int64_t row = pad256((int64_t)B * Hq * (T + 1) * 2);
+    return 2 * row + pad256(adkv_softmax_workspace_bytes(B * Hq, T + 1)) +
+           adkv_forward_ov_gqa_workspace_bytes(B, Hq, H, T, D, n_ckpt_cap, ckpt_interval);
 }
 
 int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k_new, const void *v_new,
                       const void *const *k_params, const void *const *v_params,
                       const void *mask, int rows_per_mask_row, float scaling,
                       void *out, void *weights_out,
-                      int B, int H, int T, int D, int n_super_cap,
+                      int B, int Hq, int H, int T, int D, int n_super_cap,
                       void *k_ckpt, void *v_ckpt, int n_ckpt_cap, int ckpt_interval,
                       void *workspace, int64_t workspace_bytes, void *stream)
 {
     if (!k_params || !v_params || !workspace)
         return workspace ? ADKV_E_NULL : ADKV_E_WORKSPACE;
-    if (B <= 0 || H <= 0 || T < 0)
+    if (B <= 0 || H <= 0 || Hq <= 0 || Hq % H || T < 0)
         return ADKV_E_SHAPE;
-    if (workspace_bytes < adkv_decode_fused_workspace_bytes(B, H, T, D, n_ckpt_cap, ckpt_interval))
+    if (workspace_bytes < adkv_decode_fused_workspace_bytes(B, Hq, H, T, D, n_ckpt_cap, ckpt_interval))
         return ADKV_E_WORKSPACE;
     if ((uintptr_t)workspace & 255)
         return ADKV_E_ALIGN;
-    const int64_t row = pad256((int64_t)B * H * (T + 1) * 2);
+    const int64_t row = pad256((int64_t)B * Hq * (T + 1) * 2);
     char *ws = (char *)workspace;
     void *logits = ws;
     void *weights = weights_out ? weights_out : (void *)(ws + row);
-    int rc = adkv_forward_qk_ex(q, k_cache, k_new, logits, k_params[0], k_params[1], k_params[2],
-                                k_params[3], k_params[4], B, H, T, D, n_super_cap, nullptr,
-                                k_ckpt, n_ckpt_cap, ckpt_interval, stream);
+    int rc = adkv_forward_qk_gqa(q, k_cache, k_new, logits, k_params[0], k_params[1], k_params[2],
+                                 k_params[3], k_params[4], B, Hq, H, T, D, n_super_cap, nullptr,
+                                 k_ckpt, n_ckpt_cap, ckpt_interval, stream);
     if (rc)
         return rc;
-    rc = adkv_softmax(logits, weights, mask, B * H, T + 1, rows_per_mask_row, scaling, stream);
+    const int64_t smb = pad256(adkv_softmax_workspace_bytes(B * Hq, T + 1));
+    rc = adkv_softmax_ex(logits, weights, mask, B * Hq, T + 1, rows_per_mask_row, scaling,
+                         smb ? ws + 2 * row : nullptr, smb, stream);
     if (rc)
         return rc;
-    return adkv_forward_ov_ex(weights, v_cache, v_new, out, v_params[0], v_params[1], v_params[2],
-                              v_params[3], v_params[4], B, H, T, D, n_super_cap, nullptr,
-                              v_ckpt, n_ckpt_cap, ckpt_interval, ws + 2 * row,
-                              workspace_bytes - 2 * row, stream);
+    return adkv_forward_ov_gqa(weights, v_cache, v_new, out, v_params[0], v_params[1], v_params[2],
+                               v_params[3], v_params[4], B, Hq, H, T, D, n_super_cap, nullptr,
+                               v_ckpt, n_ckpt_cap, ckpt_interval, ws + 2 * row + smb,
+                               workspace_bytes - 2 * row - smb, stream);
 }
 
 } // extern "C"

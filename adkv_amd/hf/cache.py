@@ -190,8 +190,10 @@ class KVCacheLayer_ADKV:
         H, Tk = key_states.shape[1], key_states.shape[2]
         if Tq != 1 or Tk != 1:
             raise ValueError("decode expects exactly one query/key/value token")
-        if Hq != H:
-            raise ValueError("ADKV decode supports MHA (num_attention_heads == num_key_value_heads)")
+        if Hq % H or Hq // H not in (1, 2, 4, 8) or (Hq != H and C != 128):
+            # the reference only takes Hq == H (llama_adkv.py:235-238); grouped queries are an extension
+            raise ValueError("ADKV decode supports 1, 2, 4 or 8 query heads per KV head "
+                             "(more than one only with head_dim 128)")
         self._check_geometry(B, H, C, query_states.device)
         ctx = self._quant_len
         self._cap_buffers(ctx + 1)
@@ -201,7 +203,7 @@ class KVCacheLayer_ADKV:
         S = self._ckpt_interval
         dev = query_states.device
         ncap = self._key_ckpt.shape[2] if S else 0
-        ws = _workspace(dev, decode_fused_workspace_bytes(B, H, ctx, C, ncap, S))
+        ws = _workspace(dev, decode_fused_workspace_bytes(B, Hq, H, ctx, C, ncap, S))
         out, weights = decode_fused(
             f16(query_states), self._key_buf, self._value_buf, f16(key_states), f16(value_states),
             (v(key_zp_init), v(key_scale_init), v(key_alpha), v(key_beta), v(key_quant_target)),

@@ -18,6 +18,7 @@ from .. import _lib
 
 _TILE = 4
 _DIMS = (128, 256, 512)
+_GROUPS = (1, 2, 4, 8)   # query heads per KV head
 
 
 def _chk(cond: bool, msg: str) -> None:
@@ -104,12 +105,15 @@ def forward_qk(
     _chk(k_new.dtype == torch.float16, "k_new must be float16")
     _chk(k_cache.dtype == torch.uint8, "k_cache must be uint8")
     _chk(k_cache.is_contiguous(), "k_cache must be contiguous (appended in place)")
-    B, nh = q.shape[0], q.shape[1]
+    B, nq = q.shape[0], q.shape[1]
+    nh = k_cache.shape[1]          # KV heads; nq is a multiple of it under grouped-query attention
     n_super_cap, n_cgroup = k_cache.shape[2], k_cache.shape[3]
     DIM = n_cgroup * _TILE
     zp, sc, al, be, tg = _params((k_zp, k_sc, k_alpha, k_beta, k_t),
                                  ("k_zp", "k_sc", "k_alpha", "k_beta", "k_t"), nh, DIM)
     _chk(DIM == q.shape[3], "q head dimension does not match k_cache")
+    _chk(nq % nh == 0 and nq // nh in _GROUPS, "query heads must be 1, 2, 4 or 8 times the KV heads")
+    _chk(nq == nh or DIM == 128, "grouped-query attention needs DIM == 128")
     _chk(T >= 0, "T must be non-negative")
     _chk((T >> 1) // _TILE < n_super_cap, f"k_cache has no free supergroup to append token {T}")
     _chk(DIM in _DIMS, "DIM must be 128, 256 or 512")
@@ -117,19 +121,19 @@ def forward_qk(
 
     q_flat = q.contiguous()
     k_new_flat = k_new.reshape(B * nh, DIM).contiguous()
-    o = torch.empty((B * nh, T + 1), dtype=torch.float16, device=dev)
+    o = torch.empty((B * nq, T + 1), dtype=torch.float16, device=dev)
     if state_out is not None:
         _chk(state_out.dtype == torch.float16 and state_out.is_contiguous()
              and state_out.numel() == B * nh * DIM * 2, "state_out must be contiguous fp16 [B,nh,DIM,2]")
     cp, ccap, civ = _ckpt_args(ckpt, ckpt_interval, B, nh, DIM)
     with torch.cuda.device(dev):
-        rc = _lib.lib().adkv_forward_qk_ex(
+        rc = _lib.lib().adkv_forward_qk_gqa(
             q_flat.data_ptr(), k_cache.data_ptr(), k_new_flat.data_ptr(), o.data_ptr(),
             zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
-            B, nh, T, DIM, n_super_cap, _ptr(state_out), cp, ccap, civ,
+            B, nq, nh, T, DIM, n_super_cap, _ptr(state_out), cp, ccap, civ,
             _lib.current_stream_ptr(dev))
     _lib.check(rc, "forward_qk")
-    return o.reshape(B, nh, T + 1)
+    return o.reshape(B, nq, T + 1)
 
 
 def forward_ov(
@@ -160,7 +164,8 @@ def forward_ov(
     _chk(v_new.dtype == torch.float16, "v_new must be float16")
     _chk(v_cache.dtype == torch.uint8, "v_cache must be uint8")
     _chk(v_cache.is_contiguous(), "v_cache must be contiguous (appended in place)")
-    B, nh = attn.shape[0], attn.shape[1]
+    B, nq = attn.shape[0], attn.shape[1]
+    nh = v_cache.shape[1]
     _chk(attn.shape[2] >= 1, "attn must contain the cached weights plus the self weight")
     T = attn.shape[2] - 1
     n_super_cap, n_cgroup = v_cache.shape[2], v_cache.shape[3]
@@ -168,6 +173,8 @@ def forward_ov(
     zp, sc, al, be, tg = _params((v_zp, v_sc, v_alpha, v_beta, v_t),
                                  ("v_zp", "v_sc", "v_alpha", "v_beta", "v_t"), nh, DIM)
     _chk(DIM == v_new.shape[-1], "v_new head dimension does not match v_cache")
+    _chk(nq % nh == 0 and nq // nh in _GROUPS, "query heads must be 1, 2, 4 or 8 times the KV heads")
+    _chk(nq == nh or DIM == 128, "grouped-query attention needs DIM == 128")
     _chk(T >= 0, "T must be non-negative")
     _chk((T >> 1) // _TILE < n_super_cap, f"v_cache has no free supergroup to append token {T}")
     _chk(DIM in _DIMS, "DIM must be 128, 256 or 512")
@@ -175,7 +182,7 @@ def forward_ov(
 
     attn_flat = attn.contiguous()
     v_new_flat = v_new.reshape(B * nh, DIM).contiguous()
-    o = torch.empty((B * nh, DIM), dtype=torch.float16, device=dev)
+    o = torch.empty((B * nq, DIM), dtype=torch.float16, device=dev)
     if state_out is not None:
         _chk(state_out.dtype == torch.float16 and state_out.is_contiguous()
              and state_out.numel() == B * nh * DIM * 2, "state_out must be contiguous fp16 [B,nh,DIM,2]")
@@ -183,14 +190,14 @@ def forward_ov(
     L = _lib.lib()
     ws, ws_bytes = None, 0
     if cp is not None:
-        ws_bytes = L.adkv_forward_ov_workspace_bytes(B, nh, T, DIM, ccap, civ)
+        ws_bytes = L.adkv_forward_ov_gqa_workspace_bytes(B, nq, nh, T, DIM, ccap, civ)
         if ws_bytes:
             ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dev)
     with torch.cuda.device(dev):
-        rc = L.adkv_forward_ov_ex(
+        rc = L.adkv_forward_ov_gqa(
             attn_flat.data_ptr(), v_cache.data_ptr(), v_new_flat.data_ptr(), o.data_ptr(),
             zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
-            B, nh, T, DIM, n_super_cap, _ptr(state_out), cp, ccap, civ,
+            B, nq, nh, T, DIM, n_super_cap, _ptr(state_out), cp, ccap, civ,
             _ptr(ws), ws_bytes, _lib.current_stream_ptr(dev))
     _lib.check(rc, "forward_ov")
     return o.view(attn.shape[0], attn.shape[1], -1)
@@ -322,9 +329,12 @@ def softmax_scale_mask(logits: torch.Tensor, scaling: float,
         rpm = nh if mk.shape[1] == 1 else 1
         mk = mk.to(device=dev, dtype=torch.float32).contiguous()
         mptr = mk.data_ptr()
+    L = _lib.lib()
+    wsb = L.adkv_softmax_workspace_bytes(B * nh, n)
+    ws = torch.empty(wsb, dtype=torch.uint8, device=dev) if wsb else None
     with torch.cuda.device(dev):
-        rc = _lib.lib().adkv_softmax(lg.data_ptr(), out.data_ptr(), mptr, B * nh, n, rpm,
-                                     float(scaling), _lib.current_stream_ptr(dev))
+        rc = L.adkv_softmax_ex(lg.data_ptr(), out.data_ptr(), mptr, B * nh, n, rpm, float(scaling),
+                               _ptr(ws), wsb, _lib.current_stream_ptr(dev))
     _lib.check(rc, "softmax_scale_mask")
     return out
 
@@ -361,8 +371,10 @@ def decode_fused(
         _chk(t.dtype == torch.uint8, f"{n} must be uint8")
         _chk(t.is_contiguous(), f"{n} must be contiguous (appended in place)")
     _chk(k_cache.shape == v_cache.shape, "k_cache and v_cache shapes differ")
-    B, nh = q.shape[0], q.shape[1]
+    B, nq, nh = q.shape[0], q.shape[1], k_cache.shape[1]
     n_super_cap, DIM = k_cache.shape[2], k_cache.shape[3] * _TILE
+    _chk(nq % nh == 0 and nq // nh in _GROUPS, "query heads must be 1, 2, 4 or 8 times the KV heads")
+    _chk(nq == nh or DIM == 128, "grouped-query attention needs DIM == 128")
     kp = _params(k_params, ("k_zp", "k_sc", "k_alpha", "k_beta", "k_t"), nh, DIM)
     vp = _params(v_params, ("v_zp", "v_sc", "v_alpha", "v_beta", "v_t"), nh, DIM)
     _chk(DIM == q.shape[-1], "q head dimension does not match k_cache")
@@ -374,9 +386,9 @@ def decode_fused(
     rpm, mptr, mk = 1, None, None
     if mask is not None:
         mk = mask[:, :, 0, :] if mask.dim() == 4 else mask
-        _chk(mk.dim() == 3 and mk.shape[0] == B and mk.shape[2] == n and mk.shape[1] in (1, nh),
+        _chk(mk.dim() == 3 and mk.shape[0] == B and mk.shape[2] == n and mk.shape[1] in (1, nq),
              "mask must broadcast to [B, nh, n]")
-        rpm = nh if mk.shape[1] == 1 else 1
+        rpm = nq if mk.shape[1] == 1 else 1
         mk = mk.to(device=dev, dtype=torch.float32).contiguous()
         mptr = mk.data_ptr()
     kcp, ccap, civ = _ckpt_args(k_ckpt, ckpt_interval, B, nh, DIM)
@@ -384,7 +396,7 @@ def decode_fused(
     _chk((k_ckpt is None) == (v_ckpt is None) and ccap == vcap,
          "k_ckpt and v_ckpt must both be given, with the same capacity, or both omitted")
     L = _lib.lib()
-    need = L.adkv_decode_fused_workspace_bytes(B, nh, T, DIM, ccap, civ)
+    need = L.adkv_decode_fused_workspace_bytes(B, nq, nh, T, DIM, ccap, civ)
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     _chk(workspace.dtype == torch.uint8 and workspace.is_cuda and workspace.numel() >= need,
@@ -392,20 +404,22 @@ def decode_fused(
     qf = q.contiguous()
     knf = k_new.reshape(B * nh, DIM).contiguous()
     vnf = v_new.reshape(B * nh, DIM).contiguous()
-    out = torch.empty((B, nh, DIM), dtype=torch.float16, device=dev)
-    weights = torch.empty((B, nh, n), dtype=torch.float16, device=dev)
+    out = torch.empty((B, nq, DIM), dtype=torch.float16, device=dev)
+    weights = torch.empty((B, nq, n), dtype=torch.float16, device=dev)
     arr = _lib.C.c_void_p * 5
     with torch.cuda.device(dev):
         rc = L.adkv_decode_fused(
             qf.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), knf.data_ptr(), vnf.data_ptr(),
             arr(*[t.data_ptr() for t in kp]), arr(*[t.data_ptr() for t in vp]),
             mptr, rpm, float(scaling), out.data_ptr(), weights.data_ptr(),
-            B, nh, T, DIM, n_super_cap, kcp, vcp, ccap, civ,
+            B, nq, nh, T, DIM, n_super_cap, kcp, vcp, ccap, civ,
             workspace.data_ptr(), workspace.numel(), _lib.current_stream_ptr(dev))
     _lib.check(rc, "decode_fused")
     return out, weights
 
 
-def decode_fused_workspace_bytes(B: int, nh: int, T: int, DIM: int, n_ckpt_cap: int = 0,
+def decode_fused_workspace_bytes(B: int, nq: int, nh: int, T: int, DIM: int, n_ckpt_cap: int = 0,
                                  ckpt_interval: int = 0) -> int:
-    return int(_lib.lib().adkv_decode_fused_workspace_bytes(B, nh, T, DIM, n_ckpt_cap, ckpt_interval))
+    """Bytes ``decode_fused`` needs for ``nq`` query heads over ``nh`` KV heads."""
+    return int(_lib.lib().adkv_decode_fused_workspace_bytes(B, nq, nh, T, DIM, n_ckpt_cap,
+                                                            ckpt_interval))

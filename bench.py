@@ -39,6 +39,9 @@ def parse():
                          "B=8 ctx=32768 prefill, then 256 single-token appends)")
     ap.add_argument("--batch", type=int, default=128)
     ap.add_argument("--heads", type=int, default=32)
+    ap.add_argument("--kv-heads", type=int, default=0,
+                    help="KV heads when fewer than --heads query heads share them (grouped-query "
+                         "attention); default: as many as --heads")
     ap.add_argument("--dim", type=int, default=128)
     ap.add_argument("--ctx", type=int, default=4096)
     ap.add_argument("--layer-buffers", type=int, default=4,
@@ -184,7 +187,7 @@ def encode_main(args):
         "data": "synthetic",
         "config": {"workload": f"cfg3 streaming quantise: prefill B={B} H={H} d={D} ctx={T} fp16 -> 4-bit codes, "
                                f"then {n_app} single-token appends with carried state",
-                   "batch": B, "heads": H, "head_dim": D, "ctx": T, "bits": 4, "ckpt_interval": S},
+                   "batch": B, "heads": Hq, "kv_heads": H, "head_dim": D, "ctx": T, "bits": 4, "ckpt_interval": S},
         "append_us_per_token_step": append_us,
         "codes_bit_exact_vs_oracle": exact,
         "roofline": {"kernel": "encode_kernel", "bound": "hbm", "achieved": achieved,
@@ -220,7 +223,8 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    B, H, D, T = args.batch, args.heads, args.dim, args.ctx
+    B, Hq, D, T = args.batch, args.heads, args.dim, args.ctx
+    H = args.kv_heads or Hq          # KV heads own the caches and parameters
     smin, smax = math.exp(-4.0), math.exp(4.0)
     NL = args.layer_buffers
 
@@ -242,7 +246,7 @@ def main():
         del x
         kps.append(kp.astuple()); vps.append(vp.astuple()); kcs.append(kc); vcs.append(vc)
         kks.append(kk); vks.append(vk)
-    q = synth.make_q(B, H, D, device=dev)
+    q = synth.make_q(B, Hq, D, device=dev)
     k_new = synth.make_k(B, H, 1, D, seed=11, dtype=torch.float16, device=dev, t0=T)
     v_new = synth.make_v(B, H, 1, D, seed=12, dtype=torch.float16, device=dev)
     scaling = D ** -0.5
@@ -310,10 +314,11 @@ def main():
         "dtype": "f16",
         "data": "synthetic",
         "config": {
-            "workload": f"cfg2 Llama-2-7B-shaped ADKV decode attention: B={B} H={H} d={D} ctx={T} "
+            "workload": f"{'cfg2 Llama-2-7B-shaped' if H == Hq else 'grouped-query'} ADKV decode attention: "
+                        f"B={B} H={Hq}{'' if H == Hq else f' (KV heads {H})'} d={D} ctx={T} "
                         f"4-bit K+V codes, step = forward_qk+softmax+forward_ov, {NL} rotating layer caches, "
                         f"state checkpoints every {S} tokens",
-            "batch": B, "heads": H, "head_dim": D, "ctx": T, "bits": 4, "ckpt_interval": S,
+            "batch": B, "heads": Hq, "kv_heads": H, "head_dim": D, "ctx": T, "bits": 4, "ckpt_interval": S,
             "parallelism": "1 GPU",
         },
         "kernel_ms": {"forward_qk": qk_ms, "softmax": sm_ms, "forward_ov": ov_ms,
@@ -331,9 +336,9 @@ def main():
             "traffic": 1.1227e9 if (B, H, D, T, S) == (128, 32, 128, 4096, 256) else None,
         },
     }
-    if not args.no_fp16_comparator and D == 128:
+    if not args.no_fp16_comparator and D == 128 and H == Hq:
         res["fp16_kv_comparator"] = fp16_comparator(args, dev, ms_step)
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and H == Hq:
         res["cpu_baseline"] = cpu_baseline(args, T, D)
     print(json.dumps(res))
 

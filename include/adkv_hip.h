@@ -32,6 +32,12 @@ extern "C" {
 
 /* ABI version of this header; bumped on any signature change. */
 int adkv_abi_version(void);
+
+/* Tuning knob, no counterpart in the reference: which decode kernels a launch with as many query
+ * heads as KV heads and head dim 128 uses: 1 = the matrix-core kernels (the ones grouped-query
+ * launches always use), 0 = the vector kernels, -1 = the library's default (ADKV_MFMA in the
+ * environment overrides it).  Results agree to the tolerance of the fp32 accumulation order. */
+void adkv_set_mha_kernel(int use_matrix_cores);
 const char *adkv_strerror(int code);
 /* hipError_t (as int) of the last failed launch in this thread, 0 if none. */
 int adkv_last_hip_error(void);
@@ -84,6 +90,14 @@ int adkv_forward_ov(const void *attn, void *v_cache, const void *v_new, void *ou
  */
 int adkv_softmax(const void *logits, void *weights, const void *mask,
                  int rows, int n, int rows_per_mask_row, float scaling, void *stream);
+
+/* The same with a workspace of adkv_softmax_workspace_bytes(rows, n) bytes (0 for short rows):
+ * long rows (contexts of tens of thousands of tokens) are then cut into chunks that many
+ * workgroups process, instead of one workgroup walking the row three times. */
+int64_t adkv_softmax_workspace_bytes(int rows, int n);
+int adkv_softmax_ex(const void *logits, void *weights, const void *mask,
+                    int rows, int n, int rows_per_mask_row, float scaling,
+                    void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
  * ---- Extensions with state checkpoints (no counterpart in the reference's code; its paper sketches
@@ -138,22 +152,46 @@ int adkv_forward_ov_ex(const void *attn, void *v_cache, const void *v_new, void 
                        void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
+ * Grouped-query attention: Hq query heads share H KV heads (Hq % H == 0; query head j reads KV
+ * head j / (Hq/H)).  The reference refuses this (src/adkv/hf/llama_adkv.py:235-238 requires
+ * num_attention_heads == num_key_value_heads); here the state replay runs once per KV head and
+ * the contraction with all of its query heads goes to the matrix cores.  Head dim 128 only when
+ * Hq > H.  q: [B, Hq, D]; logits / attn: [B, Hq, T+1]; out: [B, Hq, D]; everything else as in the
+ * _ex entry points.  The OV workspace is adkv_forward_ov_gqa_workspace_bytes(...) bytes.
+ */
+int adkv_forward_qk_gqa(const void *q, void *k_cache, const void *k_new, void *logits,
+                        const void *zp, const void *sc, const void *alpha, const void *beta,
+                        const void *tgt,
+                        int B, int Hq, int H, int T, int D, int n_super_cap,
+                        void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
+                        void *stream);
+int64_t adkv_forward_ov_gqa_workspace_bytes(int B, int Hq, int H, int T, int D, int n_ckpt_cap,
+                                            int ckpt_interval);
+int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void *out,
+                        const void *zp, const void *sc, const void *alpha, const void *beta,
+                        const void *tgt,
+                        int B, int Hq, int H, int T, int D, int n_super_cap,
+                        void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
+                        void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
  * One decode-attention step of one layer in a single call: forward_qk -> scale/mask/softmax ->
  * forward_ov, appending k_new / v_new at slot T of both caches.  Replaces the body of
  * KVCacheLayer_ADKV.decode (src/adkv/hf/llama_adkv.py:245-276).
+ * q: fp16 [B, Hq, D] with Hq a multiple of the H KV heads (Hq == H is the reference's case).
  * k_params / v_params: host arrays of five device pointers {zp, sc, alpha, beta, tgt}, each
- * fp16 [H, D].  mask: optional fp32 additive mask as in adkv_softmax.  out: fp16 [B, H, D].
- * weights_out: optional fp16 [B, H, T+1] (the attention weights the reference returns); when
+ * fp16 [H, D].  mask: optional fp32 additive mask as in adkv_softmax.  out: fp16 [B, Hq, D].
+ * weights_out: optional fp16 [B, Hq, T+1] (the attention weights the reference returns); when
  * NULL they live in the workspace.  Checkpoint tensors as in the _ex entry points (NULL = none).
  * workspace: >= adkv_decode_fused_workspace_bytes(...) bytes, 256-byte aligned.
  */
-int64_t adkv_decode_fused_workspace_bytes(int B, int H, int T, int D, int n_ckpt_cap,
+int64_t adkv_decode_fused_workspace_bytes(int B, int Hq, int H, int T, int D, int n_ckpt_cap,
                                           int ckpt_interval);
 int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k_new,
                       const void *v_new, const void *const *k_params, const void *const *v_params,
                       const void *mask, int rows_per_mask_row, float scaling,
                       void *out, void *weights_out,
-                      int B, int H, int T, int D, int n_super_cap,
+                      int B, int Hq, int H, int T, int D, int n_super_cap,
                       void *k_ckpt, void *v_ckpt, int n_ckpt_cap, int ckpt_interval,
                       void *workspace, int64_t workspace_bytes, void *stream);
 

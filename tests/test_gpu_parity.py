@@ -106,7 +106,8 @@ def test_forward_qk_and_ov(gpu, oracle, B, H, T, D):
     assert np.all(np.abs(goto - o_want) <= _ulp16(o_want) + 1e-3)
 
 
-@pytest.mark.parametrize("rows,n,mask_mode", [(6, 1, None), (6, 130, None), (8, 4097, "b1"), (8, 257, "bh")])
+@pytest.mark.parametrize("rows,n,mask_mode", [(6, 1, None), (6, 130, None), (8, 4097, "b1"), (8, 257, "bh"),
+                                              (4, 5121, None), (6, 20000, "b1"), (2, 131073, "bh")])
 def test_softmax(gpu, rows, n, mask_mode):
     g = torch.Generator().manual_seed(n)
     B, H = 2, rows // 2
@@ -416,3 +417,72 @@ def test_decode_fused_equals_three_calls(gpu, B, H, T, D, S, masked):
     if S:
         assert torch.equal(kk.view(torch.int16), kk2.view(torch.int16))
         assert torch.equal(vk.view(torch.int16), vk2.view(torch.int16))
+
+
+# ------------------------------------------------------------------ grouped-query / matrix-core kernels
+def _gqa_case(gpu, oracle, B, Hkv, G, T, S, seed=0):
+    """One QK + OV pass with G query heads per KV head against the oracle run once per group member
+    on a copy of the same cache (query head j reads KV head j // G)."""
+    D = 128
+    Hq = Hkv * G
+    x, p = _inputs(B, Hkv, T + 1, D, seed=seed)
+    pn = [_np16(t) for t in p.astuple()]
+    pg = [t.to(gpu) for t in p.astuple()]
+    g = torch.Generator().manual_seed(50 + seed)
+    q = torch.randn(B, Hq, 1, D, generator=g).half()
+    attn = torch.softmax(2.0 * torch.randn(B, Hq, T + 1, generator=g), dim=-1).half()
+    cache0 = oracle.alloc_cache(B, Hkv, T + 8, D)
+    if T:
+        oracle.encode_kv_f16(cache0, _np16(x)[:, :, :T], *pn)
+    ncap = (T + 8) // S + 1 if S else 0
+    ck = None
+    if S:
+        ck = torch.from_numpy(_oracle_ckpts(oracle, cache0, pn, T, S, ncap).view(np.int16)).view(torch.float16).to(gpu)
+    xn = _np16(x)[:, :, T:T + 1]
+    want_l = np.zeros((B, Hq, T + 1))
+    want_o = np.zeros((B, Hq, D))
+    qn, an = _np16(q).reshape(B, Hkv, G, D), _np16(attn).reshape(B, Hkv, G, T + 1)
+    for j in range(G):
+        c = cache0.copy()
+        l, _ = oracle.forward_qk_f16(qn[:, :, j], c, xn, *pn, T)
+        want_l.reshape(B, Hkv, G, T + 1)[:, :, j] = l
+        c2 = cache0.copy()
+        o, _ = oracle.forward_ov_f16(an[:, :, j], c2, xn, *pn)
+        want_o.reshape(B, Hkv, G, D)[:, :, j] = o
+    kc = torch.from_numpy(cache0.copy()).to(gpu)
+    vc = torch.from_numpy(cache0.copy()).to(gpu)
+    ckv = ck.clone() if ck is not None else None
+    st_k = torch.zeros(B, Hkv, D, 2, dtype=torch.float16, device=gpu)
+    logits = gemv.forward_qk(q.to(gpu), kc, x[:, :, T:T + 1].to(gpu), *pg, T, SMIN, SMAX,
+                             state_out=st_k, ckpt=ck, ckpt_interval=S)
+    out = gemv.forward_ov(attn.to(gpu), vc, x[:, :, T:T + 1].to(gpu), *pg, SMIN, SMAX,
+                          ckpt=ckv, ckpt_interval=S)
+    torch.cuda.synchronize()
+    assert logits.shape == (B, Hq, T + 1) and out.shape == (B, Hq, D)
+    assert np.array_equal(kc.cpu().numpy(), c) and np.array_equal(vc.cpu().numpy(), c2)
+    _, st_want = oracle.replay_f16(cache0, *pn, T, want_khat=False)
+    assert np.array_equal(st_k.cpu().view(torch.int16).numpy().view(np.uint16), st_want)
+    lg, og = _np16(logits).astype(np.float64), _np16(out).astype(np.float64)
+    assert np.all(np.abs(lg - want_l) <= _ulp16(want_l) + 1e-3), np.abs(lg - want_l).max()
+    assert np.all(np.abs(og - want_o) <= _ulp16(want_o) + 1e-3), np.abs(og - want_o).max()
+    if S:
+        assert torch.equal(ck.view(torch.int16), ckv.view(torch.int16))
+
+
+@pytest.mark.parametrize("B,Hkv,G,T,S", [
+    (1, 2, 4, 0, 0), (2, 2, 4, 5, 0), (1, 3, 2, 8, 0), (2, 2, 4, 71, 0), (1, 2, 8, 40, 0),
+    (2, 3, 4, 530, 64), (1, 2, 2, 256, 64), (1, 1, 8, 200, 16), (1, 5, 4, 1025, 0)])
+def test_grouped_query_kernels(gpu, oracle, B, Hkv, G, T, S):
+    _gqa_case(gpu, oracle, B, Hkv, G, T, S, seed=T % 7)
+
+
+@pytest.mark.parametrize("B,H,T,S", [(2, 3, 0, 0), (1, 2, 7, 0), (2, 2, 130, 0), (2, 3, 530, 64)])
+def test_matrix_core_kernels_for_equal_heads(gpu, oracle, B, H, T, S):
+    """The same matrix-core kernels with one query head per KV head (selected by the tuning knob)
+    meet the bar of the vector kernels."""
+    from adkv_amd import _lib
+    _lib.lib().adkv_set_mha_kernel(1)
+    try:
+        _gqa_case(gpu, oracle, B, H, 1, T, S, seed=3)
+    finally:
+        _lib.lib().adkv_set_mha_kernel(-1)

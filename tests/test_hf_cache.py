@@ -55,8 +55,8 @@ def test_cache_errors_cpu():
     q = torch.zeros(1, 2, 1, 128)
     with pytest.raises(ValueError, match="exactly one query/key/value token"):
         c.decode(torch.zeros(1, 2, 2, 128), q, q, *kp, *kp)
-    with pytest.raises(ValueError, match="supports MHA"):
-        c.decode(torch.zeros(1, 4, 1, 128), q, q, *kp, *kp)
+    with pytest.raises(ValueError, match="query heads per KV head"):
+        c.decode(torch.zeros(1, 6, 1, 128), q, q, *kp, *kp)     # 3 query heads per KV head
     c._quant_len, c._state_valid = 3, False      # as after decode steps: the carried state is gone
     with pytest.raises(NotImplementedError, match="chunked prefill is not supported"):
         c.prefill(torch.zeros(1, 2, 4, 128), torch.zeros(1, 2, 4, 128), *kp, *kp)
