@@ -211,8 +211,28 @@ static inline uint16_t int_to_h(int q) { return adkv_o_d2h((double)q); }
 /* semantics B scalar steps                                                                     */
 /* ------------------------------------------------------------------------------------------ */
 
+/* Code width of the semantics-B functions below.  4 is the reference's deployment format
+ * (gemv.cu throughout).  2 is this build's extension of the same recurrence to the code range
+ * [-2, 1] (QL/QU as train_model.py:96-97 define them for bits=2) with 16 tokens per 32-bit word;
+ * the reference has no fp16 kernel for it, so nothing there pins it. */
+static int g_bits = 4;
+
+int adkv_o_set_bits(int bits)
+{
+    if (bits != 2 && bits != 4)
+        return -1;
+    g_bits = bits;
+    return 0;
+}
+
+int adkv_o_get_bits(void) { return g_bits; }
+
+static inline int q_lo(void) { return -(1 << (g_bits - 1)); }
+static inline int q_hi(void) { return (1 << (g_bits - 1)) - 1; }
+static inline int tokens_per_word(void) { return 32 / g_bits; }
+
 /* gemv.cu:150-154: fp32 subtract, IEEE fp32 divide, round-half-even to int (NaN -> 0,
- * out-of-range saturates, as __float2int_rn), clamp to [-8, 7]. */
+ * out-of-range saturates, as __float2int_rn), clamp to [-8, 7] ([-2, 1] for 2-bit codes). */
 int adkv_o_quantize_f16(uint16_t x, uint16_t zp, uint16_t sc)
 {
     volatile float d = adkv_o_h2f(x) - adkv_o_h2f(zp);
@@ -220,10 +240,10 @@ int adkv_o_quantize_f16(uint16_t x, uint16_t zp, uint16_t sc)
     if (u != u)
         return 0;
     float r = nearbyintf(u); /* default rounding mode: to nearest even */
-    if (r < -8.0f)
-        return -8;
-    if (r > 7.0f)
-        return 7;
+    if (r < (float)q_lo())
+        return q_lo();
+    if (r > (float)q_hi())
+        return q_hi();
     return (int)r;
 }
 
@@ -262,28 +282,30 @@ uint16_t adkv_o_dequant1_f16(int q, uint16_t zp, uint16_t sc)
 /* ------------------------------------------------------------------------------------------ */
 
 /* [n_super, D/4, 4 (channel in group), 4 (byte row)] ; byte row br holds tokens 8sg+2br (low
- * nibble) and 8sg+2br+1 (high nibble).  gemv.cu:502-510, 91-146, 243-305. */
+ * nibble) and 8sg+2br+1 (high nibble).  gemv.cu:502-510, 91-146, 243-305.
+ * 2-bit codes: a supergroup is 16 tokens, byte row br holds tokens 16sg+4br .. +3, token i of the
+ * byte at bits 2i..2i+1; code = q + 2. */
 int64_t adkv_o_byte_offset(int t, int c, int D)
 {
-    int sg = t / 8, br = (t % 8) / 2;
+    int tpw = tokens_per_word();
+    int sg = t / tpw, br = (t % tpw) / (tpw / 4);
     return (((int64_t)sg * (D / 4) + c / 4) * 4 + c % 4) * 4 + br;
 }
 
 int adkv_o_get_code(const uint8_t *cache_bh, int t, int c, int D)
 {
     uint8_t b = cache_bh[adkv_o_byte_offset(t, c, D)];
-    int n = (t & 1) ? (b >> 4) : (b & 0x0F);
-    return n - 8;
+    int per_byte = 8 / g_bits, sh = (t % per_byte) * g_bits;
+    return ((b >> sh) & ((1 << g_bits) - 1)) + q_lo();
 }
 
 void adkv_o_put_code(uint8_t *cache_bh, int t, int c, int D, int q)
 {
     uint8_t *p = &cache_bh[adkv_o_byte_offset(t, c, D)];
-    uint8_t n = (uint8_t)((q + 8) & 0x0F);
-    if (t & 1)
-        *p = (uint8_t)((*p & 0x0F) | (n << 4));
-    else
-        *p = (uint8_t)((*p & 0xF0) | n);
+    int per_byte = 8 / g_bits, sh = (t % per_byte) * g_bits;
+    uint8_t m = (uint8_t)(((1 << g_bits) - 1) << sh);
+    uint8_t n = (uint8_t)(((q - q_lo()) << sh) & m);
+    *p = (uint8_t)((*p & ~m) | n);
 }
 
 /* ------------------------------------------------------------------------------------------ */
@@ -298,7 +320,7 @@ void adkv_o_encode_kv_f16(uint8_t *cache, const uint16_t *kv_new,
                           int B, int H, int T, int D, int n_super_cap,
                           uint16_t *state_out)
 {
-    int n_super = ((T + 1) / 2 + 3) / 4;
+    int n_super = (T + tokens_per_word() - 1) / tokens_per_word();
     for (int bx = 0; bx < B * H; bx++) {
         int h = bx % H;
         uint8_t *cb = cache + (int64_t)bx * bh_bytes(D, n_super_cap);

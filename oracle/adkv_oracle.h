@@ -32,6 +32,12 @@ uint16_t adkv_o_hadd(uint16_t a, uint16_t b);
 uint16_t adkv_o_hsub(uint16_t a, uint16_t b);
 uint16_t adkv_o_hfma(uint16_t a, uint16_t b, uint16_t c); /* one rounding */
 
+/* Code width used by every semantics-B function below: 4 (the reference's format, default) or 2
+ * (this build's extension: codes in [-2, 1], 16 tokens per word).  Process-wide; returns 0, or
+ * -1 for an unsupported width. */
+int      adkv_o_set_bits(int bits);
+int      adkv_o_get_bits(void);
+
 /* ---- semantics B scalar steps ---- */
 /* gemv.cu:150-154 */
 int      adkv_o_quantize_f16(uint16_t x, uint16_t zp, uint16_t sc);

@@ -86,9 +86,33 @@ def _p(a):
     return None if a is None else a.ctypes.data_as(C.c_void_p)
 
 
+def get_bits() -> int:
+    return lib().adkv_o_get_bits()
+
+
+class code_bits:
+    """``with code_bits(2): ...`` runs the semantics-B functions with 2-bit codes (the default, 4,
+    is the reference's format) and restores the previous width afterwards."""
+
+    def __init__(self, bits: int):
+        self.bits = bits
+
+    def __enter__(self):
+        self.prev = get_bits()
+        if lib().adkv_o_set_bits(self.bits) != 0:
+            raise ValueError(f"unsupported code width {self.bits}")
+        return self
+
+    def __exit__(self, *exc):
+        lib().adkv_o_set_bits(self.prev)
+        return False
+
+
 def n_super(tokens: int) -> int:
-    """Supergroups (8 tokens each) covering ``tokens`` tokens; llama_adkv.py:84-85."""
-    return (tokens + 7) // 8
+    """Supergroups (8 tokens each; 16 with 2-bit codes) covering ``tokens`` tokens;
+    llama_adkv.py:84-85."""
+    tpw = 32 // get_bits()
+    return (tokens + tpw - 1) // tpw
 
 
 def alloc_cache(B: int, H: int, cap_tokens: int, D: int) -> np.ndarray:
@@ -100,11 +124,13 @@ def unpack_codes(cache: np.ndarray, T: int) -> np.ndarray:
     """[B,H,T,D] int8 codes from a packed cache (pure numpy; independent of the C unpacker)."""
     B, H, S, G, _, _ = cache.shape
     D = G * 4
+    bits = get_bits()
+    per_byte, tpw = 8 // bits, 32 // bits
     c = cache.reshape(B, H, S, D, 4)                      # (.., sg, channel, byte_row)
-    lo = (c & 0x0F).astype(np.int8) - 8                   # token 8sg+2br
-    hi = (c >> 4).astype(np.int8) - 8                     # token 8sg+2br+1
-    tok = np.stack([lo, hi], axis=-1).reshape(B, H, S, D, 8)   # (.., sg, channel, t%8)
-    tok = tok.transpose(0, 1, 2, 4, 3).reshape(B, H, S * 8, D)
+    fields = [((c >> (bits * i)) & ((1 << bits) - 1)).astype(np.int8) - (1 << (bits - 1))
+              for i in range(per_byte)]                   # token tpw*sg + per_byte*br + i
+    tok = np.stack(fields, axis=-1).reshape(B, H, S, D, tpw)   # (.., sg, channel, t % tpw)
+    tok = tok.transpose(0, 1, 2, 4, 3).reshape(B, H, S * tpw, D)
     return np.ascontiguousarray(tok[:, :, :T])
 
 
@@ -141,7 +167,7 @@ def forward_qk_f16(q, cache, k_new, zp, sc, alpha, beta, tgt, T, refemu=False):
     B, H, cap, G = cache.shape[:4]
     D = G * 4
     qh, kn = _h(q).reshape(B, H, D), _h(k_new).reshape(B, H, D)
-    assert T // 8 < cap
+    assert T // (32 // get_bits()) < cap
     out = np.zeros((B, H, T + 1), dtype=np.float64)
     emu = np.zeros((B, H, T + 1), dtype=np.uint16) if refemu else None
     ps = [_h(x) for x in (zp, sc, alpha, beta, tgt)]
@@ -157,7 +183,7 @@ def forward_ov_f16(attn, cache, v_new, zp, sc, alpha, beta, tgt, refemu=False):
     a = _h(attn)
     T = a.shape[2] - 1
     vn = _h(v_new).reshape(B, H, D)
-    assert T // 8 < cap
+    assert T // (32 // get_bits()) < cap
     out = np.zeros((B, H, D), dtype=np.float64)
     emu = np.zeros((B, H, D), dtype=np.uint16) if refemu else None
     ps = [_h(x) for x in (zp, sc, alpha, beta, tgt)]
