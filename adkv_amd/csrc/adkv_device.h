@@ -113,42 +113,103 @@ __device__ __forceinline__ void update_pair_abs(Pair &p, h2 qabs, h2 qs)
     p.sc = p.sc * f;
 }
 
+// Code width.  4 bits is the reference's format (8 tokens per 32-bit channel word, codes in
+// [-8, 7], stored as q + 8).  2 bits is the same recurrence over codes in [-2, 1] (the range the
+// reference's train model uses for bits = 2, train_model.py:96-97), stored as q + 2, 16 tokens per
+// word; the reference has no kernel for it.
+template <int BITS>
+struct Code {
+    static_assert(BITS == 2 || BITS == 4, "code width");
+    static constexpr int TPW = 32 / BITS;                 // tokens per channel word = per supergroup
+    static constexpr int QLO = -(1 << (BITS - 1));
+    static constexpr int QHI = (1 << (BITS - 1)) - 1;
+    static constexpr uint32_t FIELD = (1u << BITS) - 1u;
+    static constexpr uint32_t BIAS = BITS == 4 ? 0x88888888u : 0xAAAAAAAAu; // -QLO in every field
+};
+
 // gemv.cu:150-154: fp32 subtract, IEEE fp32 divide, round-half-even, NaN -> 0, clamp to [-8,7].
+template <int BITS = 4>
 __device__ __forceinline__ int quantize(h1 x, h1 zp, h1 sc)
 {
     const float d = (float)x - (float)zp;
     const float u = d / (float)sc;
     float r = __builtin_rintf(u);
     r = (u != u) ? 0.0f : r;
-    r = __builtin_fminf(__builtin_fmaxf(r, -8.0f), 7.0f);
+    r = __builtin_fminf(__builtin_fmaxf(r, (float)Code<BITS>::QLO), (float)Code<BITS>::QHI);
     return (int)r;
 }
 
 // The encoder's form of quantize(): same value, fewer instructions.  x - zp as one fp32 fma with
 // fp16 operands (exactly the rounded fp32 difference), IEEE divide, round-half-even, then the
 // hardware float->int conversion, which saturates and maps NaN to 0 as CUDA's __float2int_rn does.
+template <int BITS = 4>
 __device__ __forceinline__ int quantize_enc(h1 x, h1 zp, h1 sc)
 {
     const float d = __builtin_fmaf((float)x, 1.0f, -(float)zp);
     const float r = __builtin_rintf(d / (float)sc);
     int q;
     asm("v_cvt_i32_f32 %0, %1" : "=v"(q) : "v"(r));
-    return q < -8 ? -8 : (q > 7 ? 7 : q);
+    return q < Code<BITS>::QLO ? Code<BITS>::QLO : (q > Code<BITS>::QHI ? Code<BITS>::QHI : q);
 }
 
 __device__ __forceinline__ h2 codes_to_h2(int q0, int q1) { return (h2){(h1)q0, (h1)q1}; }
 
-// Quantise one new token's channel pair with the current state and patch its two nibbles into the
-// channel words at token slot tt (0..7) of the supergroup (gemv.cu:91-146).  Returns the code pair.
+// Quantise one new token's channel pair with the current state and patch its two codes into the
+// channel words at token slot tt of the supergroup (gemv.cu:91-146).  Returns the code pair.
+template <int BITS = 4>
 __device__ __forceinline__ h2 append_pair(uint32_t &wa, uint32_t &wb, int tt, h2 x, const Pair &p)
 {
-    const int q0 = quantize(x.x, p.zp.x, p.sc.x);
-    const int q1 = quantize(x.y, p.zp.y, p.sc.y);
-    const uint32_t sh = 4u * (uint32_t)tt;
-    const uint32_t m = ~(0xFu << sh);
-    wa = (wa & m) | (((uint32_t)(q0 + 8) & 0xFu) << sh);
-    wb = (wb & m) | (((uint32_t)(q1 + 8) & 0xFu) << sh);
+    const int q0 = quantize<BITS>(x.x, p.zp.x, p.sc.x);
+    const int q1 = quantize<BITS>(x.y, p.zp.y, p.sc.y);
+    const uint32_t sh = (uint32_t)BITS * (uint32_t)tt;
+    const uint32_t m = ~(Code<BITS>::FIELD << sh);
+    wa = (wa & m) | (((uint32_t)(q0 - Code<BITS>::QLO) & Code<BITS>::FIELD) << sh);
+    wb = (wb & m) | (((uint32_t)(q1 - Code<BITS>::QLO) & Code<BITS>::FIELD) << sh);
     return codes_to_h2(q0, q1);
+}
+
+// Code pair of token slot tt straight from the channel words (ragged tails only).
+template <int BITS>
+__device__ __forceinline__ h2 extract_pair(uint32_t wa, uint32_t wb, int tt)
+{
+    const uint32_t sh = (uint32_t)BITS * (uint32_t)tt;
+    return codes_to_h2((int)((wa >> sh) & Code<BITS>::FIELD) + Code<BITS>::QLO,
+                       (int)((wb >> sh) & Code<BITS>::FIELD) + Code<BITS>::QLO);
+}
+
+// ---------------------------------------------------------------------------------------------
+// 2-bit codes: the table is indexed by a byte that holds TWO tokens of a channel pair and returns
+// 16 bytes, (q, |q|) for the low nibble's token then for the high nibble's.  16 copies per entry
+// (256-byte stride again, same 64 KB): a ds_read_b128 serves 16 lanes per clock.
+//   even.byte[j] = tokens 4j (low nibble) and 4j+2;  odd.byte[j] = tokens 4j+1 and 4j+3;
+//   nibble = code_A | code_B << 2.
+// ---------------------------------------------------------------------------------------------
+constexpr int LUT2_COPIES = 16;
+
+__device__ __forceinline__ void lut2_fill(uint2 *lut, int tid, int nthreads)
+{
+    uint4 *l4 = reinterpret_cast<uint4 *>(lut);
+    for (int i = tid; i < LUT_ENTRIES * LUT2_COPIES; i += nthreads) {
+        const int b = i / LUT2_COPIES;
+        const h2 lo = (h2){(h1)((b & 3) - 2), (h1)(((b >> 2) & 3) - 2)};
+        const h2 hi = (h2){(h1)(((b >> 4) & 3) - 2), (h1)((b >> 6) - 2)};
+        l4[i] = make_uint4(as_u32(lo), as_u32(lo) & 0x7FFF7FFFu, as_u32(hi), as_u32(hi) & 0x7FFF7FFFu);
+    }
+}
+
+__device__ __forceinline__ void pair_bytes2(uint32_t wa, uint32_t wb, uint32_t &even, uint32_t &odd)
+{
+    constexpr uint32_t m = 0x33333333u;
+    even = (wa & m) | ((wb & m) << 2);
+    odd = ((wa >> 2) & m) | (wb & ~m);
+}
+
+// lane_copy = (lane % 16) * 16.  k: byte of `bytes`, a compile-time constant after unrolling.
+__device__ __forceinline__ uint4 lut2_get(const uint2 *lut, uint32_t bytes, uint32_t lane_copy, int k)
+{
+    const uint32_t sel = 0x0C0C0000u | ((4u + (uint32_t)k) << 8);
+    const uint32_t addr = __builtin_amdgcn_perm(bytes, lane_copy, sel);
+    return *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(lut) + addr);
 }
 
 } // namespace adkv

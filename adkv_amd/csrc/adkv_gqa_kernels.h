@@ -1,5 +1,6 @@
 // Decode kernels for head dim 128 that put the contraction on the matrix cores, for GQ >= 1 query
-// heads per KV head.  Included inside namespace adkv by adkv_kernels.hip.
+// heads per KV head and for 4-bit or 2-bit codes.  Included inside namespace adkv by
+// adkv_kernels.hip.
 //
 // The fp16 replay of the filter state (the dominant cost) is the same per-lane arithmetic as in
 // qk_kernel / ov_kernel and runs once per KV head; only what happens to the dequantised value
@@ -8,14 +9,18 @@
 // r of D (four fp32, one per row).
 //
 //   QK:  D[token][head] += A[token][4 channels] * B[4 channels][head]
-//        The dequantised keys of one supergroup (8 tokens x 2 heads x 128 channels) go through a
-//        wave-private LDS tile; a block is (KV head, 4 tokens, a quarter of the channels), eight
-//        instructions walk the quarter, two DPP rotations add the quarters.  No cross-lane
-//        reduction of per-lane partial dot products is left.
+//        The dequantised keys of 8 tokens x 2 heads x 128 channels go through a wave-private LDS
+//        tile; a block is (KV head, 4 tokens, a quarter of the channels), eight instructions walk
+//        the quarter, two DPP rotations add the quarters.  No cross-lane reduction of per-lane
+//        partial dot products is left.
 //   OV:  D[head][channel] += A[head][4 tokens] * B[4 tokens][channel]
 //        B is the lane's own channel over four consecutive tokens (two v_perm_b32 per channel pair
 //        repack token-major pairs), A the attention weights of the block's heads: every lane gets
 //        the outputs of all GQ heads for its own channels, with no data leaving the lane.
+//
+// The time axis is walked in units of 8 tokens: one unit per supergroup with 4-bit codes, two with
+// 2-bit codes (16 tokens per channel word).  Table lookups for the next unit are issued between
+// the tokens of the current one, into the register slots they vacate.
 #pragma once
 
 typedef float f4v __attribute__((ext_vector_type(4)));
@@ -38,10 +43,91 @@ __device__ __forceinline__ h4v as_h4(uint32_t lo, uint32_t hi)
     return __builtin_bit_cast(h4v, make_uint2(lo, hi));
 }
 
+// The code words of one supergroup -> the per-pair byte streams the table is indexed with.
+template <int BITS>
+__device__ __forceinline__ void code_bytes(const uint4 &u, uint32_t (*nb)[2])
+{
+    if (BITS == 4) {
+        pair_bytes(u.x, u.y, nb[0][0], nb[0][1]);
+        pair_bytes(u.z, u.w, nb[1][0], nb[1][1]);
+    } else {
+        pair_bytes2(u.x, u.y, nb[0][0], nb[0][1]);
+        pair_bytes2(u.z, u.w, nb[1][0], nb[1][1]);
+    }
+}
+
+// Table entries of one 8-token unit held in registers, and how a token finds its (q, |q|):
+//   4-bit: slot t, 8 bytes.   2-bit: slot 2*(t/4) + (t&1), 16 bytes, second half for t&2.
+template <int BITS>
+struct Lookups {
+    static constexpr int SLOTS = BITS == 4 ? 8 : 4;
+    using Entry = typename std::conditional<BITS == 4, uint2, uint4>::type;
+    Entry e[2][SLOTS];
+
+    // all lookups of unit `half` (0 or 1 within the supergroup) of the words `nb`
+    __device__ __forceinline__ void fill(const uint2 *lut, const uint32_t (*nb)[2], uint32_t lane_copy, int half)
+    {
+#pragma unroll
+        for (int p = 0; p < 2; p++) {
+            if constexpr (BITS == 4) {
+#pragma unroll
+                for (int t = 0; t < 8; t++)
+                    e[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+            } else {
+#pragma unroll
+                for (int s = 0; s < 4; s++)
+                    e[p][s] = lut2_get(lut, nb[p][s & 1], lane_copy, 2 * half + (s >> 1));
+            }
+        }
+    }
+    __device__ __forceinline__ void get(int p, int t, h2 &q, h2 &qabs) const
+    {
+        if constexpr (BITS == 4) {
+            q = as_h2(e[p][t].x);
+            qabs = as_h2(e[p][t].y);
+        } else {
+            const uint4 v = e[p][2 * (t >> 2) + (t & 1)];
+            q = as_h2((t & 2) ? v.z : v.x);
+            qabs = as_h2((t & 2) ? v.w : v.y);
+        }
+    }
+    // after token t: refill the slot it has just finished with, for the unit `next_half` of `nb`
+    __device__ __forceinline__ void refill(const uint2 *lut, const uint32_t (*nb)[2], uint32_t lane_copy,
+                                           int t, int next_half)
+    {
+        if constexpr (BITS == 4) {
+#pragma unroll
+            for (int p = 0; p < 2; p++)
+                e[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+        } else {
+            if (t & 2) {
+#pragma unroll
+                for (int p = 0; p < 2; p++)
+                    e[p][2 * (t >> 2) + (t & 1)] = lut2_get(lut, nb[p][t & 1], lane_copy, 2 * next_half + (t >> 2));
+            }
+        }
+    }
+};
+
+template <int BITS>
+__device__ __forceinline__ void fill_table(uint2 *lut, int tid, int nthreads)
+{
+    if (BITS == 4)
+        lut_fill(lut, tid, nthreads);
+    else
+        lut2_fill(lut, tid, nthreads);
+}
+
+template <int BITS>
+__device__ __forceinline__ uint32_t table_lane_offset(int lane)
+{
+    return BITS == 4 ? (uint32_t)(lane & (LUT_COPIES - 1)) * 8u : (uint32_t)(lane & (LUT2_COPIES - 1)) * 16u;
+}
+
 // ---------------------------------------------------------------------------------------------
 // forward_qk with GQ query heads per KV head
 // ---------------------------------------------------------------------------------------------
-template <int GQ, int BLK>
+template <int BITS, int GQ, int BLK>
 __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
     const h1 *__restrict__ q, uint4 *__restrict__ cache, const h1 *__restrict__ k_new,
     h1 *__restrict__ out,
@@ -51,14 +137,15 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
 {
     constexpr int D = GQA_D, CPL = GQA_CPL;
     constexpr int NB = (GQ + 3) / 4; // column sets of four heads
+    constexpr int TPW = Code<BITS>::TPW, UPS = TPW / 8;
     using G = Geo<D, CPL>;
     __shared__ uint2 smem[LUT_WORDS64 + (BLK / 64) * TILE_WORDS64];
     const uint2 *lut = smem;
-    lut_fill(smem, threadIdx.x, BLK);
+    fill_table<BITS>(smem, threadIdx.x, BLK);
     __syncthreads();
 
     const int lane = threadIdx.x & 63;
-    const uint32_t lane_copy = (uint32_t)(lane & (LUT_COPIES - 1)) * 8u;
+    const uint32_t lane_copy = table_lane_offset<BITS>(lane);
     uint2 *tile = smem + LUT_WORDS64 + (threadIdx.x >> 6) * TILE_WORDS64;
 
     const Unit<D, CPL, BLK> un(BH, sa.nseg);
@@ -87,17 +174,17 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
     const int t0 = un.seg * sa.seg_tokens;
     const int t1 = last ? T : t0 + sa.seg_tokens;
     uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV;
-    const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;
-    const int nfull = (t1 - t0) >> 3;
+    const uint4 *cb = cbh + (size_t)(t0 / TPW) * G::VPS;
+    const int nfull = (t1 - t0) / TPW;
 
     // logits of the tile's tokens: read the A operands, run the instructions, add the quarters,
-    // lane (.., qd, r) stores token tg4*4+qd of head r
+    // lane (.., qd, r) stores token tg4*4+qd of head r.  `unit` counts 8-token units from t0.
     auto emit_read = [&](uint2 *a) {
 #pragma unroll
         for (int m = 0; m < 8; m++)
             a[m] = arow[m];
     };
-    auto emit_finish = [&](const uint2 *a, int sg, int ntok) {
+    auto emit_finish = [&](const uint2 *a, int unit, int ntok) {
 #pragma unroll
         for (int n = 0; n < NB; n++) {
             f4v d = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -116,77 +203,80 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
             const float mine = qd == 0 ? s[0] : qd == 1 ? s[1] : qd == 2 ? s[2] : s[3];
             const int tok = tg4 * 4 + qd, g = 4 * n + r;
             if (active && g < GQ && tok < ntok)
-                out[((size_t)bx * GQ + g) * (T + 1) + t0 + sg * 8 + tok] = (h1)mine;
+                out[((size_t)bx * GQ + g) * (T + 1) + t0 + unit * 8 + tok] = (h1)mine;
         }
     };
 
-    auto token = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2]) {
+    Lookups<BITS> lk;
+    // token t of the current unit; then the lookups that reuse its slot for the unit after it
+    auto token = [&](int t, const uint32_t (*nbnext)[2], int next_half) {
         uint32_t kh[G::NP];
 #pragma unroll
         for (int p = 0; p < G::NP; p++) {
             Pair &s = st[p];
-            const h2 qs = as_h2(e[p][t].x) * s.sc;
+            h2 qc, qa;
+            lk.get(p, t, qc, qa);
+            const h2 qs = qc * s.sc;
             kh[p] = as_u32(qs + s.zp);
-            update_pair_abs(s, as_h2(e[p][t].y), qs);
+            update_pair_abs(s, qa, qs);
         }
         tile[t * TILE_ROW64 + lane] = make_uint2(kh[0], kh[1]);
-#pragma unroll
-        for (int p = 0; p < G::NP; p++)
-            e[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+        lk.refill(lut, nbnext, lane_copy, t, next_half);
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    uint4 buf[PF][G::NV];
-    uint2 lk[G::NP][8];
-    uint32_t nb[G::NP][2];
+    uint4 buf[PF];
+    uint32_t nbc[G::NP][2], nbn[G::NP][2]; // byte streams of the current / the next supergroup
     uint2 areg[8];
 #pragma unroll
-    for (int i = 0; i < PF; i++) {
-#pragma unroll
-        for (int v = 0; v < G::NV; v++)
-            buf[i][v] = (i < nfull) ? cb[(size_t)i * G::VPS + v] : make_uint4(0, 0, 0, 0);
-    }
+    for (int i = 0; i < PF; i++)
+        buf[i] = (i < nfull) ? cb[(size_t)i * G::VPS] : make_uint4(0, 0, 0, 0);
     if (nfull > 0) {
-        pair_bytes_of<D, CPL>(buf[0], nb);
-#pragma unroll
-        for (int t = 0; t < 8; t++)
-#pragma unroll
-            for (int p = 0; p < G::NP; p++)
-                lk[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+        code_bytes<BITS>(buf[0], nbc);
+        lk.fill(lut, nbc, lane_copy, 0);
     }
     for (int sg0 = 0; sg0 < nfull; sg0 += PF) {
 #pragma unroll
         for (int i = 0; i < PF; i++) {
             const int sg = sg0 + i;
             if (sg < nfull) {
-                pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
-                if (sg + PF < nfull) {
-#pragma unroll
-                    for (int v = 0; v < G::NV; v++)
-                        buf[i][v] = cb[(size_t)(sg + PF) * G::VPS + v];
-                }
+                // bytes of supergroup sg+1 (stale data past the end: looked up, never used)
+                code_bytes<BITS>(buf[(i + 1) % PF], nbn);
+                if (sg + PF < nfull)
+                    buf[i] = cb[(size_t)(sg + PF) * G::VPS];
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int t = 0; t < 3; t++)
-                    token(t, lk, nb);
-                // the tile reads of supergroup sg-1 were issued before these three tokens
-                // overwrote its first rows (LDS operations of a wave execute in order)
-                if (sg > 0)
-                    emit_finish(areg, sg - 1, 8);
+                for (int hf = 0; hf < UPS; hf++) {
+                    const int unit = sg * UPS + hf;
+                    const bool into_next_sg = hf == UPS - 1;
 #pragma unroll
-                for (int t = 3; t < 8; t++)
-                    token(t, lk, nb);
-                emit_read(areg);
+                    for (int t = 0; t < 3; t++)
+                        token(t, into_next_sg ? nbn : nbc, into_next_sg ? 0 : hf + 1);
+                    // the tile reads of the previous unit were issued before these three tokens
+                    // overwrote its first rows (LDS operations of a wave execute in order)
+                    if (unit > 0)
+                        emit_finish(areg, unit - 1, 8);
+#pragma unroll
+                    for (int t = 3; t < 8; t++)
+                        token(t, into_next_sg ? nbn : nbc, into_next_sg ? 0 : hf + 1);
+                    emit_read(areg);
+                }
+#pragma unroll
+                for (int p = 0; p < G::NP; p++) {
+                    nbc[p][0] = nbn[p][0];
+                    nbc[p][1] = nbn[p][1];
+                }
             }
         }
     }
     if (nfull > 0)
-        emit_finish(areg, nfull - 1, 8);
+        emit_finish(areg, nfull * UPS - 1, 8);
     if (!last)
         return;
 
-    // ragged tail (T % 8 tokens, gemv.cu:648-654) and the appended token share one more tile
-    const int ntail = (t1 - t0) & 7;
+    // ragged tail (fewer than a supergroup of tokens, gemv.cu:648-654) and the appended token
+    const int ntail = (t1 - t0) % TPW;
+    int unit = nfull * UPS, row = 0;
     if (ntail) {
         const uint4 u = cb[(size_t)nfull * G::VPS];
         const uint32_t w[4] = {u.x, u.y, u.z, u.w};
@@ -195,29 +285,33 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
 #pragma unroll
             for (int pp = 0; pp < 2; pp++) {
                 Pair &s = st[pp];
-                const uint32_t na = (w[2 * pp] >> (4 * tt)) & 0xFu;
-                const uint32_t nbb = (w[2 * pp + 1] >> (4 * tt)) & 0xFu;
-                const h2 qc = codes_to_h2((int)na - 8, (int)nbb - 8);
+                const h2 qc = extract_pair<BITS>(w[2 * pp], w[2 * pp + 1], tt);
                 const h2 qs = qc * s.sc;
                 kh[pp] = as_u32(qs + s.zp);
                 update_pair(s, qc, qs);
             }
-            tile[tt * TILE_ROW64 + lane] = make_uint2(kh[0], kh[1]);
+            tile[row * TILE_ROW64 + lane] = make_uint2(kh[0], kh[1]);
+            if (++row == 8) {
+                emit_read(areg);
+                emit_finish(areg, unit, 8);
+                unit++;
+                row = 0;
+            }
         }
     }
     if (active)
         publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
     h2 deq[G::NP];
-    append_new_token<D, CPL>(cbh, T, k_new + (size_t)bx * D + c0, st, deq, active);
-    tile[ntail * TILE_ROW64 + lane] = make_uint2(as_u32(deq[0]), as_u32(deq[1]));
+    append_new_token<D, CPL, BITS>(cbh, T, k_new + (size_t)bx * D + c0, st, deq, active);
+    tile[row * TILE_ROW64 + lane] = make_uint2(as_u32(deq[0]), as_u32(deq[1]));
     emit_read(areg);
-    emit_finish(areg, nfull, ntail + 1);
+    emit_finish(areg, unit, row + 1);
 }
 
 // ---------------------------------------------------------------------------------------------
 // forward_ov with GQ query heads per KV head
 // ---------------------------------------------------------------------------------------------
-template <int GQ, int BLK>
+template <int BITS, int GQ, int BLK>
 __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
     const h1 *__restrict__ attn, uint4 *__restrict__ cache, const h1 *__restrict__ v_new,
     h1 *__restrict__ out, float *__restrict__ partial,
@@ -227,12 +321,15 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
 {
     constexpr int D = GQA_D, CPL = GQA_CPL;
     constexpr int NB = (GQ + 3) / 4;
+    constexpr int TPW = Code<BITS>::TPW, UPS = TPW / 8;
+    constexpr int WPF = 4; // weight vectors (8 tokens each) in flight
+    static_assert((PF * UPS) % WPF == 0, "weight ring must line up with the unrolled loop");
     using G = Geo<D, CPL>;
     __shared__ uint2 lut[LUT_WORDS64];
-    lut_fill(lut, threadIdx.x, BLK);
+    fill_table<BITS>(lut, threadIdx.x, BLK);
     __syncthreads();
     const int lane = threadIdx.x & 63;
-    const uint32_t lane_copy = (uint32_t)(lane & (LUT_COPIES - 1)) * 8u;
+    const uint32_t lane_copy = table_lane_offset<BITS>(lane);
 
     const Unit<D, CPL, BLK> un(BH, sa.nseg);
     const int bx = un.bx, lh = un.lh, c0 = un.c0;
@@ -253,8 +350,9 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
     const int t0 = un.seg * sa.seg_tokens;
     const int t1 = last ? T : t0 + sa.seg_tokens;
     uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV;
-    const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;
-    const int nfull = (t1 - t0) >> 3;
+    const uint4 *cb = cbh + (size_t)(t0 / TPW) * G::VPS;
+    const int nfull = (t1 - t0) / TPW;
+    const int nunits = nfull * UPS;
     // A operand rows: the weights of head r (+4 per column set) of this lane's KV head
     const h1 *wb[NB];
     bool wok[NB];
@@ -263,9 +361,9 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
         wok[n] = 4 * n + r < GQ;
         wb[n] = attn + ((size_t)bx * GQ + (wok[n] ? 4 * n + r : 0)) * (T + 1) + t0;
     }
-    auto load_w = [&](int n, int sg) {
+    auto load_w = [&](int n, int unit) {
         uint4 v;
-        __builtin_memcpy(&v, wb[n] + (size_t)sg * 8, 16); // rows are only 2-byte aligned
+        __builtin_memcpy(&v, wb[n] + (size_t)unit * 8, 16); // rows are only 2-byte aligned
         return wok[n] ? v : make_uint4(0u, 0u, 0u, 0u);
     };
 
@@ -288,68 +386,73 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
         }
     };
     uint32_t kh[G::NP][4];
-    auto token = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2]) {
+    Lookups<BITS> lk;
+    auto token = [&](int t, const uint32_t (*nbnext)[2], int next_half) {
 #pragma unroll
         for (int p = 0; p < G::NP; p++) {
             Pair &s = st[p];
-            const h2 qs = as_h2(e[p][t].x) * s.sc;
+            h2 qc, qa;
+            lk.get(p, t, qc, qa);
+            const h2 qs = qc * s.sc;
             kh[p][t & 3] = as_u32(qs + s.zp);
-            update_pair_abs(s, as_h2(e[p][t].y), qs);
+            update_pair_abs(s, qa, qs);
         }
-#pragma unroll
-        for (int p = 0; p < G::NP; p++)
-            e[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+        lk.refill(lut, nbnext, lane_copy, t, next_half);
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    uint4 buf[PF][G::NV];
-    uint4 wbuf[PF][NB];
-    uint2 lk[G::NP][8];
-    uint32_t nb[G::NP][2];
+    uint4 buf[PF];
+    uint4 wbuf[WPF][NB];
+    uint32_t nbc[G::NP][2], nbn[G::NP][2];
 #pragma unroll
-    for (int i = 0; i < PF; i++) {
+    for (int i = 0; i < PF; i++)
+        buf[i] = (i < nfull) ? cb[(size_t)i * G::VPS] : make_uint4(0, 0, 0, 0);
 #pragma unroll
-        for (int v = 0; v < G::NV; v++)
-            buf[i][v] = (i < nfull) ? cb[(size_t)i * G::VPS + v] : make_uint4(0, 0, 0, 0);
+    for (int i = 0; i < WPF; i++)
 #pragma unroll
         for (int n = 0; n < NB; n++)
-            wbuf[i][n] = (i < nfull) ? load_w(n, i) : make_uint4(0, 0, 0, 0);
-    }
+            wbuf[i][n] = (i < nunits) ? load_w(n, i) : make_uint4(0, 0, 0, 0);
     if (nfull > 0) {
-        pair_bytes_of<D, CPL>(buf[0], nb);
-#pragma unroll
-        for (int t = 0; t < 8; t++)
-#pragma unroll
-            for (int p = 0; p < G::NP; p++)
-                lk[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
+        code_bytes<BITS>(buf[0], nbc);
+        lk.fill(lut, nbc, lane_copy, 0);
     }
     for (int sg0 = 0; sg0 < nfull; sg0 += PF) {
 #pragma unroll
         for (int i = 0; i < PF; i++) {
             const int sg = sg0 + i;
             if (sg < nfull) {
-                pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
-                uint4 wcur[NB];
+                code_bytes<BITS>(buf[(i + 1) % PF], nbn);
+                if (sg + PF < nfull)
+                    buf[i] = cb[(size_t)(sg + PF) * G::VPS];
 #pragma unroll
-                for (int n = 0; n < NB; n++)
-                    wcur[n] = wbuf[i][n];
-                if (sg + PF < nfull) {
-#pragma unroll
-                    for (int v = 0; v < G::NV; v++)
-                        buf[i][v] = cb[(size_t)(sg + PF) * G::VPS + v];
+                for (int hf = 0; hf < UPS; hf++) {
+                    const int unit = sg * UPS + hf;
+                    const int ws = (i * UPS + hf) % WPF; // compile-time after unrolling
+                    uint4 wcur[NB];
 #pragma unroll
                     for (int n = 0; n < NB; n++)
-                        wbuf[i][n] = load_w(n, sg + PF);
+                        wcur[n] = wbuf[ws][n];
+                    if (unit + WPF < nunits) {
+#pragma unroll
+                        for (int n = 0; n < NB; n++)
+                            wbuf[ws][n] = load_w(n, unit + WPF);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    const bool into_next_sg = hf == UPS - 1;
+#pragma unroll
+                    for (int t = 0; t < 4; t++)
+                        token(t, into_next_sg ? nbn : nbc, into_next_sg ? 0 : hf + 1);
+                    contract(kh, wcur, 0);
+#pragma unroll
+                    for (int t = 4; t < 8; t++)
+                        token(t, into_next_sg ? nbn : nbc, into_next_sg ? 0 : hf + 1);
+                    contract(kh, wcur, 1);
                 }
-                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int t = 0; t < 4; t++)
-                    token(t, lk, nb);
-                contract(kh, wcur, 0);
-#pragma unroll
-                for (int t = 4; t < 8; t++)
-                    token(t, lk, nb);
-                contract(kh, wcur, 1);
+                for (int p = 0; p < G::NP; p++) {
+                    nbc[p][0] = nbn[p][0];
+                    nbc[p][1] = nbn[p][1];
+                }
             }
         }
     }
@@ -368,7 +471,7 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
                 }
             }
         };
-        const int ntail = (t1 - t0) & 7;
+        const int ntail = (t1 - t0) % TPW;
         if (ntail) {
             const uint4 u = cb[(size_t)nfull * G::VPS];
             const uint32_t w[4] = {u.x, u.y, u.z, u.w};
@@ -377,20 +480,18 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
 #pragma unroll
                 for (int pp = 0; pp < 2; pp++) {
                     Pair &s = st[pp];
-                    const uint32_t na = (w[2 * pp] >> (4 * tt)) & 0xFu;
-                    const uint32_t nbb = (w[2 * pp + 1] >> (4 * tt)) & 0xFu;
-                    const h2 qc = codes_to_h2((int)na - 8, (int)nbb - 8);
+                    const h2 qc = extract_pair<BITS>(w[2 * pp], w[2 * pp + 1], tt);
                     const h2 qs = qc * s.sc;
                     vd[pp] = qs + s.zp;
                     update_pair(s, qc, qs);
                 }
-                add_token(vd, t0 + nfull * 8 + tt);
+                add_token(vd, t0 + nfull * TPW + tt);
             }
         }
         if (active)
             publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
         h2 deq[G::NP];
-        append_new_token<D, CPL>(cbh, T, v_new + (size_t)bx * D + c0, st, deq, active);
+        append_new_token<D, CPL, BITS>(cbh, T, v_new + (size_t)bx * D + c0, st, deq, active);
         add_token(deq, T);
     }
     if (!active)

@@ -21,6 +21,8 @@
 
 #include <stdlib.h>
 
+#include <type_traits>
+
 #pragma clang fp contract(off)
 
 namespace adkv {
@@ -183,7 +185,7 @@ __device__ __forceinline__ void init_pairs(Pair *st, const h1 *zp, const h1 *sc,
 // summed as signed q << 4t and biased once by 0x8888... instead of being masked in one by one.
 constexpr int ENC_PF = 3; // supergroup input buffers in rotation
 
-template <int CPL, int BLK>
+template <int BITS, int CPL, int BLK>
 __global__ __launch_bounds__(BLK) void encode_kernel(
     uint32_t *__restrict__ cache, const h1 *__restrict__ kv_new,
     const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
@@ -194,6 +196,8 @@ __global__ __launch_bounds__(BLK) void encode_kernel(
     // Quantises tokens [T0, T) of a stream whose first T0 tokens are already in the cache; kv_new
     // holds the T - T0 new rows; state_in is the state after token T0-1 (ignored when T0 == 0).
     constexpr int NP = CPL >= 2 ? CPL / 2 : 1;
+    constexpr int TPW = Code<BITS>::TPW; // tokens per channel word
+    constexpr int G8 = TPW / 8;          // 8-token input groups per word
     const long total = (long)BH * D;
     long ci = ((long)blockIdx.x * BLK + threadIdx.x) * CPL;
     const bool active = ci < total;
@@ -240,18 +244,18 @@ __global__ __launch_bounds__(BLK) void encode_kernel(
     auto step = [&](const h2 *x, int tt, uint32_t *w) {
 #pragma unroll
         for (int p = 0; p < NP; p++) {
-            const int q0 = quantize_enc(x[p].x, st[p].zp.x, st[p].sc.x);
-            w[CPL >= 2 ? 2 * p : 0] += (uint32_t)q0 << (4 * tt);
+            const int q0 = quantize_enc<BITS>(x[p].x, st[p].zp.x, st[p].sc.x);
+            w[CPL >= 2 ? 2 * p : 0] += (uint32_t)q0 << (BITS * tt);
             int q1 = q0;
             if (CPL >= 2) {
-                q1 = quantize_enc(x[p].y, st[p].zp.y, st[p].sc.y);
-                w[2 * p + 1] += (uint32_t)q1 << (4 * tt);
+                q1 = quantize_enc<BITS>(x[p].y, st[p].zp.y, st[p].sc.y);
+                w[2 * p + 1] += (uint32_t)q1 << (BITS * tt);
             }
             const h2 q = (h2){(h1)(short)q0, (h1)(short)q1};
             update_pair(st[p], q, q * st[p].sc);
         }
     };
-    // bias adds 8 to the nibbles written now; keep selects nibbles of earlier tokens to preserve
+    // bias adds -QLO to the codes written now; keep selects codes of earlier tokens to preserve
     auto store_sg = [&](int sg, const uint32_t *w, uint32_t bias, uint32_t keep) {
         if (!active)
             return;
@@ -272,7 +276,7 @@ __global__ __launch_bounds__(BLK) void encode_kernel(
         else
             dst[0] = o[0];
         // state before token (j+1)*interval
-        const int tend = sg * 8 + 8;
+        const int tend = sg * TPW + TPW;
         if (sa.ckpt != nullptr && tend <= T && tend % sa.ckpt_interval == 0) {
             const int j = tend / sa.ckpt_interval - 1;
             if (j < sa.n_ckpt_cap)
@@ -280,62 +284,69 @@ __global__ __launch_bounds__(BLK) void encode_kernel(
         }
     };
 
-    auto nib_mask = [](int k) { return k >= 8 ? 0xFFFFFFFFu : ((1u << (4 * k)) - 1u); };
+    auto nib_mask = [](int k) { return k >= TPW ? 0xFFFFFFFFu : ((1u << (BITS * k)) - 1u); };
+    constexpr uint32_t BIAS = Code<BITS>::BIAS;
 
-    // a stream that resumes inside a supergroup first completes it (nibbles below T0 are kept)
+    // a stream that resumes inside a word first completes it (codes below T0 are kept)
     int t = T0;
-    if ((t & 7) && t < T) {
-        const int lo = t & 7, sg = t >> 3;
+    if ((t % TPW) && t < T) {
+        const int lo = t % TPW, sg = t / TPW;
         uint32_t w[CPL];
 #pragma unroll
         for (int c = 0; c < CPL; c++)
             w[c] = 0u;
-        for (; t < T && (t >> 3) == sg; t++) {
+        for (; t < T && t / TPW == sg; t++) {
             h2 x[NP];
             load_tok(t, x);
-            step(x, t & 7, w);
+            step(x, t % TPW, w);
         }
-        const int hi = (t >> 3) == sg ? (t & 7) : 8;
-        store_sg(sg, w, 0x88888888u & nib_mask(hi) & ~nib_mask(lo), nib_mask(lo));
+        const int hi = t / TPW == sg ? t % TPW : TPW;
+        store_sg(sg, w, BIAS & nib_mask(hi) & ~nib_mask(lo), nib_mask(lo));
     }
 
-    // full supergroups: no per-token conditions, inputs ENC_PF-1 supergroups ahead
-    const int sgb = t >> 3;                     // first full supergroup
-    const int nfull = (T - t) >> 3;
+    // full words: no per-token conditions, inputs ENC_PF-1 groups of 8 tokens ahead
+    const int sgb = t / TPW;                    // first full word
+    const int nfull = (T - t) / TPW;
+    const int ng = nfull * G8;
     h2 xbuf[ENC_PF][8][NP];
+    uint32_t w[CPL];
+#pragma unroll
+    for (int c = 0; c < CPL; c++)
+        w[c] = 0u;
 #pragma unroll
     for (int i = 0; i < ENC_PF - 1; i++)
-        if (i < nfull) {
+        if (i < ng) {
 #pragma unroll
             for (int tt = 0; tt < 8; tt++)
-                load_tok((sgb + i) * 8 + tt, xbuf[i][tt]);
+                load_tok(t + i * 8 + tt, xbuf[i][tt]);
         }
-    for (int sg0 = 0; sg0 < nfull; sg0 += ENC_PF) {
+    for (int g0 = 0; g0 < ng; g0 += ENC_PF) {
 #pragma unroll
         for (int i = 0; i < ENC_PF; i++) {
-            const int sg = sg0 + i;
-            if (sg < nfull) {
-                if (sg + ENC_PF - 1 < nfull) {
+            const int g = g0 + i;
+            if (g < ng) {
+                if (g + ENC_PF - 1 < ng) {
 #pragma unroll
                     for (int tt = 0; tt < 8; tt++)
-                        load_tok((sgb + sg + ENC_PF - 1) * 8 + tt, xbuf[(i + ENC_PF - 1) % ENC_PF][tt]);
+                        load_tok(t + (g + ENC_PF - 1) * 8 + tt, xbuf[(i + ENC_PF - 1) % ENC_PF][tt]);
                 }
-                uint32_t w[CPL];
-#pragma unroll
-                for (int c = 0; c < CPL; c++)
-                    w[c] = 0u;
+                const int sub = G8 == 1 ? 0 : (g % G8) * 8;
 #pragma unroll
                 for (int tt = 0; tt < 8; tt++)
-                    step(xbuf[i][tt], tt, w);
-                store_sg(sgb + sg, w, 0x88888888u, 0u); // code = q + 8
+                    step(xbuf[i][tt], sub + tt, w);
+                if (G8 == 1 || g % G8 == G8 - 1) {
+                    store_sg(sgb + g / G8, w, BIAS, 0u);
+#pragma unroll
+                    for (int c = 0; c < CPL; c++)
+                        w[c] = 0u;
+                }
             }
         }
     }
-    // ragged last supergroup: codes of the tokens present, zero nibbles after them
-    t += nfull * 8;
+    // ragged last word: codes of the tokens present, zero fields after them
+    t += nfull * TPW;
     if (t < T) {
         const int ntail = T - t;
-        uint32_t w[CPL];
 #pragma unroll
         for (int c = 0; c < CPL; c++)
             w[c] = 0u;
@@ -344,7 +355,7 @@ __global__ __launch_bounds__(BLK) void encode_kernel(
             load_tok(t + tt, x);
             step(x, tt, w);
         }
-        store_sg(t >> 3, w, 0x88888888u & nib_mask(ntail), 0u);
+        store_sg(t / TPW, w, BIAS & nib_mask(ntail), 0u);
     }
     if (state_out != nullptr && active)
         store_state_n<CPL>(state_out + ((size_t)bx * D + c0) * 2, st);
@@ -353,12 +364,12 @@ __global__ __launch_bounds__(BLK) void encode_kernel(
 // Shared tail of the two decode kernels: quantise the new token with the state after token T-1,
 // patch it into slot T, return the fused dequant r16(q*sc + zp) per pair (gemv.cu:744-798,
 // 1105-1157).  The state is NOT advanced.
-template <int D, int CPL>
+template <int D, int CPL, int BITS = 4>
 __device__ __forceinline__ void append_new_token(uint4 *cb, int T, const h1 *xnew, const Pair *st,
                                                  h2 *deq, bool active)
 {
     using G = Geo<D, CPL>;
-    const int sg = T >> 3, tt = T & 7;
+    const int sg = T / Code<BITS>::TPW, tt = T % Code<BITS>::TPW;
 #pragma unroll
     for (int v = 0; v < G::NV; v++) {
         uint4 *slot = cb + (size_t)sg * G::VPS + v;
@@ -368,7 +379,7 @@ __device__ __forceinline__ void append_new_token(uint4 *cb, int T, const h1 *xne
         for (int pp = 0; pp < 2; pp++) {
             const int p = 2 * v + pp;
             const h2 x = *reinterpret_cast<const h2 *>(xnew + 2 * p);
-            const h2 q = append_pair(w[2 * pp], w[2 * pp + 1], tt, x, st[p]);
+            const h2 q = append_pair<BITS>(w[2 * pp], w[2 * pp + 1], tt, x, st[p]);
             deq[p] = pk_fma(q, st[p].sc, st[p].zp);
         }
         if (active)
@@ -1032,24 +1043,31 @@ static void launch_units(long threads, int big, F256 f256, FBIG fbig)
 
 // Matrix-core kernels (head dim 128): 16-wave workgroups for big launches, 8-wave ones otherwise
 // (their LDS tile leaves room for one workgroup per CU either way).
-#define ADKV_LAUNCH_GQA(KERNEL, GQV, ...)                                                          \
+#define ADKV_LAUNCH_GQA(KERNEL, BB, GQV, ...)                                                      \
     do {                                                                                            \
         const long threads = (long)BH * seg.nseg * 32;                                              \
         if (threads >= 1024L * 256)                                                                 \
-            hipLaunchKernelGGL((KERNEL<GQV, 1024>), dim3((unsigned)((threads + 1023) / 1024)),      \
+            hipLaunchKernelGGL((KERNEL<BB, GQV, 1024>), dim3((unsigned)((threads + 1023) / 1024)),  \
                                dim3(1024), 0, st, __VA_ARGS__);                                     \
         else                                                                                        \
-            hipLaunchKernelGGL((KERNEL<GQV, 512>), dim3((unsigned)((threads + 511) / 512)),         \
+            hipLaunchKernelGGL((KERNEL<BB, GQV, 512>), dim3((unsigned)((threads + 511) / 512)),     \
                                dim3(512), 0, st, __VA_ARGS__);                                      \
     } while (0)
 
-#define ADKV_DISPATCH_GQ(KERNEL, ...)                                                              \
+#define ADKV_DISPATCH_GQ_BITS(KERNEL, BB, ...)                                                     \
     switch (GQ) {                                                                                   \
-    case 1: ADKV_LAUNCH_GQA(KERNEL, 1, __VA_ARGS__); break;                                         \
-    case 2: ADKV_LAUNCH_GQA(KERNEL, 2, __VA_ARGS__); break;                                         \
-    case 4: ADKV_LAUNCH_GQA(KERNEL, 4, __VA_ARGS__); break;                                         \
-    case 8: ADKV_LAUNCH_GQA(KERNEL, 8, __VA_ARGS__); break;                                         \
+    case 1: ADKV_LAUNCH_GQA(KERNEL, BB, 1, __VA_ARGS__); break;                                     \
+    case 2: ADKV_LAUNCH_GQA(KERNEL, BB, 2, __VA_ARGS__); break;                                     \
+    case 4: ADKV_LAUNCH_GQA(KERNEL, BB, 4, __VA_ARGS__); break;                                     \
+    case 8: ADKV_LAUNCH_GQA(KERNEL, BB, 8, __VA_ARGS__); break;                                     \
     default: return ADKV_E_UNSUPPORTED;                                                             \
+    }
+
+#define ADKV_DISPATCH_GQ(KERNEL, ...)                                                              \
+    if (bits == 4) {                                                                                \
+        ADKV_DISPATCH_GQ_BITS(KERNEL, 4, __VA_ARGS__)                                               \
+    } else {                                                                                        \
+        ADKV_DISPATCH_GQ_BITS(KERNEL, 2, __VA_ARGS__)                                               \
     }
 
 // Whether single-query-head launches (GQ == 1, head dim 128) also take the matrix-core kernels:
@@ -1065,11 +1083,12 @@ static bool mfma_for_mha()
     return g_mha_kernel != 0;
 }
 
-static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval)
+static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval, int bits = 4)
 {
     if (!ckpt)
         return ADKV_OK;
-    if (n_ckpt_cap <= 0 || ckpt_interval <= 0 || (ckpt_interval & 7))
+    // a checkpoint sits on a supergroup boundary: 8 tokens with 4-bit codes, 16 with 2-bit ones
+    if (n_ckpt_cap <= 0 || ckpt_interval <= 0 || (ckpt_interval % (32 / bits)))
         return ADKV_E_SHAPE;
     if ((uintptr_t)ckpt & 3)
         return ADKV_E_ALIGN;
@@ -1078,7 +1097,7 @@ static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval)
 
 extern "C" {
 
-int adkv_abi_version(void) { return 5; }
+int adkv_abi_version(void) { return 6; }
 
 void adkv_set_mha_kernel(int use_matrix_cores) { g_mha_kernel = use_matrix_cores; }
 
@@ -1105,10 +1124,12 @@ static int encode_common(void *cache, const void *kv_new,
                          const void *tgt,
                          int B, int H, int T0, int T, int D, int n_super_cap,
                          const void *state_in, void *state_out, void *ckpt_out, int n_ckpt_cap,
-                         int ckpt_interval, void *stream)
+                         int ckpt_interval, void *stream, int bits = 4)
 {
     if (!cache || !kv_new || !zp || !sc || !alpha || !beta || !tgt)
         return ADKV_E_NULL;
+    if (bits != 2 && bits != 4)
+        return ADKV_E_UNSUPPORTED;
     int rc = check_common(B, H, T, D, n_super_cap);
     if (rc)
         return rc;
@@ -1116,11 +1137,12 @@ static int encode_common(void *cache, const void *kv_new,
         return ADKV_E_SHAPE;
     if (T0 > 0 && !state_in)
         return ADKV_E_NULL;
-    if ((T + 7) / 8 > n_super_cap)
+    const int tpw = 32 / bits;
+    if ((T + tpw - 1) / tpw > n_super_cap)
         return ADKV_E_CAPACITY;
     if (((uintptr_t)cache & 15) || ((uintptr_t)kv_new & 3))
         return ADKV_E_ALIGN;
-    if ((rc = check_ckpt(ckpt_out, n_ckpt_cap, ckpt_interval)))
+    if ((rc = check_ckpt(ckpt_out, n_ckpt_cap, ckpt_interval, bits)))
         return rc;
     if (T == T0 && (state_out == nullptr || state_out == state_in))
         return ADKV_OK;
@@ -1144,17 +1166,25 @@ static int encode_common(void *cache, const void *kv_new,
     }
     const long lanes = channels / cpl;
     const dim3 grid((unsigned)((lanes + 255) / 256)), block(256);
-#define ADKV_ENC(C)                                                                              \
-    hipLaunchKernelGGL((encode_kernel<C, 256>), grid, block, 0, st, (uint32_t *)cache,           \
+#define ADKV_ENC(BB, C)                                                                          \
+    hipLaunchKernelGGL((encode_kernel<BB, C, 256>), grid, block, 0, st, (uint32_t *)cache,       \
                        (const h1 *)kv_new, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,    \
                        (const h1 *)beta, (const h1 *)tgt, BH, H, T0, T, D, n_super_cap,          \
                        (const h1 *)state_in, (h1 *)state_out, seg)
-    if (cpl == 4)
-        ADKV_ENC(4);
-    else if (cpl == 2)
-        ADKV_ENC(2);
+#define ADKV_ENC_CPL(BB)                                                                         \
+    do {                                                                                         \
+        if (cpl == 4)                                                                            \
+            ADKV_ENC(BB, 4);                                                                     \
+        else if (cpl == 2)                                                                       \
+            ADKV_ENC(BB, 2);                                                                     \
+        else                                                                                     \
+            ADKV_ENC(BB, 1);                                                                     \
+    } while (0)
+    if (bits == 4)
+        ADKV_ENC_CPL(4);
     else
-        ADKV_ENC(1);
+        ADKV_ENC_CPL(2);
+#undef ADKV_ENC_CPL
 #undef ADKV_ENC
     return check_launch();
 }
@@ -1173,7 +1203,7 @@ int adkv_encode_kv_ex(void *cache, const void *kv_new,
 int adkv_append_kv(void *cache, const void *kv_new,
                    const void *zp, const void *sc, const void *alpha, const void *beta,
                    const void *tgt,
-                   int B, int H, int T0, int n_new, int D, int n_super_cap,
+                   int B, int H, int T0, int n_new, int D, int n_super_cap, int bits,
                    void *state_io, void *ckpt, int n_ckpt_cap, int ckpt_interval, void *stream)
 {
     if (!state_io)
@@ -1183,7 +1213,8 @@ int adkv_append_kv(void *cache, const void *kv_new,
     if (n_new == 0)
         return ADKV_OK; // nothing to quantise; state_io already is the answer
     return encode_common(cache, kv_new, zp, sc, alpha, beta, tgt, B, H, T0, T0 + n_new, D,
-                         n_super_cap, state_io, state_io, ckpt, n_ckpt_cap, ckpt_interval, stream);
+                         n_super_cap, state_io, state_io, ckpt, n_ckpt_cap, ckpt_interval, stream,
+                         bits);
 }
 
 int adkv_encode_kv(void *cache, const void *kv_new,
@@ -1199,30 +1230,32 @@ int adkv_encode_kv(void *cache, const void *kv_new,
 int adkv_forward_qk_gqa(const void *q, void *k_cache, const void *k_new, void *logits,
                         const void *zp, const void *sc, const void *alpha, const void *beta,
                         const void *tgt,
-                        int B, int Hq, int H, int T, int D, int n_super_cap,
+                        int B, int Hq, int H, int T, int D, int n_super_cap, int bits,
                         void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
                         void *stream)
 {
     if (!q || !k_cache || !k_new || !logits || !zp || !sc || !alpha || !beta || !tgt)
         return ADKV_E_NULL;
+    if (bits != 2 && bits != 4)
+        return ADKV_E_UNSUPPORTED;
     int rc = check_common(B, H, T, D, n_super_cap);
     if (rc)
         return rc;
     if (Hq <= 0 || Hq % H)
         return ADKV_E_SHAPE;
     const int GQ = Hq / H;
-    if (GQ > 1 && D != 128)
+    if ((GQ > 1 || bits != 4) && D != 128)
         return ADKV_E_UNSUPPORTED;
-    if ((T >> 3) >= n_super_cap)
+    if (T / (32 / bits) >= n_super_cap)
         return ADKV_E_CAPACITY;
     if (((uintptr_t)k_cache & 15) || ((uintptr_t)q & 7) || ((uintptr_t)k_new & 3))
         return ADKV_E_ALIGN;
-    if ((rc = check_ckpt(ckpt, n_ckpt_cap, ckpt_interval)))
+    if ((rc = check_ckpt(ckpt, n_ckpt_cap, ckpt_interval, bits)))
         return rc;
     const int BH = B * H;
     hipStream_t st = (hipStream_t)stream;
     const Seg seg = plan_segments(ckpt, n_ckpt_cap, ckpt_interval, BH, T, D);
-    if (D == 128 && (GQ > 1 || mfma_for_mha())) {
+    if (D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha())) {
         ADKV_DISPATCH_GQ(qk_gqa_kernel, (const h1 *)q, (uint4 *)k_cache, (const h1 *)k_new,
                          (h1 *)logits, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,
                          (const h1 *)beta, (const h1 *)tgt, BH, H, T, n_super_cap, (h1 *)state_out,
@@ -1243,7 +1276,7 @@ int adkv_forward_qk_ex(const void *q, void *k_cache, const void *k_new, void *lo
                        void *stream)
 {
     return adkv_forward_qk_gqa(q, k_cache, k_new, logits, zp, sc, alpha, beta, tgt, B, H, H, T, D,
-                               n_super_cap, state_out, ckpt, n_ckpt_cap, ckpt_interval, stream);
+                               n_super_cap, 4, state_out, ckpt, n_ckpt_cap, ckpt_interval, stream);
 }
 
 int adkv_forward_qk(const void *q, void *k_cache, const void *k_new, void *logits,
@@ -1268,25 +1301,27 @@ int64_t adkv_forward_ov_workspace_bytes(int B, int H, int T, int D, int n_ckpt_c
 int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void *out,
                         const void *zp, const void *sc, const void *alpha, const void *beta,
                         const void *tgt,
-                        int B, int Hq, int H, int T, int D, int n_super_cap,
+                        int B, int Hq, int H, int T, int D, int n_super_cap, int bits,
                         void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
                         void *workspace, int64_t workspace_bytes, void *stream)
 {
     if (!attn || !v_cache || !v_new || !out || !zp || !sc || !alpha || !beta || !tgt)
         return ADKV_E_NULL;
+    if (bits != 2 && bits != 4)
+        return ADKV_E_UNSUPPORTED;
     int rc = check_common(B, H, T, D, n_super_cap);
     if (rc)
         return rc;
     if (Hq <= 0 || Hq % H)
         return ADKV_E_SHAPE;
     const int GQ = Hq / H;
-    if (GQ > 1 && D != 128)
+    if ((GQ > 1 || bits != 4) && D != 128)
         return ADKV_E_UNSUPPORTED;
-    if ((T >> 3) >= n_super_cap)
+    if (T / (32 / bits) >= n_super_cap)
         return ADKV_E_CAPACITY;
     if (((uintptr_t)v_cache & 15) || ((uintptr_t)out & 3) || ((uintptr_t)v_new & 3))
         return ADKV_E_ALIGN;
-    if ((rc = check_ckpt(ckpt, n_ckpt_cap, ckpt_interval)))
+    if ((rc = check_ckpt(ckpt, n_ckpt_cap, ckpt_interval, bits)))
         return rc;
     const int BH = B * H;
     hipStream_t st = (hipStream_t)stream;
@@ -1297,7 +1332,7 @@ int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void
         if ((uintptr_t)workspace & 15)
             return ADKV_E_ALIGN;
     }
-    if (D == 128 && (GQ > 1 || mfma_for_mha())) {
+    if (D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha())) {
         ADKV_DISPATCH_GQ(ov_gqa_kernel, (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new,
                          (h1 *)out, (float *)workspace, (const h1 *)zp, (const h1 *)sc,
                          (const h1 *)alpha, (const h1 *)beta, (const h1 *)tgt, BH, H, T, n_super_cap,
@@ -1327,7 +1362,7 @@ int adkv_forward_ov_ex(const void *attn, void *v_cache, const void *v_new, void 
                        void *workspace, int64_t workspace_bytes, void *stream)
 {
     return adkv_forward_ov_gqa(attn, v_cache, v_new, out, zp, sc, alpha, beta, tgt, B, H, H, T, D,
-                               n_super_cap, state_out, ckpt, n_ckpt_cap, ckpt_interval, workspace,
+                               n_super_cap, 4, state_out, ckpt, n_ckpt_cap, ckpt_interval, workspace,
                                workspace_bytes, stream);
 }
 
@@ -1410,7 +1445,7 @@ int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k
                       const void *const *k_params, const void *const *v_params,
                       const void *mask, int rows_per_mask_row, float scaling,
                       void *out, void *weights_out,
-                      int B, int Hq, int H, int T, int D, int n_super_cap,
+                      int B, int Hq, int H, int T, int D, int n_super_cap, int bits,
                       void *k_ckpt, void *v_ckpt, int n_ckpt_cap, int ckpt_interval,
                       void *workspace, int64_t workspace_bytes, void *stream)
 {
@@ -1427,7 +1462,7 @@ int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k
     void *logits = ws;
     void *weights = weights_out ? weights_out : (void *)(ws + row);
     int rc = adkv_forward_qk_gqa(q, k_cache, k_new, logits, k_params[0], k_params[1], k_params[2],
-                                 k_params[3], k_params[4], B, Hq, H, T, D, n_super_cap, nullptr,
+                                 k_params[3], k_params[4], B, Hq, H, T, D, n_super_cap, bits, nullptr,
                                  k_ckpt, n_ckpt_cap, ckpt_interval, stream);
     if (rc)
         return rc;
@@ -1437,7 +1472,7 @@ int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k
     if (rc)
         return rc;
     return adkv_forward_ov_gqa(weights, v_cache, v_new, out, v_params[0], v_params[1], v_params[2],
-                               v_params[3], v_params[4], B, Hq, H, T, D, n_super_cap, nullptr,
+                               v_params[3], v_params[4], B, Hq, H, T, D, n_super_cap, bits, nullptr,
                                v_ckpt, n_ckpt_cap, ckpt_interval, ws + 2 * row + smb,
                                workspace_bytes - 2 * row - smb, stream);
 }

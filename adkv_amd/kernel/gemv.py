@@ -51,7 +51,7 @@ def _ptr(t: torch.Tensor | None) -> int | None:
     return None if t is None else t.data_ptr()
 
 
-def _ckpt_args(ckpt: torch.Tensor | None, ckpt_interval: int, B: int, nh: int, DIM: int):
+def _ckpt_args(ckpt: torch.Tensor | None, ckpt_interval: int, B: int, nh: int, DIM: int, bits: int = 4):
     """Validates a checkpoint tensor ``[B, nh, n_ckpt_cap, DIM, 2]`` fp16 -> (ptr, cap, interval)."""
     if ckpt is None:
         return None, 0, 0
@@ -59,7 +59,9 @@ def _ckpt_args(ckpt: torch.Tensor | None, ckpt_interval: int, B: int, nh: int, D
          and ckpt.shape[0] == B and ckpt.shape[1] == nh and ckpt.shape[3] == DIM and ckpt.shape[4] == 2
          and ckpt.shape[2] >= 1,
          "ckpt must be contiguous fp16 [B, nh, n_ckpt_cap, DIM, 2]")
-    _chk(ckpt_interval > 0 and ckpt_interval % 8 == 0, "ckpt_interval must be a positive multiple of 8")
+    tps = 32 // bits
+    _chk(ckpt_interval > 0 and ckpt_interval % tps == 0,
+         f"ckpt_interval must be a positive multiple of {tps}")
     return ckpt.data_ptr(), ckpt.shape[2], int(ckpt_interval)
 
 
@@ -79,6 +81,7 @@ def forward_qk(
     state_out: torch.Tensor | None = None,
     ckpt: torch.Tensor | None = None,
     ckpt_interval: int = 0,
+    bits: int = 4,
 ) -> torch.Tensor:
     """Decode-phase QK^T over the nibble-packed ADKV cache (reference gemv.py:16-55).
 
@@ -115,7 +118,9 @@ def forward_qk(
     _chk(nq % nh == 0 and nq // nh in _GROUPS, "query heads must be 1, 2, 4 or 8 times the KV heads")
     _chk(nq == nh or DIM == 128, "grouped-query attention needs DIM == 128")
     _chk(T >= 0, "T must be non-negative")
-    _chk((T >> 1) // _TILE < n_super_cap, f"k_cache has no free supergroup to append token {T}")
+    _chk(bits in (2, 4), "bits must be 2 or 4")
+    _chk(bits == 4 or DIM == 128, "2-bit codes need DIM == 128")
+    _chk(T // (32 // bits) < n_super_cap, f"k_cache has no free supergroup to append token {T}")
     _chk(DIM in _DIMS, "DIM must be 128, 256 or 512")
     dev = _need_device(q, k_cache, k_new, zp, sc, al, be, tg)
 
@@ -125,12 +130,12 @@ def forward_qk(
     if state_out is not None:
         _chk(state_out.dtype == torch.float16 and state_out.is_contiguous()
              and state_out.numel() == B * nh * DIM * 2, "state_out must be contiguous fp16 [B,nh,DIM,2]")
-    cp, ccap, civ = _ckpt_args(ckpt, ckpt_interval, B, nh, DIM)
+    cp, ccap, civ = _ckpt_args(ckpt, ckpt_interval, B, nh, DIM, bits)
     with torch.cuda.device(dev):
         rc = _lib.lib().adkv_forward_qk_gqa(
             q_flat.data_ptr(), k_cache.data_ptr(), k_new_flat.data_ptr(), o.data_ptr(),
             zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
-            B, nq, nh, T, DIM, n_super_cap, _ptr(state_out), cp, ccap, civ,
+            B, nq, nh, T, DIM, n_super_cap, bits, _ptr(state_out), cp, ccap, civ,
             _lib.current_stream_ptr(dev))
     _lib.check(rc, "forward_qk")
     return o.reshape(B, nq, T + 1)
@@ -151,6 +156,7 @@ def forward_ov(
     state_out: torch.Tensor | None = None,
     ckpt: torch.Tensor | None = None,
     ckpt_interval: int = 0,
+    bits: int = 4,
 ) -> torch.Tensor:
     """Decode-phase OV over the nibble-packed ADKV cache (reference gemv.py:58-97).
 
@@ -176,7 +182,9 @@ def forward_ov(
     _chk(nq % nh == 0 and nq // nh in _GROUPS, "query heads must be 1, 2, 4 or 8 times the KV heads")
     _chk(nq == nh or DIM == 128, "grouped-query attention needs DIM == 128")
     _chk(T >= 0, "T must be non-negative")
-    _chk((T >> 1) // _TILE < n_super_cap, f"v_cache has no free supergroup to append token {T}")
+    _chk(bits in (2, 4), "bits must be 2 or 4")
+    _chk(bits == 4 or DIM == 128, "2-bit codes need DIM == 128")
+    _chk(T // (32 // bits) < n_super_cap, f"v_cache has no free supergroup to append token {T}")
     _chk(DIM in _DIMS, "DIM must be 128, 256 or 512")
     dev = _need_device(attn, v_cache, v_new, zp, sc, al, be, tg)
 
@@ -186,7 +194,7 @@ def forward_ov(
     if state_out is not None:
         _chk(state_out.dtype == torch.float16 and state_out.is_contiguous()
              and state_out.numel() == B * nh * DIM * 2, "state_out must be contiguous fp16 [B,nh,DIM,2]")
-    cp, ccap, civ = _ckpt_args(ckpt, ckpt_interval, B, nh, DIM)
+    cp, ccap, civ = _ckpt_args(ckpt, ckpt_interval, B, nh, DIM, bits)
     L = _lib.lib()
     ws, ws_bytes = None, 0
     if cp is not None:
@@ -197,7 +205,7 @@ def forward_ov(
         rc = L.adkv_forward_ov_gqa(
             attn_flat.data_ptr(), v_cache.data_ptr(), v_new_flat.data_ptr(), o.data_ptr(),
             zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
-            B, nq, nh, T, DIM, n_super_cap, _ptr(state_out), cp, ccap, civ,
+            B, nq, nh, T, DIM, n_super_cap, bits, _ptr(state_out), cp, ccap, civ,
             _ptr(ws), ws_bytes, _lib.current_stream_ptr(dev))
     _lib.check(rc, "forward_ov")
     return o.view(attn.shape[0], attn.shape[1], -1)
@@ -268,6 +276,7 @@ def append_kv(
     *,
     ckpt: torch.Tensor | None = None,
     ckpt_interval: int = 0,
+    bits: int = 4,
 ) -> torch.Tensor:
     """Streaming append (extension; the reference can only append inside forward_qk/forward_ov,
     after an O(T) replay): quantise ``kv_new [B, nh, n, DIM]`` as tokens ``T0 .. T0+n-1``.
@@ -285,14 +294,16 @@ def append_kv(
     n_super_cap = kv_cache.shape[2]
     _chk(kv_cache.shape[3] * _TILE == DIM, "kv_cache channel groups do not match kv_new head dim")
     _chk(T0 >= 0, "T0 must be non-negative")
-    need = (T0 + n + 7) // 8
+    _chk(bits in (2, 4), "bits must be 2 or 4")
+    tps = 32 // bits
+    need = (T0 + n + tps - 1) // tps
     _chk(need <= n_super_cap,
          f"kv_cache capacity too small: need {need} supergroups for {T0 + n} tokens, have {n_super_cap}")
     _chk(DIM in _DIMS, "DIM must be 128, 256 or 512")
     _chk(state.dtype == torch.float16 and state.is_contiguous() and state.numel() == B * nh * DIM * 2,
          "state must be contiguous fp16 [B,nh,DIM,2]")
     dev = _need_device(kv_cache, kv_new, zp, sc, al, be, tg, state)
-    cp, ccap, civ = _ckpt_args(ckpt, ckpt_interval, B, nh, DIM)
+    cp, ccap, civ = _ckpt_args(ckpt, ckpt_interval, B, nh, DIM, bits)
     if n == 0:
         return kv_cache
     x = kv_new.contiguous()
@@ -300,7 +311,7 @@ def append_kv(
         rc = _lib.lib().adkv_append_kv(
             kv_cache.data_ptr(), x.data_ptr(),
             zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
-            B, nh, T0, n, DIM, n_super_cap, state.data_ptr(), cp, ccap, civ,
+            B, nh, T0, n, DIM, n_super_cap, bits, state.data_ptr(), cp, ccap, civ,
             _lib.current_stream_ptr(dev))
     _lib.check(rc, "append_kv")
     return kv_cache
@@ -354,6 +365,7 @@ def decode_fused(
     k_ckpt: torch.Tensor | None = None,
     v_ckpt: torch.Tensor | None = None,
     ckpt_interval: int = 0,
+    bits: int = 4,
     workspace: torch.Tensor | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """One decode-attention step of a layer through a single library call.
@@ -379,7 +391,9 @@ def decode_fused(
     vp = _params(v_params, ("v_zp", "v_sc", "v_alpha", "v_beta", "v_t"), nh, DIM)
     _chk(DIM == q.shape[-1], "q head dimension does not match k_cache")
     _chk(T >= 0, "T must be non-negative")
-    _chk((T >> 1) // _TILE < n_super_cap, f"k_cache has no free supergroup to append token {T}")
+    _chk(bits in (2, 4), "bits must be 2 or 4")
+    _chk(bits == 4 or DIM == 128, "2-bit codes need DIM == 128")
+    _chk(T // (32 // bits) < n_super_cap, f"k_cache has no free supergroup to append token {T}")
     _chk(DIM in _DIMS, "DIM must be 128, 256 or 512")
     dev = _need_device(q, k_cache, v_cache, k_new, v_new, *kp, *vp)
     n = T + 1
@@ -391,8 +405,8 @@ def decode_fused(
         rpm = nq if mk.shape[1] == 1 else 1
         mk = mk.to(device=dev, dtype=torch.float32).contiguous()
         mptr = mk.data_ptr()
-    kcp, ccap, civ = _ckpt_args(k_ckpt, ckpt_interval, B, nh, DIM)
-    vcp, vcap, _ = _ckpt_args(v_ckpt, ckpt_interval, B, nh, DIM)
+    kcp, ccap, civ = _ckpt_args(k_ckpt, ckpt_interval, B, nh, DIM, bits)
+    vcp, vcap, _ = _ckpt_args(v_ckpt, ckpt_interval, B, nh, DIM, bits)
     _chk((k_ckpt is None) == (v_ckpt is None) and ccap == vcap,
          "k_ckpt and v_ckpt must both be given, with the same capacity, or both omitted")
     L = _lib.lib()
@@ -412,7 +426,7 @@ def decode_fused(
             qf.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), knf.data_ptr(), vnf.data_ptr(),
             arr(*[t.data_ptr() for t in kp]), arr(*[t.data_ptr() for t in vp]),
             mptr, rpm, float(scaling), out.data_ptr(), weights.data_ptr(),
-            B, nq, nh, T, DIM, n_super_cap, kcp, vcp, ccap, civ,
+            B, nq, nh, T, DIM, n_super_cap, bits, kcp, vcp, ccap, civ,
             workspace.data_ptr(), workspace.numel(), _lib.current_stream_ptr(dev))
     _lib.check(rc, "decode_fused")
     return out, weights

@@ -81,7 +81,8 @@ def n_super(tokens: int) -> int:
     return (tokens + 7) // 8
 
 
-def alloc_cache(B: int, H: int, cap_tokens: int, D: int, device) -> torch.Tensor:
+def alloc_cache(B: int, H: int, cap_tokens: int, D: int, device, bits: int = 4) -> torch.Tensor:
     """Zero-filled packed cache ``[B, H, n_super, D/4, 4, 4]`` uint8
-    (src/adkv/hf/llama_adkv.py:87-94)."""
-    return torch.zeros((B, H, n_super(cap_tokens), D // 4, 4, 4), dtype=torch.uint8, device=device)
+    (src/adkv/hf/llama_adkv.py:87-94); a supergroup is ``32 // bits`` tokens."""
+    tps = 32 // bits
+    return torch.zeros((B, H, -(-cap_tokens // tps), D // 4, 4, 4), dtype=torch.uint8, device=device)

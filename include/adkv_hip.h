@@ -130,7 +130,7 @@ int adkv_encode_kv_ex(void *cache, const void *kv_new,
 int adkv_append_kv(void *cache, const void *kv_new,
                    const void *zp, const void *sc, const void *alpha, const void *beta,
                    const void *tgt,
-                   int B, int H, int T0, int n_new, int D, int n_super_cap,
+                   int B, int H, int T0, int n_new, int D, int n_super_cap, int bits,
                    void *state_io, void *ckpt, int n_ckpt_cap, int ckpt_interval, void *stream);
 
 int adkv_forward_qk_ex(const void *q, void *k_cache, const void *k_new, void *logits,
@@ -158,11 +158,17 @@ int adkv_forward_ov_ex(const void *attn, void *v_cache, const void *v_new, void 
  * the contraction with all of its query heads goes to the matrix cores.  Head dim 128 only when
  * Hq > H.  q: [B, Hq, D]; logits / attn: [B, Hq, T+1]; out: [B, Hq, D]; everything else as in the
  * _ex entry points.  The OV workspace is adkv_forward_ov_gqa_workspace_bytes(...) bytes.
+ *
+ * bits: 4 = the reference's code format.  2 = the same fp16 recurrence over codes in [-2, 1]
+ * (QL/QU of src/adkv/train/train_model.py:96-97 for bits = 2), stored as q + 2 with 16 tokens per
+ * 32-bit channel word, i.e. supergroups of 16 tokens in the same uint8 [B,H,n_super,D/4,4,4]
+ * tensor; head dim 128 only, checkpoint intervals a multiple of 16.  The reference has no kernel
+ * for it.  adkv_append_kv (T0 = 0 for a whole prompt) writes such caches.
  */
 int adkv_forward_qk_gqa(const void *q, void *k_cache, const void *k_new, void *logits,
                         const void *zp, const void *sc, const void *alpha, const void *beta,
                         const void *tgt,
-                        int B, int Hq, int H, int T, int D, int n_super_cap,
+                        int B, int Hq, int H, int T, int D, int n_super_cap, int bits,
                         void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
                         void *stream);
 int64_t adkv_forward_ov_gqa_workspace_bytes(int B, int Hq, int H, int T, int D, int n_ckpt_cap,
@@ -170,7 +176,7 @@ int64_t adkv_forward_ov_gqa_workspace_bytes(int B, int Hq, int H, int T, int D, 
 int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void *out,
                         const void *zp, const void *sc, const void *alpha, const void *beta,
                         const void *tgt,
-                        int B, int Hq, int H, int T, int D, int n_super_cap,
+                        int B, int Hq, int H, int T, int D, int n_super_cap, int bits,
                         void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
                         void *workspace, int64_t workspace_bytes, void *stream);
 
@@ -191,7 +197,7 @@ int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k
                       const void *v_new, const void *const *k_params, const void *const *v_params,
                       const void *mask, int rows_per_mask_row, float scaling,
                       void *out, void *weights_out,
-                      int B, int Hq, int H, int T, int D, int n_super_cap,
+                      int B, int Hq, int H, int T, int D, int n_super_cap, int bits,
                       void *k_ckpt, void *v_ckpt, int n_ckpt_cap, int ckpt_interval,
                       void *workspace, int64_t workspace_bytes, void *stream);
 

@@ -29,8 +29,8 @@ def _np16(t: torch.Tensor) -> np.ndarray:
     return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.float16)
 
 
-def _inputs(B, H, T, D, seed=0):
-    p = synth.make_params(H, D, seed=3 + seed)
+def _inputs(B, H, T, D, seed=0, bits=4):
+    p = synth.make_params(H, D, bits=bits, seed=3 + seed)
     # spread the parameters more than the benchmark does, to exercise the recurrence
     g = torch.Generator().manual_seed(100 + seed)
     p.zp_init = (0.3 * torch.randn(H, D, generator=g)).half()
@@ -420,47 +420,50 @@ def test_decode_fused_equals_three_calls(gpu, B, H, T, D, S, masked):
 
 
 # ------------------------------------------------------------------ grouped-query / matrix-core kernels
-def _gqa_case(gpu, oracle, B, Hkv, G, T, S, seed=0):
+def _gqa_case(gpu, oracle, B, Hkv, G, T, S, seed=0, bits=4):
     """One QK + OV pass with G query heads per KV head against the oracle run once per group member
     on a copy of the same cache (query head j reads KV head j // G)."""
     D = 128
     Hq = Hkv * G
-    x, p = _inputs(B, Hkv, T + 1, D, seed=seed)
+    tps = 32 // bits
+    x, p = _inputs(B, Hkv, T + 1, D, seed=seed, bits=bits)
     pn = [_np16(t) for t in p.astuple()]
     pg = [t.to(gpu) for t in p.astuple()]
     g = torch.Generator().manual_seed(50 + seed)
     q = torch.randn(B, Hq, 1, D, generator=g).half()
     attn = torch.softmax(2.0 * torch.randn(B, Hq, T + 1, generator=g), dim=-1).half()
-    cache0 = oracle.alloc_cache(B, Hkv, T + 8, D)
-    if T:
-        oracle.encode_kv_f16(cache0, _np16(x)[:, :, :T], *pn)
-    ncap = (T + 8) // S + 1 if S else 0
-    ck = None
-    if S:
-        ck = torch.from_numpy(_oracle_ckpts(oracle, cache0, pn, T, S, ncap).view(np.int16)).view(torch.float16).to(gpu)
     xn = _np16(x)[:, :, T:T + 1]
     want_l = np.zeros((B, Hq, T + 1))
     want_o = np.zeros((B, Hq, D))
     qn, an = _np16(q).reshape(B, Hkv, G, D), _np16(attn).reshape(B, Hkv, G, T + 1)
-    for j in range(G):
-        c = cache0.copy()
-        l, _ = oracle.forward_qk_f16(qn[:, :, j], c, xn, *pn, T)
-        want_l.reshape(B, Hkv, G, T + 1)[:, :, j] = l
-        c2 = cache0.copy()
-        o, _ = oracle.forward_ov_f16(an[:, :, j], c2, xn, *pn)
-        want_o.reshape(B, Hkv, G, D)[:, :, j] = o
+    ncap = (T + tps) // S + 1 if S else 0
+    ck = None
+    with oracle.code_bits(bits):
+        cache0 = oracle.alloc_cache(B, Hkv, T + tps, D)
+        if T:
+            oracle.encode_kv_f16(cache0, _np16(x)[:, :, :T], *pn)
+        if S:
+            ck = torch.from_numpy(_oracle_ckpts(oracle, cache0, pn, T, S, ncap).view(np.int16)) \
+                .view(torch.float16).to(gpu)
+        for j in range(G):
+            c = cache0.copy()
+            l, _ = oracle.forward_qk_f16(qn[:, :, j], c, xn, *pn, T)
+            want_l.reshape(B, Hkv, G, T + 1)[:, :, j] = l
+            c2 = cache0.copy()
+            o, _ = oracle.forward_ov_f16(an[:, :, j], c2, xn, *pn)
+            want_o.reshape(B, Hkv, G, D)[:, :, j] = o
+        _, st_want = oracle.replay_f16(cache0, *pn, T, want_khat=False)
     kc = torch.from_numpy(cache0.copy()).to(gpu)
     vc = torch.from_numpy(cache0.copy()).to(gpu)
     ckv = ck.clone() if ck is not None else None
     st_k = torch.zeros(B, Hkv, D, 2, dtype=torch.float16, device=gpu)
     logits = gemv.forward_qk(q.to(gpu), kc, x[:, :, T:T + 1].to(gpu), *pg, T, SMIN, SMAX,
-                             state_out=st_k, ckpt=ck, ckpt_interval=S)
+                             state_out=st_k, ckpt=ck, ckpt_interval=S, bits=bits)
     out = gemv.forward_ov(attn.to(gpu), vc, x[:, :, T:T + 1].to(gpu), *pg, SMIN, SMAX,
-                          ckpt=ckv, ckpt_interval=S)
+                          ckpt=ckv, ckpt_interval=S, bits=bits)
     torch.cuda.synchronize()
     assert logits.shape == (B, Hq, T + 1) and out.shape == (B, Hq, D)
     assert np.array_equal(kc.cpu().numpy(), c) and np.array_equal(vc.cpu().numpy(), c2)
-    _, st_want = oracle.replay_f16(cache0, *pn, T, want_khat=False)
     assert np.array_equal(st_k.cpu().view(torch.int16).numpy().view(np.uint16), st_want)
     lg, og = _np16(logits).astype(np.float64), _np16(out).astype(np.float64)
     assert np.all(np.abs(lg - want_l) <= _ulp16(want_l) + 1e-3), np.abs(lg - want_l).max()
@@ -486,3 +489,53 @@ def test_matrix_core_kernels_for_equal_heads(gpu, oracle, B, H, T, S):
         _gqa_case(gpu, oracle, B, H, 1, T, S, seed=3)
     finally:
         _lib.lib().adkv_set_mha_kernel(-1)
+
+
+# ------------------------------------------------------------------ 2-bit codes
+@pytest.mark.parametrize("B,H,T", [(1, 2, 1), (2, 3, 15), (2, 3, 16), (1, 5, 17), (1, 4, 100), (2, 2, 1024)])
+def test_encode_2bit_bit_exact(gpu, oracle, B, H, T):
+    """2-bit prompt quantisation (append from token 0): codes and final state equal the oracle's."""
+    D = 128
+    x, p = _inputs(B, H, T, D, seed=T % 5, bits=2)
+    pn = [_np16(t) for t in p.astuple()]
+    with oracle.code_bits(2):
+        want = oracle.alloc_cache(B, H, T + 16, D)
+        st_want = oracle.encode_kv_f16(want, _np16(x), *pn)
+    cache = synth.alloc_cache(B, H, T + 16, D, gpu, bits=2)
+    assert cache.shape == want.shape
+    st = torch.zeros(B, H, D, 2, dtype=torch.float16, device=gpu)
+    gemv.append_kv(cache, x.to(gpu), *[t.to(gpu) for t in p.astuple()], 0, st, bits=2)
+    torch.cuda.synchronize()
+    assert np.array_equal(cache.cpu().numpy(), want)
+    assert np.array_equal(st.cpu().view(torch.int16).numpy().view(np.uint16), st_want)
+
+
+@pytest.mark.parametrize("cuts,S", [((0, 5, 16, 17, 40, 41, 90), 0), ((0, 33, 34, 64, 150), 32)])
+def test_streaming_append_2bit(gpu, oracle, cuts, S):
+    B, H, D = 2, 2, 128
+    T = cuts[-1]
+    x, p = _inputs(B, H, T, D, seed=2, bits=2)
+    pn = [_np16(t) for t in p.astuple()]
+    pg = [t.to(gpu) for t in p.astuple()]
+    ncap = T // S + 1 if S else 0
+    with oracle.code_bits(2):
+        want = oracle.alloc_cache(B, H, T + 16, D)
+        st_want = oracle.encode_kv_f16(want, _np16(x), *pn)
+        ck_want = _oracle_ckpts(oracle, want, pn, T, S, ncap) if S else None
+    cache = synth.alloc_cache(B, H, T + 16, D, gpu, bits=2)
+    st = torch.zeros(B, H, D, 2, dtype=torch.float16, device=gpu)
+    ck = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=gpu) if S else None
+    for a, b in zip(cuts[:-1], cuts[1:]):
+        gemv.append_kv(cache, x[:, :, a:b].to(gpu), *pg, a, st, ckpt=ck, ckpt_interval=S, bits=2)
+    torch.cuda.synchronize()
+    assert np.array_equal(cache.cpu().numpy(), want)
+    assert np.array_equal(st.cpu().view(torch.int16).numpy().view(np.uint16), st_want)
+    if S:
+        assert np.array_equal(ck.cpu().view(torch.int16).numpy().view(np.uint16), ck_want)
+
+
+@pytest.mark.parametrize("B,Hkv,G,T,S", [
+    (1, 2, 1, 0, 0), (2, 2, 1, 7, 0), (1, 3, 1, 16, 0), (2, 2, 4, 9, 0), (1, 2, 4, 31, 0), (2, 3, 4, 77, 0),
+    (1, 2, 8, 40, 0), (2, 3, 4, 530, 64), (1, 2, 2, 256, 64), (1, 1, 1, 200, 16), (1, 5, 4, 1033, 0)])
+def test_decode_kernels_2bit(gpu, oracle, B, Hkv, G, T, S):
+    _gqa_case(gpu, oracle, B, Hkv, G, T, S, seed=T % 7, bits=2)
