@@ -50,7 +50,12 @@ def _workspace(dev: torch.device, need: int) -> torch.Tensor:
 class KVCacheLayer_ADKV:
     """Quantised K/V store of one attention layer."""
 
-    def __init__(self):
+    def __init__(self, bits: int = 4):
+        if bits not in (2, 4):
+            raise ValueError("ADKV code width must be 2 or 4 bits")
+        # 4 = the reference's format; 2 = the same recurrence over codes in [-2, 1], 16 tokens per
+        # supergroup (head_dim 128 only), an extension the reference does not have
+        self._bits = bits
         self._key_buf: torch.Tensor | None = None
         self._value_buf: torch.Tensor | None = None
         self._key_ckpt: torch.Tensor | None = None
@@ -88,9 +93,8 @@ class KVCacheLayer_ADKV:
         return self._value_buf
 
     # ------------------------------------------------------------------ storage
-    @staticmethod
-    def _n_super(tokens: int) -> int:
-        return -(-tokens // 8)
+    def _n_super(self, tokens: int) -> int:
+        return -(-tokens // (32 // self._bits))
 
     def _n_ckpt(self, cap_tokens: int) -> int:
         return cap_tokens // self._ckpt_interval + 1 if self._ckpt_interval else 0
@@ -99,14 +103,16 @@ class KVCacheLayer_ADKV:
         ns = self._n_super(cap_tokens)
         shape = (self._B, self._H, ns, self._C // 4, 4, 4)
         mk = lambda: torch.zeros(shape, dtype=torch.uint8, device=self._device)
-        ck = (lambda: torch.zeros((self._B, self._H, self._n_ckpt(ns * 8), self._C, 2),
+        ck = (lambda: torch.zeros((self._B, self._H, self._n_ckpt(ns * (32 // self._bits)), self._C, 2),
                                   dtype=torch.float16, device=self._device)) \
             if self._ckpt_interval else (lambda: None)
-        return ns * 8, mk(), mk(), ck(), ck()
+        return ns * (32 // self._bits), mk(), mk(), ck(), ck()
 
     def _init_buffers(self, B: int, H: int, C: int, device: torch.device):
         if C not in _HEAD_DIMS:
             raise ValueError(f"ADKV kernels support head_dim in (128, 256, 512), got {C}")
+        if self._bits == 2 and C != 128:
+            raise ValueError("2-bit ADKV codes need head_dim 128")
         self._B, self._H, self._C, self._device = B, H, C, device
         self._quant_len = 0
         (self._cap_len, self._key_buf, self._value_buf,
@@ -149,11 +155,12 @@ class KVCacheLayer_ADKV:
         S = self._ckpt_interval
         append_kv(self._key_buf, key_states.to(torch.float16).contiguous(),
                   v(key_zp_init), v(key_scale_init), v(key_alpha), v(key_beta), v(key_quant_target),
-                  self._quant_len, self._key_state, ckpt=self._key_ckpt, ckpt_interval=S)
+                  self._quant_len, self._key_state, ckpt=self._key_ckpt, ckpt_interval=S, bits=self._bits)
         append_kv(self._value_buf, value_states.to(torch.float16).contiguous(),
                   v(value_zp_init), v(value_scale_init), v(value_alpha), v(value_beta),
                   v(value_quant_target),
-                  self._quant_len, self._value_state, ckpt=self._value_ckpt, ckpt_interval=S)
+                  self._quant_len, self._value_state, ckpt=self._value_ckpt, ckpt_interval=S,
+                  bits=self._bits)
         self._quant_len += key_states.shape[2]
 
     def prefill(self, key_states, value_states,
@@ -210,7 +217,8 @@ class KVCacheLayer_ADKV:
             (v(value_zp_init), v(value_scale_init), v(value_alpha), v(value_beta),
              v(value_quant_target)),
             ctx, scaling, attention_mask,
-            k_ckpt=self._key_ckpt, v_ckpt=self._value_ckpt, ckpt_interval=S, workspace=ws)
+            k_ckpt=self._key_ckpt, v_ckpt=self._value_ckpt, ckpt_interval=S, bits=self._bits,
+            workspace=ws)
         self._quant_len = ctx + 1
         self._state_valid = False
         return out.to(query_states.dtype), weights
@@ -224,7 +232,7 @@ class KVCacheLayer_ADKV:
             return {"quant_len": 0}
         ns = self._n_super(self._quant_len)
         nck = self._quant_len // self._ckpt_interval if self._ckpt_interval else 0
-        sd = {"quant_len": self._quant_len, "ckpt_interval": self._ckpt_interval,
+        sd = {"quant_len": self._quant_len, "ckpt_interval": self._ckpt_interval, "bits": self._bits,
               "geometry": (self._B, self._H, self._C),
               "key_codes": self._key_buf[:, :, :ns].contiguous(),
               "value_codes": self._value_buf[:, :, :ns].contiguous()}
@@ -239,8 +247,9 @@ class KVCacheLayer_ADKV:
         """Rebuild the layer from ``state_dict()`` output on ``device`` (default: where the saved
         tensors live).  Slots past the saved tokens are zero, as the append kernels expect."""
         if sd.get("quant_len", 0) == 0 and "key_codes" not in sd:
-            self.__init__()
+            self.__init__(self._bits)
             return
+        self._bits = int(sd.get("bits", 4))
         B, H, C = sd["geometry"]
         dev = torch.device(device) if device is not None else sd["key_codes"].device
         T = int(sd["quant_len"])
@@ -274,8 +283,8 @@ class KVCacheLayer_ADKV:
 class KVCache_ADKV(list):
     """One ``KVCacheLayer_ADKV`` per decoder layer (reference llama_adkv.py:279-288)."""
 
-    def __init__(self, num_layers: int):
-        super().__init__(KVCacheLayer_ADKV() for _ in range(num_layers))
+    def __init__(self, num_layers: int, bits: int = 4):
+        super().__init__(KVCacheLayer_ADKV(bits) for _ in range(num_layers))
 
     def get_seq_length(self, layer_idx: int = 0) -> int:
         return self[layer_idx].get_seq_length()

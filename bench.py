@@ -42,6 +42,8 @@ def parse():
     ap.add_argument("--kv-heads", type=int, default=0,
                     help="KV heads when fewer than --heads query heads share them (grouped-query "
                          "attention); default: as many as --heads")
+    ap.add_argument("--bits", type=int, default=4, choices=[2, 4],
+                    help="code width of the decode workload (2 needs --dim 128)")
     ap.add_argument("--dim", type=int, default=128)
     ap.add_argument("--ctx", type=int, default=4096)
     ap.add_argument("--layer-buffers", type=int, default=4,
@@ -187,7 +189,7 @@ def encode_main(args):
         "data": "synthetic",
         "config": {"workload": f"cfg3 streaming quantise: prefill B={B} H={H} d={D} ctx={T} fp16 -> 4-bit codes, "
                                f"then {n_app} single-token appends with carried state",
-                   "batch": B, "heads": Hq, "kv_heads": H, "head_dim": D, "ctx": T, "bits": 4, "ckpt_interval": S},
+                   "batch": B, "heads": H, "head_dim": D, "ctx": T, "bits": 4, "ckpt_interval": S},
         "append_us_per_token_step": append_us,
         "codes_bit_exact_vs_oracle": exact,
         "roofline": {"kernel": "encode_kernel", "bound": "hbm", "achieved": achieved,
@@ -229,20 +231,22 @@ def main():
     NL = args.layer_buffers
 
     S = args.ckpt_interval
+    bits = args.bits
     ncap = T // S + 1 if S else 0
     kps, vps, kcs, vcs, kks, vks = [], [], [], [], [], []
+    state = torch.zeros(B, H, D, 2, dtype=torch.float16, device=dev)
     for l in range(NL):
-        kp = synth.make_params(H, D, seed=3, layer=l).to(dev)
-        vp = synth.make_params(H, D, seed=4, layer=l).to(dev)
-        kc = synth.alloc_cache(B, H, T + 8, D, dev)
-        vc = synth.alloc_cache(B, H, T + 8, D, dev)
+        kp = synth.make_params(H, D, bits=bits, seed=3, layer=l).to(dev)
+        vp = synth.make_params(H, D, bits=bits, seed=4, layer=l).to(dev)
+        kc = synth.alloc_cache(B, H, T + 16, D, dev, bits=bits)
+        vc = synth.alloc_cache(B, H, T + 16, D, dev, bits=bits)
         kk = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=dev) if S else None
         vk = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=dev) if S else None
         x = synth.make_k(B, H, T, D, layer=l, dtype=torch.float16, device=dev)
-        gemv.encode_kv(kc, x, *kp.astuple(), smin, smax, ckpt=kk, ckpt_interval=S)
+        gemv.append_kv(kc, x, *kp.astuple(), 0, state, ckpt=kk, ckpt_interval=S, bits=bits)
         del x
         x = synth.make_v(B, H, T, D, layer=l, dtype=torch.float16, device=dev)
-        gemv.encode_kv(vc, x, *vp.astuple(), smin, smax, ckpt=vk, ckpt_interval=S)
+        gemv.append_kv(vc, x, *vp.astuple(), 0, state, ckpt=vk, ckpt_interval=S, bits=bits)
         del x
         kps.append(kp.astuple()); vps.append(vp.astuple()); kcs.append(kc); vcs.append(vc)
         kks.append(kk); vks.append(vk)
@@ -269,13 +273,15 @@ def main():
         if timed:
             e = [ev() for _ in range(4)]
             e[0].record()
-        logits = gemv.forward_qk(q, kcs[l], k_new, *kps[l], T, smin, smax, ckpt=kks[l], ckpt_interval=S)
+        logits = gemv.forward_qk(q, kcs[l], k_new, *kps[l], T, smin, smax, ckpt=kks[l], ckpt_interval=S,
+                                 bits=bits)
         if timed:
             e[1].record()
         w = gemv.softmax_scale_mask(logits, scaling)
         if timed:
             e[2].record()
-        out = gemv.forward_ov(w, vcs[l], v_new, *vps[l], smin, smax, ckpt=vks[l], ckpt_interval=S)
+        out = gemv.forward_ov(w, vcs[l], v_new, *vps[l], smin, smax, ckpt=vks[l], ckpt_interval=S,
+                              bits=bits)
         if timed:
             e[3].record()
             marks.append(e)
@@ -296,7 +302,7 @@ def main():
     ov_ms = sum(e[2].elapsed_time(e[3]) for e in marks) / len(marks)
     dev_ms = sorted(e[0].elapsed_time(e[3]) for e in marks)[len(marks) // 2]
 
-    code_bytes = B * H * T * D * 0.5                    # one tensor's codes: bytes per QK launch
+    code_bytes = B * H * T * D * bits / 8.0             # one tensor's codes: bytes per QK launch
     achieved = code_bytes / (qk_ms * 1e-3) / 1e9
     tokens_s = B / (N_LAYERS_MODEL * ms_step * 1e-3)
 
@@ -316,16 +322,16 @@ def main():
         "config": {
             "workload": f"{'cfg2 Llama-2-7B-shaped' if H == Hq else 'grouped-query'} ADKV decode attention: "
                         f"B={B} H={Hq}{'' if H == Hq else f' (KV heads {H})'} d={D} ctx={T} "
-                        f"4-bit K+V codes, step = forward_qk+softmax+forward_ov, {NL} rotating layer caches, "
+                        f"{bits}-bit K+V codes, step = forward_qk+softmax+forward_ov, {NL} rotating layer caches, "
                         f"state checkpoints every {S} tokens",
-            "batch": B, "heads": Hq, "kv_heads": H, "head_dim": D, "ctx": T, "bits": 4, "ckpt_interval": S,
+            "batch": B, "heads": Hq, "kv_heads": H, "head_dim": D, "ctx": T, "bits": bits, "ckpt_interval": S,
             "parallelism": "1 GPU",
         },
         "kernel_ms": {"forward_qk": qk_ms, "softmax": sm_ms, "forward_ov": ov_ms,
                       "step_device_median": dev_ms},
         "step_code_GBps": 2 * code_bytes / (ms_step * 1e-3) / 1e9,
         "roofline": {
-            "kernel": "qk_kernel",
+            "kernel": "qk_kernel" if (H == Hq and bits == 4) else "qk_gqa_kernel",
             "bound": "hbm",
             "achieved": achieved,
             "peak": HBM_PEAK_GBPS,
@@ -333,12 +339,12 @@ def main():
             "frac": achieved / HBM_PEAK_GBPS,
             # HBM bytes per QK launch from rocprofv3 FETCH_SIZE/WRITE_SIZE scaled by a 1 GiB copy
             # (profiles/decode_cfg2_pmc_traffic.md); measured for the default workload only
-            "traffic": 1.1227e9 if (B, H, D, T, S) == (128, 32, 128, 4096, 256) else None,
+            "traffic": 1.1227e9 if (B, Hq, H, D, T, S, bits) == (128, 32, 32, 128, 4096, 256, 4) else None,
         },
     }
-    if not args.no_fp16_comparator and D == 128 and H == Hq:
+    if not args.no_fp16_comparator and D == 128 and H == Hq and bits == 4:
         res["fp16_kv_comparator"] = fp16_comparator(args, dev, ms_step)
-    if not args.no_cpu_baseline and H == Hq:
+    if not args.no_cpu_baseline and H == Hq and bits == 4:
         res["cpu_baseline"] = cpu_baseline(args, T, D)
     print(json.dumps(res))
 

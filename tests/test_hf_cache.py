@@ -36,7 +36,8 @@ def test_cache_storage_management_cpu():
     c._cap_buffers(1000)
     assert c._cap_len == 1024 and c._key_ckpt.shape[2] == 1024 // C.CKPT_INTERVAL + 1
     assert c.get_mask_sizes(torch.arange(3)) == (3, 0)
-    assert KVCacheLayer_ADKV._n_super(0) == 0 and KVCacheLayer_ADKV._n_super(9) == 2
+    assert KVCacheLayer_ADKV()._n_super(0) == 0 and KVCacheLayer_ADKV()._n_super(9) == 2
+    assert KVCacheLayer_ADKV(bits=2)._n_super(17) == 2
 
 
 def test_cache_errors_cpu():
@@ -185,7 +186,7 @@ def test_cache_save_and_restore_continues_identically(gpu, tmp_path, monkeypatch
         o2, w2 = step(again[0], t)
         assert torch.equal(o1.view(torch.int16), o2.view(torch.int16))
         assert torch.equal(w1.view(torch.int16), w2.view(torch.int16))
-    n = C.KVCacheLayer_ADKV._n_super(T0 + 30)
+    n = cache[0]._n_super(T0 + 30)
     assert torch.equal(cache[0].key_states[:, :, :n], again[0].key_states[:, :, :n])
     assert torch.equal(cache[0].value_states[:, :, :n], again[0].value_states[:, :, :n])
     with pytest.raises(NotImplementedError):
@@ -196,6 +197,50 @@ def test_cache_save_and_restore_continues_identically(gpu, tmp_path, monkeypatch
     chunked[0].prefill(k[:, :, T0:T0 + 9], v[:, :, T0:T0 + 9], *kg, *vg)
     whole = KVCacheLayer_ADKV()
     whole.prefill(k[:, :, :T0 + 9], v[:, :, :T0 + 9], *kg, *vg)
-    n = C.KVCacheLayer_ADKV._n_super(T0 + 9)
+    n = whole._n_super(T0 + 9)
     assert torch.equal(chunked[0].key_states[:, :, :n], whole.key_states[:, :, :n])
     assert torch.equal(chunked[0].value_states[:, :, :n], whole.value_states[:, :, :n])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("bits,G,dtype", [(2, 1, torch.float16), (4, 4, torch.bfloat16), (2, 4, torch.bfloat16)])
+def test_cache_layer_grouped_queries_two_bit_and_bf16(gpu, oracle, bits, G, dtype):
+    """The cache object with 2-bit codes, 4 query heads per KV head and bf16 activations: prompt in
+    two chunks, then steps across a capacity growth; codes bit-exact, outputs within 2e-3 of the
+    oracle evaluated per query head (query head j reads KV head j // G)."""
+    B, H, D, T0, steps = 2, 2, 128, 45, 25
+    Hq = H * G
+    kp, vp = synth.make_params(H, D, bits=bits, seed=3), synth.make_params(H, D, bits=bits, seed=4)
+    k = synth.make_k(B, H, T0 + steps, D, dtype=torch.float16)
+    v = synth.make_v(B, H, T0 + steps, D, dtype=torch.float16)
+    if dtype == torch.bfloat16:          # values a bf16 model would hand over: exact in fp16 as well
+        k, v = k.to(dtype).to(torch.float16), v.to(dtype).to(torch.float16)
+    gq = torch.Generator().manual_seed(2)
+    scaling = D ** -0.5
+    kpn, vpn = [_np16(t) for t in kp.astuple()], [_np16(t) for t in vp.astuple()]
+    layer = KVCacheLayer_ADKV(bits=bits)
+    kg, vg = _flat(kp.to(gpu)), _flat(vp.to(gpu))
+    layer.prefill(k[:, :, :19].to(gpu).to(dtype), v[:, :, :19].to(gpu).to(dtype), *kg, *vg)
+    layer.prefill(k[:, :, 19:T0].to(gpu).to(dtype), v[:, :, 19:T0].to(gpu).to(dtype), *kg, *vg)
+    with oracle.code_bits(bits):
+        ko, vo = oracle.alloc_cache(B, H, T0 + steps + 16, D), oracle.alloc_cache(B, H, T0 + steps + 16, D)
+        oracle.encode_kv_f16(ko, _np16(k)[:, :, :T0], *kpn)
+        oracle.encode_kv_f16(vo, _np16(v)[:, :, :T0], *vpn)
+        for s in range(steps):
+            T = T0 + s
+            q = torch.randn(B, Hq, 1, D, generator=gq).to(dtype)
+            out, w = layer.decode(q.to(gpu), k[:, :, T:T + 1].to(gpu).to(dtype), v[:, :, T:T + 1].to(gpu).to(dtype),
+                                  *kg, *vg, scaling=scaling)
+            assert out.dtype == dtype and out.shape == (B, Hq, D) and w.shape == (B, Hq, T + 1)
+            qn = _np16(q.to(torch.float16)).reshape(B, H, G, D)
+            got = out.float().cpu().numpy().reshape(B, H, G, D)
+            for j in range(G):
+                kc, vc = ko.copy(), vo.copy()
+                want, _, _ = oracle.decode_step_f16(qn[:, :, j], kc, vc, _np16(k)[:, :, T:T + 1],
+                                                    _np16(v)[:, :, T:T + 1], kpn, vpn, T, scaling)
+                tol = 2e-3 if dtype == torch.float16 else 2e-3 + 2.0 ** -8 * np.abs(want)
+                assert np.all(np.abs(got[:, :, j] - want) <= tol), (s, j)
+            ko, vo = kc, vc
+        n = oracle.n_super(T0 + steps)
+    assert np.array_equal(layer.key_states.cpu().numpy()[:, :, :n], ko[:, :, :n])
+    assert np.array_equal(layer.value_states.cpu().numpy()[:, :, :n], vo[:, :, :n])
