@@ -13,7 +13,7 @@ import torch  # noqa: F401  (loads libamdhip64 first)
 
 _DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_DIR, "libadkv_hip.so")
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _vp, _i, _f = C.c_void_p, C.c_int, C.c_float
 
@@ -28,17 +28,18 @@ PROTOTYPES = {
     "adkv_forward_ov": (_i, [_vp] * 9 + [_i] * 5 + [_f, _f, _vp, _vp]),
     "adkv_softmax": (_i, [_vp] * 3 + [_i] * 3 + [_f, _vp]),
     "adkv_softmax_workspace_bytes": (C.c_int64, [_i, _i]),
-    "adkv_softmax_ex": (_i, [_vp] * 3 + [_i] * 3 + [_f, _vp, C.c_int64, _vp]),
+    "adkv_row_pitch": (C.c_int64, [_i]),
+    "adkv_softmax_ex": (_i, [_vp] * 3 + [_i, _i, C.c_int64, _i, _f, _vp, C.c_int64, _vp]),
     "adkv_encode_kv_ex": (_i, [_vp] * 7 + [_i] * 5 + [_vp, _vp, _i, _i, _vp]),
     "adkv_append_kv": (_i, [_vp] * 7 + [_i] * 7 + [_vp, _vp, _i, _i, _vp]),
     "adkv_forward_qk_ex": (_i, [_vp] * 9 + [_i] * 5 + [_vp, _vp, _i, _i, _vp]),
     "adkv_forward_ov_workspace_bytes": (C.c_int64, [_i] * 6),
     "adkv_forward_ov_ex": (_i, [_vp] * 9 + [_i] * 5 + [_vp, _vp, _i, _i, _vp, C.c_int64, _vp]),
-    "adkv_forward_qk_gqa": (_i, [_vp] * 9 + [_i] * 7 + [_vp, _vp, _i, _i, _vp]),
+    "adkv_forward_qk_gqa": (_i, [_vp] * 9 + [_i] * 7 + [C.c_int64, _vp, _vp, _i, _i, _vp]),
     "adkv_forward_ov_gqa_workspace_bytes": (C.c_int64, [_i] * 7),
-    "adkv_forward_ov_gqa": (_i, [_vp] * 9 + [_i] * 7 + [_vp, _vp, _i, _i, _vp, C.c_int64, _vp]),
+    "adkv_forward_ov_gqa": (_i, [_vp] * 9 + [_i] * 7 + [C.c_int64, _vp, _vp, _i, _i, _vp, C.c_int64, _vp]),
     "adkv_decode_fused_workspace_bytes": (C.c_int64, [_i] * 7),
-    "adkv_decode_fused": (_i, [_vp] * 8 + [_i, _f, _vp, _vp] + [_i] * 7 + [_vp, _vp, _i, _i, _vp,
+    "adkv_decode_fused": (_i, [_vp] * 8 + [_i, _f, _vp, _vp, C.c_int64] + [_i] * 7 + [_vp, _vp, _i, _i, _vp,
                                                                             C.c_int64, _vp]),
     "adkv_quant_f32": (_i, [_vp] * 12 + [_i] * 3 + [C.c_int64, C.c_int64] + [_i] * 3 + [_f, _f, _vp]),
     "adkv_fp16_decode_workspace_bytes": (C.c_int64, [_i] * 3),

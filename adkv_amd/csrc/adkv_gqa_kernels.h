@@ -1,6 +1,6 @@
 // Decode kernels for head dim 128 that put the contraction on the matrix cores, for GQ >= 1 query
-// heads per KV head and for 4-bit or 2-bit codes.  Included inside namespace adkv by
-// adkv_kernels.hip.
+// heads per KV head and for 4-bit or 2-bit codes.  Included by adkv_kernels.hip after
+// the shared device helpers.
 //
 // The fp16 replay of the filter state (the dominant cost) is the same per-lane arithmetic as in
 // qk_kernel / ov_kernel and runs once per KV head; only what happens to the dequantised value
@@ -22,6 +22,8 @@
 // 2-bit codes (16 tokens per channel word).  Table lookups for the next unit are issued between
 // the tokens of the current one, into the register slots they vacate.
 #pragma once
+
+namespace adkv {
 
 typedef float f4v __attribute__((ext_vector_type(4)));
 typedef _Float16 h4v __attribute__((ext_vector_type(4)));
@@ -138,6 +140,8 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
     constexpr int D = GQA_D, CPL = GQA_CPL;
     constexpr int NB = (GQ + 3) / 4; // column sets of four heads
     constexpr int TPW = Code<BITS>::TPW, UPS = TPW / 8;
+    // supergroups in flight per lane: fewer where a supergroup is 16 tokens or registers are short
+    constexpr int GPF = (BITS == 2 || NB > 1) ? 2 : PF;
     using G = Geo<D, CPL>;
     __shared__ uint2 smem[LUT_WORDS64 + (BLK / 64) * TILE_WORDS64];
     const uint2 *lut = smem;
@@ -203,7 +207,7 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
             const float mine = qd == 0 ? s[0] : qd == 1 ? s[1] : qd == 2 ? s[2] : s[3];
             const int tok = tg4 * 4 + qd, g = 4 * n + r;
             if (active && g < GQ && tok < ntok)
-                out[((size_t)bx * GQ + g) * (T + 1) + t0 + unit * 8 + tok] = (h1)mine;
+                out[((size_t)bx * GQ + g) * sa.row_pitch + t0 + unit * 8 + tok] = (h1)mine;
         }
     };
 
@@ -225,25 +229,25 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    uint4 buf[PF];
+    uint4 buf[GPF];
     uint32_t nbc[G::NP][2], nbn[G::NP][2]; // byte streams of the current / the next supergroup
     uint2 areg[8];
 #pragma unroll
-    for (int i = 0; i < PF; i++)
+    for (int i = 0; i < GPF; i++)
         buf[i] = (i < nfull) ? cb[(size_t)i * G::VPS] : make_uint4(0, 0, 0, 0);
     if (nfull > 0) {
         code_bytes<BITS>(buf[0], nbc);
         lk.fill(lut, nbc, lane_copy, 0);
     }
-    for (int sg0 = 0; sg0 < nfull; sg0 += PF) {
+    for (int sg0 = 0; sg0 < nfull; sg0 += GPF) {
 #pragma unroll
-        for (int i = 0; i < PF; i++) {
+        for (int i = 0; i < GPF; i++) {
             const int sg = sg0 + i;
             if (sg < nfull) {
                 // bytes of supergroup sg+1 (stale data past the end: looked up, never used)
-                code_bytes<BITS>(buf[(i + 1) % PF], nbn);
-                if (sg + PF < nfull)
-                    buf[i] = cb[(size_t)(sg + PF) * G::VPS];
+                code_bytes<BITS>(buf[(i + 1) % GPF], nbn);
+                if (sg + GPF < nfull)
+                    buf[i] = cb[(size_t)(sg + GPF) * G::VPS];
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int hf = 0; hf < UPS; hf++) {
@@ -322,8 +326,9 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
     constexpr int D = GQA_D, CPL = GQA_CPL;
     constexpr int NB = (GQ + 3) / 4;
     constexpr int TPW = Code<BITS>::TPW, UPS = TPW / 8;
-    constexpr int WPF = 4; // weight vectors (8 tokens each) in flight
-    static_assert((PF * UPS) % WPF == 0, "weight ring must line up with the unrolled loop");
+    constexpr int GPF = (BITS == 2 || NB > 1) ? 2 : PF;    // supergroups in flight per lane
+    constexpr int WPF = 2;                                 // weight vectors (8 tokens each) in flight
+    static_assert((GPF * UPS) % WPF == 0, "weight ring must line up with the unrolled loop");
     using G = Geo<D, CPL>;
     __shared__ uint2 lut[LUT_WORDS64];
     fill_table<BITS>(lut, threadIdx.x, BLK);
@@ -359,7 +364,7 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
 #pragma unroll
     for (int n = 0; n < NB; n++) {
         wok[n] = 4 * n + r < GQ;
-        wb[n] = attn + ((size_t)bx * GQ + (wok[n] ? 4 * n + r : 0)) * (T + 1) + t0;
+        wb[n] = attn + ((size_t)bx * GQ + (wok[n] ? 4 * n + r : 0)) * sa.row_pitch + t0;
     }
     auto load_w = [&](int n, int unit) {
         uint4 v;
@@ -401,11 +406,11 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    uint4 buf[PF];
+    uint4 buf[GPF];
     uint4 wbuf[WPF][NB];
     uint32_t nbc[G::NP][2], nbn[G::NP][2];
 #pragma unroll
-    for (int i = 0; i < PF; i++)
+    for (int i = 0; i < GPF; i++)
         buf[i] = (i < nfull) ? cb[(size_t)i * G::VPS] : make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int i = 0; i < WPF; i++)
@@ -416,14 +421,14 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
         code_bytes<BITS>(buf[0], nbc);
         lk.fill(lut, nbc, lane_copy, 0);
     }
-    for (int sg0 = 0; sg0 < nfull; sg0 += PF) {
+    for (int sg0 = 0; sg0 < nfull; sg0 += GPF) {
 #pragma unroll
-        for (int i = 0; i < PF; i++) {
+        for (int i = 0; i < GPF; i++) {
             const int sg = sg0 + i;
             if (sg < nfull) {
-                code_bytes<BITS>(buf[(i + 1) % PF], nbn);
-                if (sg + PF < nfull)
-                    buf[i] = cb[(size_t)(sg + PF) * G::VPS];
+                code_bytes<BITS>(buf[(i + 1) % GPF], nbn);
+                if (sg + GPF < nfull)
+                    buf[i] = cb[(size_t)(sg + GPF) * G::VPS];
 #pragma unroll
                 for (int hf = 0; hf < UPS; hf++) {
                     const int unit = sg * UPS + hf;
@@ -462,7 +467,7 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
         auto add_token = [&](const h2 *vd, int t) {
 #pragma unroll
             for (int g = 0; g < GQ; g++) {
-                const float wt = (float)attn[((size_t)bx * GQ + g) * (T + 1) + t];
+                const float wt = (float)attn[((size_t)bx * GQ + g) * sa.row_pitch + t];
 #pragma unroll
                 for (int p = 0; p < G::NP; p++) {
                     acc[g >> 2][2 * p][g & 3] = __builtin_fmaf(wt, (float)vd[p].x, acc[g >> 2][2 * p][g & 3]);
@@ -511,3 +516,5 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
         }
     }
 }
+
+} // namespace adkv

@@ -53,6 +53,7 @@ struct Seg {
     int ckpt_interval;  // 0 when ckpt is null
     int seg_tokens;     // >= T when there is one segment
     int nseg;
+    long row_pitch;     // elements between rows of the logits / attention-weight matrix (>= T + 1)
 };
 
 __device__ __forceinline__ float wave_xor_add(float v, int mask)
@@ -455,7 +456,7 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
     const int t1 = last ? T : t0 + sa.seg_tokens;
     uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV; // this head, this lane
     const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;                  // this segment
-    h1 *ob = out + (size_t)bx * (T + 1) + t0;
+    h1 *ob = out + (size_t)bx * sa.row_pitch + t0;
     const int nfull = (t1 - t0) >> 3;
     const int tk = lane & 7, g8 = lane >> 3;
 
@@ -599,7 +600,7 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
         self = __builtin_amdgcn_fdot2(qv[p], deq[p], self, false);
     self = head_allreduce<G::LPH>(self);
     if (active && lh == 0)
-        out[(size_t)bx * (T + 1) + T] = (h1)self;
+        out[(size_t)bx * sa.row_pitch + T] = (h1)self;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -640,7 +641,7 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
     const int t1 = last ? T : t0 + sa.seg_tokens;
     uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV;
     const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;
-    const h1 *wrow = attn + (size_t)bx * (T + 1);
+    const h1 *wrow = attn + (size_t)bx * sa.row_pitch;
     const h1 *wb = wrow + t0;
     const int nfull = (t1 - t0) >> 3;
 
@@ -801,12 +802,12 @@ __device__ __forceinline__ float block_reduce(float v, float *sm, bool is_max)
 
 __global__ __launch_bounds__(SM_BLOCK) void softmax_kernel(
     const h1 *__restrict__ logits, h1 *__restrict__ weights, const float *__restrict__ mask,
-    int n, int rows_per_mask_row, float scaling)
+    int n, long ld, int rows_per_mask_row, float scaling)
 {
     __shared__ float sm[SM_BLOCK / 64];
     const int row = blockIdx.x;
-    const h1 *l = logits + (size_t)row * n;
-    h1 *w = weights + (size_t)row * n;
+    const h1 *l = logits + (size_t)row * ld;
+    h1 *w = weights + (size_t)row * ld;
     const float *mk = mask ? mask + (size_t)(row / rows_per_mask_row) * n : nullptr;
 
     // rows up to SM_BLOCK*KEEP elements are read from memory once and kept in registers
@@ -895,11 +896,11 @@ __device__ __forceinline__ void softmax_load_chunk(const h1 *l, const float *mk,
 
 __global__ __launch_bounds__(SM_BLOCK) void softmax_part_kernel(
     const h1 *__restrict__ logits, const float *__restrict__ mask, float2 *__restrict__ part,
-    int n, int nchunk, int rows_per_mask_row, float scaling)
+    int n, long ld, int nchunk, int rows_per_mask_row, float scaling)
 {
     __shared__ float sm[SM_BLOCK / 64];
     const int row = blockIdx.y, ck = blockIdx.x;
-    const h1 *l = logits + (size_t)row * n;
+    const h1 *l = logits + (size_t)row * ld;
     const float *mk = mask ? mask + (size_t)(row / rows_per_mask_row) * n : nullptr;
     float x[SM_KEEP], mx;
     softmax_load_chunk(l, mk, n, ck * SM_CHUNK, scaling, x, mx);
@@ -917,11 +918,11 @@ __global__ __launch_bounds__(SM_BLOCK) void softmax_part_kernel(
 
 __global__ __launch_bounds__(SM_BLOCK) void softmax_norm_kernel(
     const h1 *__restrict__ logits, h1 *__restrict__ weights, const float *__restrict__ mask,
-    const float2 *__restrict__ part, int n, int nchunk, int rows_per_mask_row, float scaling)
+    const float2 *__restrict__ part, int n, long ld, int nchunk, int rows_per_mask_row, float scaling)
 {
     const int row = blockIdx.y, ck = blockIdx.x;
-    const h1 *l = logits + (size_t)row * n;
-    h1 *w = weights + (size_t)row * n;
+    const h1 *l = logits + (size_t)row * ld;
+    h1 *w = weights + (size_t)row * ld;
     const float *mk = mask ? mask + (size_t)(row / rows_per_mask_row) * n : nullptr;
     const float2 *pr = part + (size_t)row * nchunk;
     float M = -INFINITY;
@@ -991,6 +992,7 @@ static Seg plan_segments(void *ckpt, int n_ckpt_cap, int ckpt_interval, int BH, 
     s.ckpt_interval = ckpt ? ckpt_interval : 0;
     s.seg_tokens = T > 0 ? T : 1;
     s.nseg = 1;
+    s.row_pitch = T + 1;
     if (!ckpt || ckpt_interval <= 0 || T <= ckpt_interval)
         return s;
     const int avail = (T + ckpt_interval - 1) / ckpt_interval;               // finest split
@@ -1046,8 +1048,9 @@ static void launch_units(long threads, int big, F256 f256, FBIG fbig)
 #define ADKV_LAUNCH_GQA(KERNEL, BB, GQV, ...)                                                      \
     do {                                                                                            \
         const long threads = (long)BH * seg.nseg * 32;                                              \
-        if (threads >= 1024L * 256)                                                                 \
-            hipLaunchKernelGGL((KERNEL<BB, GQV, 1024>), dim3((unsigned)((threads + 1023) / 1024)),  \
+        /* eight heads per KV head need more registers than a 16-wave workgroup leaves a lane */   \
+        if (GQV <= 4 && threads >= 1024L * 256)                                                     \
+            hipLaunchKernelGGL((KERNEL<BB, (GQV <= 4 ? GQV : 1), 1024>), dim3((unsigned)((threads + 1023) / 1024)),  \
                                dim3(1024), 0, st, __VA_ARGS__);                                     \
         else                                                                                        \
             hipLaunchKernelGGL((KERNEL<BB, GQV, 512>), dim3((unsigned)((threads + 511) / 512)),     \
@@ -1097,7 +1100,7 @@ static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval, int b
 
 extern "C" {
 
-int adkv_abi_version(void) { return 6; }
+int adkv_abi_version(void) { return 7; }
 
 void adkv_set_mha_kernel(int use_matrix_cores) { g_mha_kernel = use_matrix_cores; }
 
@@ -1154,6 +1157,7 @@ static int encode_common(void *cache, const void *kv_new,
     seg.ckpt_interval = ckpt_out ? ckpt_interval : 0;
     seg.seg_tokens = T > 0 ? T : 1;
     seg.nseg = 1;
+    seg.row_pitch = T + 1;
     // widest lane that still leaves every SIMD with about two waves
     const long channels = (long)BH * D;
     int cpl = 4;
@@ -1230,10 +1234,12 @@ int adkv_encode_kv(void *cache, const void *kv_new,
 int adkv_forward_qk_gqa(const void *q, void *k_cache, const void *k_new, void *logits,
                         const void *zp, const void *sc, const void *alpha, const void *beta,
                         const void *tgt,
-                        int B, int Hq, int H, int T, int D, int n_super_cap, int bits,
+                        int B, int Hq, int H, int T, int D, int n_super_cap, int bits, int64_t ld,
                         void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
                         void *stream)
 {
+    if (ld != 0 && ld < (int64_t)T + 1)
+        return ADKV_E_SHAPE;
     if (!q || !k_cache || !k_new || !logits || !zp || !sc || !alpha || !beta || !tgt)
         return ADKV_E_NULL;
     if (bits != 2 && bits != 4)
@@ -1254,7 +1260,9 @@ int adkv_forward_qk_gqa(const void *q, void *k_cache, const void *k_new, void *l
         return rc;
     const int BH = B * H;
     hipStream_t st = (hipStream_t)stream;
-    const Seg seg = plan_segments(ckpt, n_ckpt_cap, ckpt_interval, BH, T, D);
+    Seg seg = plan_segments(ckpt, n_ckpt_cap, ckpt_interval, BH, T, D);
+    if (ld)
+        seg.row_pitch = ld;
     if (D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha())) {
         ADKV_DISPATCH_GQ(qk_gqa_kernel, (const h1 *)q, (uint4 *)k_cache, (const h1 *)k_new,
                          (h1 *)logits, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,
@@ -1276,7 +1284,7 @@ int adkv_forward_qk_ex(const void *q, void *k_cache, const void *k_new, void *lo
                        void *stream)
 {
     return adkv_forward_qk_gqa(q, k_cache, k_new, logits, zp, sc, alpha, beta, tgt, B, H, H, T, D,
-                               n_super_cap, 4, state_out, ckpt, n_ckpt_cap, ckpt_interval, stream);
+                               n_super_cap, 4, 0, state_out, ckpt, n_ckpt_cap, ckpt_interval, stream);
 }
 
 int adkv_forward_qk(const void *q, void *k_cache, const void *k_new, void *logits,
@@ -1301,10 +1309,12 @@ int64_t adkv_forward_ov_workspace_bytes(int B, int H, int T, int D, int n_ckpt_c
 int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void *out,
                         const void *zp, const void *sc, const void *alpha, const void *beta,
                         const void *tgt,
-                        int B, int Hq, int H, int T, int D, int n_super_cap, int bits,
+                        int B, int Hq, int H, int T, int D, int n_super_cap, int bits, int64_t ld,
                         void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
                         void *workspace, int64_t workspace_bytes, void *stream)
 {
+    if (ld != 0 && ld < (int64_t)T + 1)
+        return ADKV_E_SHAPE;
     if (!attn || !v_cache || !v_new || !out || !zp || !sc || !alpha || !beta || !tgt)
         return ADKV_E_NULL;
     if (bits != 2 && bits != 4)
@@ -1325,7 +1335,9 @@ int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void
         return rc;
     const int BH = B * H;
     hipStream_t st = (hipStream_t)stream;
-    const Seg seg = plan_segments(ckpt, n_ckpt_cap, ckpt_interval, BH, T, D);
+    Seg seg = plan_segments(ckpt, n_ckpt_cap, ckpt_interval, BH, T, D);
+    if (ld)
+        seg.row_pitch = ld;
     if (seg.nseg > 1) {
         if (!workspace || workspace_bytes < (int64_t)seg.nseg * BH * GQ * D * 4)
             return ADKV_E_WORKSPACE;
@@ -1362,7 +1374,7 @@ int adkv_forward_ov_ex(const void *attn, void *v_cache, const void *v_new, void 
                        void *workspace, int64_t workspace_bytes, void *stream)
 {
     return adkv_forward_ov_gqa(attn, v_cache, v_new, out, zp, sc, alpha, beta, tgt, B, H, H, T, D,
-                               n_super_cap, 4, state_out, ckpt, n_ckpt_cap, ckpt_interval, workspace,
+                               n_super_cap, 4, 0, state_out, ckpt, n_ckpt_cap, ckpt_interval, workspace,
                                workspace_bytes, stream);
 }
 
@@ -1383,19 +1395,31 @@ int64_t adkv_softmax_workspace_bytes(int rows, int n)
     return (int64_t)rows * ((n + SM_CHUNK - 1) / SM_CHUNK) * 8;
 }
 
+int64_t adkv_row_pitch(int n)
+{
+    // smallest odd multiple of 128 elements (256 bytes) that holds n: consecutive rows then start
+    // in different memory channels even when n itself is a power of two
+    int64_t k = ((int64_t)n + 127) / 128;
+    if (!(k & 1))
+        k++;
+    return k * 128;
+}
+
 int adkv_softmax_ex(const void *logits, void *weights, const void *mask,
-                    int rows, int n, int rows_per_mask_row, float scaling,
+                    int rows, int n, int64_t ld, int rows_per_mask_row, float scaling,
                     void *workspace, int64_t workspace_bytes, void *stream)
 {
     if (!logits || !weights)
         return ADKV_E_NULL;
-    if (rows <= 0 || n <= 0 || (mask && rows_per_mask_row <= 0))
+    if (rows <= 0 || n <= 0 || (mask && rows_per_mask_row <= 0) || (ld != 0 && ld < n))
         return ADKV_E_SHAPE;
+    if (ld == 0)
+        ld = n;
     const int64_t need = adkv_softmax_workspace_bytes(rows, n);
     if (need == 0 || !workspace || rows > 65535) {
         // one workgroup per row; rows that do not fit in its registers are read three times
         hipLaunchKernelGGL(softmax_kernel, dim3((unsigned)rows), dim3(SM_BLOCK), 0, (hipStream_t)stream,
-                           (const h1 *)logits, (h1 *)weights, (const float *)mask, n,
+                           (const h1 *)logits, (h1 *)weights, (const float *)mask, n, (long)ld,
                            mask ? rows_per_mask_row : 1, scaling);
         return check_launch();
     }
@@ -1406,18 +1430,19 @@ int adkv_softmax_ex(const void *logits, void *weights, const void *mask,
     const int nchunk = (n + SM_CHUNK - 1) / SM_CHUNK;
     const dim3 grid((unsigned)nchunk, (unsigned)rows);
     hipLaunchKernelGGL(softmax_part_kernel, grid, dim3(SM_BLOCK), 0, (hipStream_t)stream,
-                       (const h1 *)logits, (const float *)mask, (float2 *)workspace, n, nchunk,
+                       (const h1 *)logits, (const float *)mask, (float2 *)workspace, n, (long)ld, nchunk,
                        mask ? rows_per_mask_row : 1, scaling);
     hipLaunchKernelGGL(softmax_norm_kernel, grid, dim3(SM_BLOCK), 0, (hipStream_t)stream,
                        (const h1 *)logits, (h1 *)weights, (const float *)mask,
-                       (const float2 *)workspace, n, nchunk, mask ? rows_per_mask_row : 1, scaling);
+                       (const float2 *)workspace, n, (long)ld, nchunk, mask ? rows_per_mask_row : 1,
+                       scaling);
     return check_launch();
 }
 
 int adkv_softmax(const void *logits, void *weights, const void *mask,
                  int rows, int n, int rows_per_mask_row, float scaling, void *stream)
 {
-    return adkv_softmax_ex(logits, weights, mask, rows, n, rows_per_mask_row, scaling, nullptr, 0,
+    return adkv_softmax_ex(logits, weights, mask, rows, n, 0, rows_per_mask_row, scaling, nullptr, 0,
                            stream);
 }
 
@@ -1436,15 +1461,15 @@ int64_t adkv_decode_fused_workspace_bytes(int B, int Hq, int H, int T, int D, in
 {
     if (B <= 0 || H <= 0 || Hq <= 0 || T < 0)
         return 0;
-    const int64_t row = pad256((int64_t)B * Hq * (T + 1) * 2);
-    return 2 * row + pad256(adkv_softmax_workspace_bytes(B * Hq, T + 1)) +
+    const int64_t mat = pad256((int64_t)B * Hq * adkv_row_pitch(T + 1) * 2);
+    return 2 * mat + pad256(adkv_softmax_workspace_bytes(B * Hq, T + 1)) +
            adkv_forward_ov_gqa_workspace_bytes(B, Hq, H, T, D, n_ckpt_cap, ckpt_interval);
 }
 
 int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k_new, const void *v_new,
                       const void *const *k_params, const void *const *v_params,
                       const void *mask, int rows_per_mask_row, float scaling,
-                      void *out, void *weights_out,
+                      void *out, void *weights_out, int64_t weights_ld,
                       int B, int Hq, int H, int T, int D, int n_super_cap, int bits,
                       void *k_ckpt, void *v_ckpt, int n_ckpt_cap, int ckpt_interval,
                       void *workspace, int64_t workspace_bytes, void *stream)
@@ -1457,24 +1482,30 @@ int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k
         return ADKV_E_WORKSPACE;
     if ((uintptr_t)workspace & 255)
         return ADKV_E_ALIGN;
-    const int64_t row = pad256((int64_t)B * Hq * (T + 1) * 2);
+    // The logits live in the workspace with padded rows.  The weights do too unless the caller
+    // wants them; the softmax writes them with the logits' pitch, so a caller-provided matrix
+    // must use that pitch as well (weights_ld == adkv_row_pitch(T + 1)) or be avoided.
+    const int64_t ld = adkv_row_pitch(T + 1);
+    if (weights_out && weights_ld != ld)
+        return ADKV_E_SHAPE;
+    const int64_t mat = pad256((int64_t)B * Hq * ld * 2);
     char *ws = (char *)workspace;
     void *logits = ws;
-    void *weights = weights_out ? weights_out : (void *)(ws + row);
+    void *weights = weights_out ? weights_out : (void *)(ws + mat);
     int rc = adkv_forward_qk_gqa(q, k_cache, k_new, logits, k_params[0], k_params[1], k_params[2],
-                                 k_params[3], k_params[4], B, Hq, H, T, D, n_super_cap, bits, nullptr,
-                                 k_ckpt, n_ckpt_cap, ckpt_interval, stream);
+                                 k_params[3], k_params[4], B, Hq, H, T, D, n_super_cap, bits, ld,
+                                 nullptr, k_ckpt, n_ckpt_cap, ckpt_interval, stream);
     if (rc)
         return rc;
     const int64_t smb = pad256(adkv_softmax_workspace_bytes(B * Hq, T + 1));
-    rc = adkv_softmax_ex(logits, weights, mask, B * Hq, T + 1, rows_per_mask_row, scaling,
-                         smb ? ws + 2 * row : nullptr, smb, stream);
+    rc = adkv_softmax_ex(logits, weights, mask, B * Hq, T + 1, ld, rows_per_mask_row, scaling,
+                         smb ? ws + 2 * mat : nullptr, smb, stream);
     if (rc)
         return rc;
     return adkv_forward_ov_gqa(weights, v_cache, v_new, out, v_params[0], v_params[1], v_params[2],
-                               v_params[3], v_params[4], B, Hq, H, T, D, n_super_cap, bits, nullptr,
-                               v_ckpt, n_ckpt_cap, ckpt_interval, ws + 2 * row + smb,
-                               workspace_bytes - 2 * row - smb, stream);
+                               v_params[3], v_params[4], B, Hq, H, T, D, n_super_cap, bits, ld,
+                               nullptr, v_ckpt, n_ckpt_cap, ckpt_interval, ws + 2 * mat + smb,
+                               workspace_bytes - 2 * mat - smb, stream);
 }
 
 } // extern "C"

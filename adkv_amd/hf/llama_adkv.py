@@ -111,7 +111,9 @@ class LlamaModel_ADKV(LlamaModel):
             use_cache = getattr(self.config, "use_cache", True)
         if use_cache and past_key_values is None:
             # created here so that HF never substitutes its DynamicCache
-            past_key_values = KVCache_ADKV(self.config.num_hidden_layers)
+            # config.adkv_bits = 2 selects the 2-bit code format (extension; default 4 as the reference)
+            past_key_values = KVCache_ADKV(self.config.num_hidden_layers,
+                                           bits=getattr(self.config, "adkv_bits", 4))
         return super().forward(input_ids=input_ids, attention_mask=attention_mask,
                                position_ids=position_ids, past_key_values=past_key_values,
                                inputs_embeds=inputs_embeds, cache_position=cache_position,

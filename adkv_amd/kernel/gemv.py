@@ -47,6 +47,24 @@ def _params(tensors, names, nh, dim):
     return res
 
 
+def _pitch(n: int) -> int:
+    """Row pitch for a ``[rows, n]`` logits / weights matrix.  Long rows are padded to the library's
+    recommended pitch (an odd multiple of 128 elements) so that rows of different heads do not all
+    start in one memory channel; short rows stay packed."""
+    return int(_lib.lib().adkv_row_pitch(n)) if n >= 1024 else n
+
+
+def _rows_view(t: torch.Tensor):
+    """``(tensor, pitch)`` for a ``[B, nh, n]`` matrix whose rows are ``pitch`` elements apart: the
+    tensor itself when it is packed or a padded view this module produced, else a packed copy."""
+    B, nh, n = t.shape
+    if t.is_contiguous():
+        return t, n
+    if t.stride(2) == 1 and t.stride(1) >= n and t.stride(0) == nh * t.stride(1):
+        return t, t.stride(1)
+    return t.contiguous(), n
+
+
 def _ptr(t: torch.Tensor | None) -> int | None:
     return None if t is None else t.data_ptr()
 
@@ -126,7 +144,8 @@ def forward_qk(
 
     q_flat = q.contiguous()
     k_new_flat = k_new.reshape(B * nh, DIM).contiguous()
-    o = torch.empty((B * nq, T + 1), dtype=torch.float16, device=dev)
+    ld = _pitch(T + 1)
+    o = torch.empty((B, nq, ld), dtype=torch.float16, device=dev)
     if state_out is not None:
         _chk(state_out.dtype == torch.float16 and state_out.is_contiguous()
              and state_out.numel() == B * nh * DIM * 2, "state_out must be contiguous fp16 [B,nh,DIM,2]")
@@ -135,10 +154,10 @@ def forward_qk(
         rc = _lib.lib().adkv_forward_qk_gqa(
             q_flat.data_ptr(), k_cache.data_ptr(), k_new_flat.data_ptr(), o.data_ptr(),
             zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
-            B, nq, nh, T, DIM, n_super_cap, bits, _ptr(state_out), cp, ccap, civ,
+            B, nq, nh, T, DIM, n_super_cap, bits, ld, _ptr(state_out), cp, ccap, civ,
             _lib.current_stream_ptr(dev))
     _lib.check(rc, "forward_qk")
-    return o.reshape(B, nq, T + 1)
+    return o[:, :, :T + 1]
 
 
 def forward_ov(
@@ -188,7 +207,7 @@ def forward_ov(
     _chk(DIM in _DIMS, "DIM must be 128, 256 or 512")
     dev = _need_device(attn, v_cache, v_new, zp, sc, al, be, tg)
 
-    attn_flat = attn.contiguous()
+    attn_flat, ld = _rows_view(attn)
     v_new_flat = v_new.reshape(B * nh, DIM).contiguous()
     o = torch.empty((B * nq, DIM), dtype=torch.float16, device=dev)
     if state_out is not None:
@@ -205,7 +224,7 @@ def forward_ov(
         rc = L.adkv_forward_ov_gqa(
             attn_flat.data_ptr(), v_cache.data_ptr(), v_new_flat.data_ptr(), o.data_ptr(),
             zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
-            B, nq, nh, T, DIM, n_super_cap, bits, _ptr(state_out), cp, ccap, civ,
+            B, nq, nh, T, DIM, n_super_cap, bits, ld, _ptr(state_out), cp, ccap, civ,
             _ptr(ws), ws_bytes, _lib.current_stream_ptr(dev))
     _lib.check(rc, "forward_ov")
     return o.view(attn.shape[0], attn.shape[1], -1)
@@ -329,8 +348,8 @@ def softmax_scale_mask(logits: torch.Tensor, scaling: float,
     _chk(logits.dim() == 3, "logits must be [B, nh, n]")
     B, nh, n = logits.shape
     dev = _need_device(logits)
-    lg = logits.contiguous()
-    out = torch.empty_like(lg)
+    lg, ld = _rows_view(logits)
+    out = torch.empty((B, nh, ld), dtype=torch.float16, device=dev)[:, :, :n]
     rpm, mptr = 1, None
     mk = None
     if mask is not None:
@@ -344,7 +363,7 @@ def softmax_scale_mask(logits: torch.Tensor, scaling: float,
     wsb = L.adkv_softmax_workspace_bytes(B * nh, n)
     ws = torch.empty(wsb, dtype=torch.uint8, device=dev) if wsb else None
     with torch.cuda.device(dev):
-        rc = L.adkv_softmax_ex(lg.data_ptr(), out.data_ptr(), mptr, B * nh, n, rpm, float(scaling),
+        rc = L.adkv_softmax_ex(lg.data_ptr(), out.data_ptr(), mptr, B * nh, n, ld, rpm, float(scaling),
                                _ptr(ws), wsb, _lib.current_stream_ptr(dev))
     _lib.check(rc, "softmax_scale_mask")
     return out
@@ -419,17 +438,18 @@ def decode_fused(
     knf = k_new.reshape(B * nh, DIM).contiguous()
     vnf = v_new.reshape(B * nh, DIM).contiguous()
     out = torch.empty((B, nq, DIM), dtype=torch.float16, device=dev)
-    weights = torch.empty((B, nq, n), dtype=torch.float16, device=dev)
+    wld = int(L.adkv_row_pitch(n))
+    weights = torch.empty((B, nq, wld), dtype=torch.float16, device=dev)
     arr = _lib.C.c_void_p * 5
     with torch.cuda.device(dev):
         rc = L.adkv_decode_fused(
             qf.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), knf.data_ptr(), vnf.data_ptr(),
             arr(*[t.data_ptr() for t in kp]), arr(*[t.data_ptr() for t in vp]),
-            mptr, rpm, float(scaling), out.data_ptr(), weights.data_ptr(),
+            mptr, rpm, float(scaling), out.data_ptr(), weights.data_ptr(), wld,
             B, nq, nh, T, DIM, n_super_cap, bits, kcp, vcp, ccap, civ,
             workspace.data_ptr(), workspace.numel(), _lib.current_stream_ptr(dev))
     _lib.check(rc, "decode_fused")
-    return out, weights
+    return out, weights[:, :, :n]
 
 
 def decode_fused_workspace_bytes(B: int, nq: int, nh: int, T: int, DIM: int, n_ckpt_cap: int = 0,

@@ -93,11 +93,19 @@ int adkv_softmax(const void *logits, void *weights, const void *mask,
 
 /* The same with a workspace of adkv_softmax_workspace_bytes(rows, n) bytes (0 for short rows):
  * long rows (contexts of tens of thousands of tokens) are then cut into chunks that many
- * workgroups process, instead of one workgroup walking the row three times. */
+ * workgroups process, instead of one workgroup walking the row three times.  ld: pitch of both
+ * matrices in elements (0 = n); the mask stays packed. */
 int64_t adkv_softmax_workspace_bytes(int rows, int n);
 int adkv_softmax_ex(const void *logits, void *weights, const void *mask,
-                    int rows, int n, int rows_per_mask_row, float scaling,
+                    int rows, int n, int64_t ld, int rows_per_mask_row, float scaling,
                     void *workspace, int64_t workspace_bytes, void *stream);
+
+/* Row pitch (in elements) this library recommends for a logits / attention-weight matrix with n
+ * columns: the smallest odd multiple of 128.  The `ld` arguments of the entry points below are
+ * such pitches (0 = rows packed back to back, n = T + 1).  With packed rows and n*2 bytes close
+ * to a power of two (ctx 4096, 131072 ...), the rows of all heads start in the same memory
+ * channel and the waves, which walk their rows in step, queue up on it. */
+int64_t adkv_row_pitch(int n);
 
 /*
  * ---- Extensions with state checkpoints (no counterpart in the reference's code; its paper sketches
@@ -168,7 +176,7 @@ int adkv_forward_ov_ex(const void *attn, void *v_cache, const void *v_new, void 
 int adkv_forward_qk_gqa(const void *q, void *k_cache, const void *k_new, void *logits,
                         const void *zp, const void *sc, const void *alpha, const void *beta,
                         const void *tgt,
-                        int B, int Hq, int H, int T, int D, int n_super_cap, int bits,
+                        int B, int Hq, int H, int T, int D, int n_super_cap, int bits, int64_t ld,
                         void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
                         void *stream);
 int64_t adkv_forward_ov_gqa_workspace_bytes(int B, int Hq, int H, int T, int D, int n_ckpt_cap,
@@ -176,7 +184,7 @@ int64_t adkv_forward_ov_gqa_workspace_bytes(int B, int Hq, int H, int T, int D, 
 int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void *out,
                         const void *zp, const void *sc, const void *alpha, const void *beta,
                         const void *tgt,
-                        int B, int Hq, int H, int T, int D, int n_super_cap, int bits,
+                        int B, int Hq, int H, int T, int D, int n_super_cap, int bits, int64_t ld,
                         void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
                         void *workspace, int64_t workspace_bytes, void *stream);
 
@@ -187,8 +195,8 @@ int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void
  * q: fp16 [B, Hq, D] with Hq a multiple of the H KV heads (Hq == H is the reference's case).
  * k_params / v_params: host arrays of five device pointers {zp, sc, alpha, beta, tgt}, each
  * fp16 [H, D].  mask: optional fp32 additive mask as in adkv_softmax.  out: fp16 [B, Hq, D].
- * weights_out: optional fp16 [B, Hq, T+1] (the attention weights the reference returns); when
- * NULL they live in the workspace.  Checkpoint tensors as in the _ex entry points (NULL = none).
+ * weights_out: optional fp16 [B, Hq, weights_ld] with weights_ld == adkv_row_pitch(T + 1), columns
+ * 0..T valid (the attention weights the reference returns); when NULL they live in the workspace.  Checkpoint tensors as in the _ex entry points (NULL = none).
  * workspace: >= adkv_decode_fused_workspace_bytes(...) bytes, 256-byte aligned.
  */
 int64_t adkv_decode_fused_workspace_bytes(int B, int Hq, int H, int T, int D, int n_ckpt_cap,
@@ -196,7 +204,7 @@ int64_t adkv_decode_fused_workspace_bytes(int B, int Hq, int H, int T, int D, in
 int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k_new,
                       const void *v_new, const void *const *k_params, const void *const *v_params,
                       const void *mask, int rows_per_mask_row, float scaling,
-                      void *out, void *weights_out,
+                      void *out, void *weights_out, int64_t weights_ld,
                       int B, int Hq, int H, int T, int D, int n_super_cap, int bits,
                       void *k_ckpt, void *v_ckpt, int n_ckpt_cap, int ckpt_interval,
                       void *workspace, int64_t workspace_bytes, void *stream);
