@@ -242,18 +242,28 @@ __global__ __launch_bounds__(BLK) void encode_kernel(
             x[0] = splat(xb[(size_t)(t - T0) * D]);
         }
     };
+    // reciprocal of the current scale, refreshed right after every update (see quantize_enc_fast)
+    float rs[NP][2];
+    auto refresh = [&](int p) {
+        rs[p][0] = __builtin_amdgcn_rcpf((float)st[p].sc.x);
+        rs[p][1] = CPL >= 2 ? __builtin_amdgcn_rcpf((float)st[p].sc.y) : rs[p][0];
+    };
+#pragma unroll
+    for (int p = 0; p < NP; p++)
+        refresh(p);
     auto step = [&](const h2 *x, int tt, uint32_t *w) {
 #pragma unroll
         for (int p = 0; p < NP; p++) {
-            const int q0 = quantize_enc<BITS>(x[p].x, st[p].zp.x, st[p].sc.x);
+            const int q0 = quantize_enc_fast<BITS>(x[p].x, st[p].zp.x, st[p].sc.x, rs[p][0]);
             w[CPL >= 2 ? 2 * p : 0] += (uint32_t)q0 << (BITS * tt);
             int q1 = q0;
             if (CPL >= 2) {
-                q1 = quantize_enc<BITS>(x[p].y, st[p].zp.y, st[p].sc.y);
+                q1 = quantize_enc_fast<BITS>(x[p].y, st[p].zp.y, st[p].sc.y, rs[p][1]);
                 w[2 * p + 1] += (uint32_t)q1 << (BITS * tt);
             }
             const h2 q = (h2){(h1)(short)q0, (h1)(short)q1};
             update_pair(st[p], q, q * st[p].sc);
+            refresh(p);
         }
     };
     // bias adds -QLO to the codes written now; keep selects codes of earlier tokens to preserve

@@ -539,3 +539,31 @@ def test_streaming_append_2bit(gpu, oracle, cuts, S):
     (1, 2, 8, 40, 0), (2, 3, 4, 530, 64), (1, 2, 2, 256, 64), (1, 1, 1, 200, 16), (1, 5, 4, 1033, 0)])
 def test_decode_kernels_2bit(gpu, oracle, B, Hkv, G, T, S):
     _gqa_case(gpu, oracle, B, Hkv, G, T, S, seed=T % 7, bits=2)
+
+
+@pytest.mark.parametrize("bits", [4, 2])
+def test_encode_rounding_boundaries(gpu, oracle, bits):
+    """Inputs on and next to the quantiser's rounding boundaries: (x - zp) / sc = k + 1/2 exactly
+    (ties go to even), one fp16 step to either side, and scales that are not powers of two.  The
+    encoder decides most elements with a reciprocal multiply and must fall back to the exact
+    divide for these; codes have to match the oracle bit for bit."""
+    B, H, D, T = 1, 2, 128, 96
+    g = torch.Generator().manual_seed(11 + bits)
+    sc_choices = torch.tensor([0.25, 0.5, 1.0, 2.0, 0.75, 1.5, 3.0, 0.3330078125])
+    sc = sc_choices[torch.randint(0, len(sc_choices), (H, D), generator=g)].half()
+    k = torch.randint(-11, 11, (B, H, T, D), generator=g).float()
+    x = ((k + 0.5) * sc.float()[None, :, None, :]).half()                      # exact ties where representable
+    nudge = torch.randint(-1, 2, (B, H, T, D), generator=g).to(torch.int16)    # -1, 0, +1 fp16 steps
+    x = (x.view(torch.int16) + nudge).view(torch.float16)
+    zero = torch.zeros(H, D).half()
+    tgt = torch.full((H, D), 3.5 if bits == 4 else 0.5).half()
+    params = (zero, sc, zero, zero, tgt)                                       # alpha = beta = 0: state stays put
+    pn = [_np16(t) for t in params]
+    with oracle.code_bits(bits):
+        want = oracle.alloc_cache(B, H, T, D)
+        oracle.encode_kv_f16(want, _np16(x), *pn)
+    cache = synth.alloc_cache(B, H, T, D, gpu, bits=bits)
+    st = torch.zeros(B, H, D, 2, dtype=torch.float16, device=gpu)
+    gemv.append_kv(cache, x.to(gpu), *[t.to(gpu) for t in params], 0, st, bits=bits)
+    torch.cuda.synchronize()
+    assert np.array_equal(cache.cpu().numpy(), want)
