@@ -8,8 +8,9 @@
 //   s  = max(sc, 1e-8);  q = clamp(rint((x - zp) / s), QL, QU);  r = q*s;  xhat = r + zp
 //   zp = zp + alpha*r;   sc = clamp(sc + (sc*beta)*(|q| - tgt), sc_min, sc_max)
 //
-// One lane owns one channel and walks the tokens in order; loads run LOOKAHEAD tokens ahead of the
-// dependent chain.  The path is latency-bound (one IEEE divide per token on the critical path).
+// One lane owns one channel and walks the tokens in order; loads run a group of LOOKAHEAD tokens
+// ahead of the dependent chain.  The path is bound by the length of that chain per token, not by
+// memory.
 #include <hip/hip_runtime.h>
 #include <hip/hip_bf16.h>
 #include <stdint.h>
@@ -21,7 +22,7 @@
 namespace adkv_fp32 {
 
 constexpr int BLK = 64;
-constexpr int LOOKAHEAD = 8;
+constexpr int LOOKAHEAD = 32; // loads this far ahead also outrun the in-order completion of the stores
 
 template <typename T> struct IO;
 template <> struct IO<float> {
@@ -54,9 +55,48 @@ __device__ __forceinline__ float clamp_keep_nan(float x, float lo, float hi)
     return x < lo ? lo : (x > hi ? hi : x);
 }
 
-template <typename T>
+// One token of one channel.  The quotient is first taken with the hardware reciprocal of s (kept
+// from the previous token, off the dependent chain): r = d*rs is within 2^-22 relative of the
+// exact u = d/s, so rint(r) == rint(u) unless r lies closer than 2^-16 + |r|*2^-20 (four times the
+// error bound) to a rounding boundary k + 1/2, or is NaN; in that band the IEEE divide decides.
+// Everything after the rounding is the reference's separately rounded fp32 sequence.
+struct Chan {
+    float zp, sc, s, rs; // s = max(sc, 1e-8) (NaN kept), rs ~ 1/s
+    float al, be, tg;
+    __device__ __forceinline__ void set_scale(float v)
+    {
+        sc = v;
+        s = (v != v) ? v : (v < 1e-8f ? 1e-8f : v);
+        rs = __builtin_amdgcn_rcpf(s);
+    }
+    __device__ __forceinline__ float step(float xv, float ql, float qu, float sc_min, float sc_max, float &q)
+    {
+        const float d = xv - zp;
+        const float r = d * rs;
+        float n = __builtin_rintf(r);
+        const float margin = __builtin_fmaf(__builtin_fabsf(r), 0x1p-20f, 0x1p-16f);
+        if (__builtin_expect(!(__builtin_fabsf(r - n) < 0.5f - margin), 0))
+            n = __builtin_rintf(d / s);
+        q = clamp_keep_nan(n, ql, qu);
+        const float xr = q * s;
+        const float xh = xr + zp;
+        const float ax = al * xr;
+        const float e = __builtin_fabsf(q) - tg;
+        const float sb = sc * be;
+        const float sbe = sb * e;
+        zp = zp + ax;
+        set_scale(clamp_keep_nan(sc + sbe, sc_min, sc_max));
+        return xh;
+    }
+};
+
+// x and xhat are declared non-aliasing although the caller may pass the same buffer (in-place
+// use): every element is loaded before the token that stores to it is computed and is never read
+// again, so no ordering between a store and a later load matters; without the promise the
+// compiler serialises every prefetched load behind the stores.
+template <typename T, bool SEQ, bool OUT, bool CODES>
 __global__ __launch_bounds__(BLK) void quant_kernel(
-    const T *__restrict__ x, T *xhat, int8_t *__restrict__ codes, float *__restrict__ zp_io,
+    const T *__restrict__ x, T *__restrict__ xhat, int8_t *__restrict__ codes, float *__restrict__ zp_io,
     float *__restrict__ sc_io, const float *__restrict__ zp0, const float *__restrict__ sc0,
     const float *__restrict__ alpha, const float *__restrict__ beta, const float *__restrict__ tgt,
     float *__restrict__ zp_seq, float *__restrict__ sc_seq,
@@ -67,51 +107,53 @@ __global__ __launch_bounds__(BLK) void quant_kernel(
     if (c >= C)
         return;
     const long bc = (long)b * C + c;
-    float zp = zp0 ? zp0[c] : zp_io[bc];
-    float sc = sc0 ? sc0[c] : sc_io[bc];
-    const float al = alpha[c], be = beta[c], tg = tgt[c];
+    Chan ch;
+    ch.zp = zp0 ? zp0[c] : zp_io[bc];
+    ch.set_scale(sc0 ? sc0[c] : sc_io[bc]);
+    ch.al = alpha[c];
+    ch.be = beta[c];
+    ch.tg = tgt[c];
     const T *xp = x + b * stride_b + c;
-    T *op = xhat ? xhat + b * stride_b + c : nullptr;
+    T *op = OUT ? xhat + b * stride_b + c : nullptr;
     const long dense = (long)b * Tn * C + c; // codes / zp_seq / sc_seq are contiguous [B, T, C]
 
-    float buf[LOOKAHEAD];
-#pragma unroll
-    for (int i = 0; i < LOOKAHEAD; i++)
-        buf[i] = i < Tn ? IO<T>::ld(xp + i * stride_t) : 0.0f;
+    auto one = [&](float xv, int t) {
+        if (SEQ) {
+            zp_seq[dense + (long)t * C] = ch.zp;
+            sc_seq[dense + (long)t * C] = ch.sc;
+        }
+        float q;
+        const float xh = ch.step(xv, ql, qu, sc_min, sc_max, q);
+        if (OUT)
+            IO<T>::st(op + (long)t * stride_t, xh);
+        if (CODES)
+            codes[dense + (long)t * C] = (q != q) ? (int8_t)0 : (int8_t)q;
+    };
 
-    for (int t0 = 0; t0 < Tn; t0 += LOOKAHEAD) {
+    // full groups of LOOKAHEAD tokens with the next group's loads in flight, then the remainder
+    const int ngroups = Tn / LOOKAHEAD;
+    float buf[LOOKAHEAD];
+    if (ngroups > 0) {
+#pragma unroll
+        for (int i = 0; i < LOOKAHEAD; i++)
+            buf[i] = IO<T>::ld(xp + i * stride_t);
+    }
+    for (int g = 0; g < ngroups; g++) {
 #pragma unroll
         for (int i = 0; i < LOOKAHEAD; i++) {
-            const int t = t0 + i;
-            if (t >= Tn)
-                break;
             const float xv = buf[i];
-            if (t + LOOKAHEAD < Tn)
-                buf[i] = IO<T>::ld(xp + (long)(t + LOOKAHEAD) * stride_t);
-            if (zp_seq)
-                zp_seq[dense + (long)t * C] = zp;
-            if (sc_seq)
-                sc_seq[dense + (long)t * C] = sc;
-            const float s = (sc != sc) ? sc : (sc < 1e-8f ? 1e-8f : sc);
-            const float r = xv - zp;
-            const float u = r / s;
-            const float q = clamp_keep_nan(__builtin_rintf(u), ql, qu);
-            const float xr = q * s;
-            if (op)
-                IO<T>::st(op + (long)t * stride_t, xr + zp);
-            if (codes)
-                codes[dense + (long)t * C] = (q != q) ? (int8_t)0 : (int8_t)q;
-            const float ax = al * xr;
-            const float e = __builtin_fabsf(q) - tg;
-            const float sb = sc * be;
-            const float sbe = sb * e;
-            zp = zp + ax;
-            sc = clamp_keep_nan(sc + sbe, sc_min, sc_max);
+            // unconditional (clamped to the last token): a conditional load would have to land
+            // before the code that follows it and stall the chain
+            const int tn = min((g + 1) * LOOKAHEAD + i, Tn - 1);
+            buf[i] = IO<T>::ld(xp + (long)tn * stride_t);
+            one(xv, g * LOOKAHEAD + i);
         }
     }
+    for (int t = ngroups * LOOKAHEAD; t < Tn; t++)
+        one(IO<T>::ld(xp + (long)t * stride_t), t);
     if (zp_io) {
-        zp_io[bc] = zp;
-        sc_io[bc] = sc;
+        zp_io[bc] = ch.zp;
+        sc_io[bc] = ch.sc;
     }
 }
 
@@ -131,6 +173,8 @@ extern "C" int adkv_quant_f32(const void *x, void *xhat, void *codes, void *zp_s
         return ADKV_E_NULL;
     if (!zp_state && !zp_init)
         return ADKV_E_NULL; // no starting state at all
+    if ((zp_seq == nullptr) != (sc_seq == nullptr))
+        return ADKV_E_NULL;
     if (B <= 0 || C <= 0 || T < 0 || B > 65535 || stride_t < C || stride_b < 0)
         return ADKV_E_SHAPE;
     if (lower_limit > 0 || upper_limit < 0 || lower_limit < -128 || upper_limit > 127)
@@ -139,12 +183,31 @@ extern "C" int adkv_quant_f32(const void *x, void *xhat, void *codes, void *zp_s
         return ADKV_OK;
     const dim3 grid((unsigned)((C + BLK - 1) / BLK), (unsigned)B), block(BLK);
     hipStream_t st = (hipStream_t)stream;
-#define ADKV_Q32(TYPE)                                                                              \
-    hipLaunchKernelGGL(quant_kernel<TYPE>, grid, block, 0, st, (const TYPE *)x, (TYPE *)xhat,       \
+#define ADKV_Q32_(TYPE, SEQ, OUT, CODES)                                                            \
+    hipLaunchKernelGGL((quant_kernel<TYPE, SEQ, OUT, CODES>), grid, block, 0, st, (const TYPE *)x,  \
+                       (TYPE *)xhat,                                                                \
                        (int8_t *)codes, (float *)zp_state, (float *)sc_state, (const float *)zp_init, \
                        (const float *)sc_init, (const float *)alpha, (const float *)beta,           \
                        (const float *)tgt, (float *)zp_seq, (float *)sc_seq, T, C, (long)stride_b,  \
                        (long)stride_t, (float)lower_limit, (float)upper_limit, sc_min, sc_max)
+#define ADKV_Q32_O(TYPE, SEQ)                                                                       \
+    do {                                                                                            \
+        if (xhat && codes)                                                                          \
+            ADKV_Q32_(TYPE, SEQ, true, true);                                                       \
+        else if (xhat)                                                                              \
+            ADKV_Q32_(TYPE, SEQ, true, false);                                                      \
+        else if (codes)                                                                             \
+            ADKV_Q32_(TYPE, SEQ, false, true);                                                      \
+        else                                                                                        \
+            ADKV_Q32_(TYPE, SEQ, false, false);                                                     \
+    } while (0)
+#define ADKV_Q32(TYPE)                                                                              \
+    do {                                                                                            \
+        if (zp_seq)                                                                                 \
+            ADKV_Q32_O(TYPE, true);                                                                 \
+        else                                                                                        \
+            ADKV_Q32_O(TYPE, false);                                                                \
+    } while (0)
     switch (x_dtype) {
     case ADKV_DT_F32: ADKV_Q32(float); break;
     case ADKV_DT_F16: ADKV_Q32(_Float16); break;
@@ -152,5 +215,7 @@ extern "C" int adkv_quant_f32(const void *x, void *xhat, void *codes, void *zp_s
     default: return ADKV_E_UNSUPPORTED;
     }
 #undef ADKV_Q32
+#undef ADKV_Q32_O
+#undef ADKV_Q32_
     return hipGetLastError() == hipSuccess ? ADKV_OK : ADKV_E_LAUNCH;
 }

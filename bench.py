@@ -34,7 +34,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=40)
     ap.add_argument("--warmup", type=int, default=4)
-    ap.add_argument("--workload", choices=["decode", "encode"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "encode", "quant_f32"], default="decode",
                     help="decode = headline decode attention (cfg2); encode = streaming quantiser (cfg3: "
                          "B=8 ctx=32768 prefill, then 256 single-token appends)")
     ap.add_argument("--batch", type=int, default=128)
@@ -209,6 +209,76 @@ def encode_main(args):
     print(json.dumps(res))
 
 
+def quant_f32_main(args):
+    """cfg1: the fp32 (train / eval) recurrence over one sequence of 32 heads x 128 channels and
+    1024 tokens, K-shaped input with outlier channels.  A step is one pass over the sequence."""
+    import numpy as np
+    import torch
+    from adkv_amd import synth
+    from adkv_amd.train import quant_f32
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    B = 1 if args.batch == 128 else args.batch
+    T = 1024 if args.ctx == 4096 else args.ctx
+    H, D = args.heads, args.dim
+    C = H * D
+    p = synth.make_params(H, D, dtype=torch.float32)
+    x = synth.make_k(B, H, T, D, dtype=torch.float32).permute(0, 2, 1, 3).reshape(B, T, C).contiguous()
+    pf = [t.float().reshape(-1) for t in p.astuple()]
+    xg = x.to(dev)
+    zp_i, sc_i, al, be, tg = [t.to(dev) for t in pf]
+    smin, smax = math.exp(-4.0), math.exp(4.0)
+    zp = torch.empty(B, C, device=dev)
+    sc = torch.empty(B, C, device=dev)
+    out = torch.empty_like(xg)
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+
+    def step():
+        return quant_f32(xg, al, be, tg, -8, 7, smin, smax, zp_state=zp, sc_state=sc,
+                         zp_init=zp_i, sc_init=sc_i, out=out, want_codes=True)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    marks = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        e0, e1 = ev(), ev()
+        e0.record(); _, codes, _, _ = step(); e1.record()
+        marks.append((e0, e1))
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    k_ms = sum(a.elapsed_time(b) for a, b in marks) / len(marks)
+
+    from oracle import oracle as O
+    t0 = time.perf_counter()
+    want = O.quant_f32(x.numpy(), *[t.numpy() for t in pf])
+    cpu_s = time.perf_counter() - t0
+    exact = bool(np.array_equal(codes.cpu().numpy(), want["codes"])
+                 and np.array_equal(out.cpu().numpy().view(np.int32), want["xhat"].view(np.int32))
+                 and np.array_equal(sc.cpu().numpy().view(np.int32), want["sc"].view(np.int32)))
+    bytes_launch = B * T * C * (4 + 4 + 1)          # fp32 in, fp32 out, int8 codes
+    achieved = bytes_launch / (k_ms * 1e-3) / 1e9
+    res = {
+        "metric": "fp32-recurrence tokens quantised/sec (B*T / pass time, one tensor)",
+        "value": B * T / (ms_step * 1e-3), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"cfg1 fp32 recurrence: B={B} T={T} C={C} ({H} heads x {D}), 4-bit range, "
+                               f"K-shaped input with outlier channels",
+                   "batch": B, "heads": H, "head_dim": D, "ctx": T, "bits": 4},
+        "bit_exact_vs_oracle": exact,
+        "roofline": {"kernel": "adkv_fp32::quant_kernel", "bound": "hbm", "achieved": achieved,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
+                     "traffic": None},
+        "cpu_baseline": {"value": B * T / cpu_s, "unit": "tokens/s", "cores": 1, "kind": "port",
+                         "sample": f"C oracle adkv_o_quant_f32 over the whole workload in {cpu_s:.2f} s"},
+    }
+    print(json.dumps(res))
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -218,6 +288,8 @@ def main():
 
     if args.workload == "encode":
         return encode_main(args)
+    if args.workload == "quant_f32":
+        return quant_f32_main(args)
 
     import torch
     from adkv_amd import synth
