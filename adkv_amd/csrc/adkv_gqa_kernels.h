@@ -246,8 +246,9 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
             if (sg < nfull) {
                 // bytes of supergroup sg+1 (stale data past the end: looked up, never used)
                 code_bytes<BITS>(buf[(i + 1) % GPF], nbn);
-                if (sg + GPF < nfull)
-                    buf[i] = cb[(size_t)(sg + GPF) * G::VPS];
+                // unconditional, clamped to the segment's last supergroup: a load inside a branch
+                // makes the next wait cover every load in flight, this one included
+                buf[i] = cb[(size_t)min(sg + GPF, nfull - 1) * G::VPS];
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int hf = 0; hf < UPS; hf++) {
@@ -427,8 +428,7 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
             const int sg = sg0 + i;
             if (sg < nfull) {
                 code_bytes<BITS>(buf[(i + 1) % GPF], nbn);
-                if (sg + GPF < nfull)
-                    buf[i] = cb[(size_t)(sg + GPF) * G::VPS];
+                buf[i] = cb[(size_t)min(sg + GPF, nfull - 1) * G::VPS]; // unconditional: see qk_gqa_kernel
 #pragma unroll
                 for (int hf = 0; hf < UPS; hf++) {
                     const int unit = sg * UPS + hf;
@@ -437,11 +437,9 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
 #pragma unroll
                     for (int n = 0; n < NB; n++)
                         wcur[n] = wbuf[ws][n];
-                    if (unit + WPF < nunits) {
 #pragma unroll
-                        for (int n = 0; n < NB; n++)
-                            wbuf[ws][n] = load_w(n, unit + WPF);
-                    }
+                    for (int n = 0; n < NB; n++)
+                        wbuf[ws][n] = load_w(n, min(unit + WPF, nunits - 1));
                     __builtin_amdgcn_sched_barrier(0);
                     const bool into_next_sg = hf == UPS - 1;
 #pragma unroll

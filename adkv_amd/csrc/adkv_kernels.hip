@@ -542,10 +542,13 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
                 pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
                 if (sg > 0)
                     red_read(tmp);
-                if (sg + PF < nfull) {
+                {
+                    // unconditional, clamped to the segment's last supergroup: a load inside a
+                    // branch makes the next wait cover every load in flight, this one included
+                    const int sgp = min(sg + PF, nfull - 1);
 #pragma unroll
                     for (int v = 0; v < G::NV; v++)
-                        buf[i][v] = cb[(size_t)(sg + PF) * G::VPS + v];
+                        buf[i][v] = cb[(size_t)sgp * G::VPS + v];
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -707,11 +710,12 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
             if (sg < nfull) {
                 pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
                 const uint4 wcur = wbuf[i];
-                if (sg + PF < nfull) {
+                {
+                    const int sgp = min(sg + PF, nfull - 1); // unconditional: see qk_kernel
 #pragma unroll
                     for (int v = 0; v < G::NV; v++)
-                        buf[i][v] = cb[(size_t)(sg + PF) * G::VPS + v];
-                    wbuf[i] = load_w(sg + PF);
+                        buf[i][v] = cb[(size_t)sgp * G::VPS + v];
+                    wbuf[i] = load_w(sgp);
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
