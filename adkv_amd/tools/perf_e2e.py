@@ -16,6 +16,8 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import sys
+import threading
 import time
 
 import torch
@@ -93,6 +95,13 @@ def max_batch(args) -> dict:
             **{f"cache_MiB_per_sequence_{k}": v / 2 ** 20 for k, v in per_seq.items()}}
 
 
+def _heartbeat(stop: threading.Event, every: float = 30.0) -> None:
+    """A line on stderr every `every` seconds: long generate() calls print nothing by themselves."""
+    t0 = time.time()
+    while not stop.wait(every):
+        print(f"[perf_e2e] running, {time.time() - t0:.0f} s", file=sys.stderr, flush=True)
+
+
 def main(argv=None):
     args = parse_args(argv)
     if args.search:
@@ -104,6 +113,8 @@ def main(argv=None):
     ids = torch.randint(1, cfg.vocab_size, (args.batch_size, args.prompt_lenth), generator=g).to(device)
     mask = torch.ones_like(ids)
     gen = dict(max_new_tokens=args.output_length, min_new_tokens=args.output_length, do_sample=False)
+    stop = threading.Event()
+    threading.Thread(target=_heartbeat, args=(stop,), daemon=True).start()
     with torch.no_grad():
         model.generate(ids, attention_mask=mask, max_new_tokens=4, min_new_tokens=4, do_sample=False)
         torch.cuda.synchronize()
@@ -112,6 +123,7 @@ def main(argv=None):
         for _ in range(args.num_repeats):
             out = model.generate(ids, attention_mask=mask, **gen)
         torch.cuda.synchronize()
+    stop.set()
     ms = (time.time() - t0) / args.num_repeats * 1e3
     assert out.shape[1] == args.prompt_lenth + args.output_length
     print(json.dumps({
