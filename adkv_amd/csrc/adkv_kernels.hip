@@ -793,7 +793,10 @@ __global__ __launch_bounds__(256) void ov_finalize_kernel(const float *__restric
 // softmax(float(logits)*scaling + mask) -> fp16   (llama_adkv.py:266-271)
 // ---------------------------------------------------------------------------------------------
 constexpr int SM_BLOCK = 256;
-constexpr int SM_KEEP_FWD = 20;
+constexpr int SM_VEC = 8;                             // fp16 values per 16-byte access
+constexpr int SM_NV = 3;                              // such accesses per thread and chunk
+constexpr int SM_KEEP = SM_VEC * SM_NV;               // row elements a thread keeps in registers
+constexpr int SM_CHUNK = SM_BLOCK * SM_KEEP;          // row elements one workgroup holds
 
 __device__ __forceinline__ float block_reduce(float v, float *sm, bool is_max)
 {
@@ -814,6 +817,78 @@ __device__ __forceinline__ float block_reduce(float v, float *sm, bool is_max)
     return r;
 }
 
+// x[k] = logits*scaling + mask for the SM_KEEP elements of this thread in the chunk that starts at
+// `base` (-inf past the end of the row); 16-byte accesses wherever a whole vector lies inside the
+// row (rows are only 2-byte aligned: the hardware takes unaligned vector accesses).
+__device__ __forceinline__ void softmax_load_chunk(const h1 *l, const float *mk, int n, int base,
+                                                   float scaling, float *x, float &mx)
+{
+    mx = -INFINITY;
+#pragma unroll
+    for (int v = 0; v < SM_NV; v++) {
+        const int i0 = base + (v * SM_BLOCK + (int)threadIdx.x) * SM_VEC;
+        float *xv = x + v * SM_VEC;
+        if (i0 + SM_VEC <= n) {
+            uint4 raw;
+            __builtin_memcpy(&raw, l + i0, 16);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const h2 p = as_h2(w[k]);
+                xv[2 * k] = (float)p.x * scaling;
+                xv[2 * k + 1] = (float)p.y * scaling;
+            }
+            if (mk) {
+                float m8[SM_VEC];
+                __builtin_memcpy(m8, mk + i0, 32);
+#pragma unroll
+                for (int k = 0; k < SM_VEC; k++)
+                    xv[k] += m8[k];
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < SM_VEC; k++) {
+                const int i = i0 + k;
+                xv[k] = -INFINITY;
+                if (i < n) {
+                    xv[k] = (float)l[i] * scaling;
+                    if (mk)
+                        xv[k] += mk[i];
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < SM_VEC; k++)
+            mx = fmaxf(mx, xv[k]);
+    }
+}
+
+// w[i] = fp16(x[k] * inv) for the same elements
+__device__ __forceinline__ void softmax_store_chunk(h1 *w, int n, int base, const float *x, float inv)
+{
+#pragma unroll
+    for (int v = 0; v < SM_NV; v++) {
+        const int i0 = base + (v * SM_BLOCK + (int)threadIdx.x) * SM_VEC;
+        const float *xv = x + v * SM_VEC;
+        if (i0 + SM_VEC <= n) {
+            uint32_t o[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                o[k] = as_u32((h2){(h1)(xv[2 * k] * inv), (h1)(xv[2 * k + 1] * inv)});
+            const uint4 raw = make_uint4(o[0], o[1], o[2], o[3]);
+            __builtin_memcpy(w + i0, &raw, 16);
+        } else {
+#pragma unroll
+            for (int k = 0; k < SM_VEC; k++)
+                if (i0 + k < n)
+                    w[i0 + k] = (h1)(xv[k] * inv);
+        }
+    }
+}
+
+// One workgroup per row.  A row of up to SM_CHUNK elements is read once and kept in registers;
+// longer rows are walked three times (the chunked kernels below avoid that when the caller gives
+// a workspace).
 __global__ __launch_bounds__(SM_BLOCK) void softmax_kernel(
     const h1 *__restrict__ logits, h1 *__restrict__ weights, const float *__restrict__ mask,
     int n, long ld, int rows_per_mask_row, float scaling)
@@ -824,90 +899,43 @@ __global__ __launch_bounds__(SM_BLOCK) void softmax_kernel(
     h1 *w = weights + (size_t)row * ld;
     const float *mk = mask ? mask + (size_t)(row / rows_per_mask_row) * n : nullptr;
 
-    // rows up to SM_BLOCK*KEEP elements are read from memory once and kept in registers
-    constexpr int KEEP = SM_KEEP_FWD;
-    float x[KEEP];
-    const bool fits = n <= SM_BLOCK * KEEP;
-    float mx = -INFINITY;
-    if (fits) {
+    if (n <= SM_CHUNK) {
+        float x[SM_KEEP], mx;
+        softmax_load_chunk(l, mk, n, 0, scaling, x, mx);
+        mx = block_reduce(mx, sm, true);
+        float sum = 0.0f;
 #pragma unroll
-        for (int k = 0; k < KEEP; k++) {
-            const int i = threadIdx.x + k * SM_BLOCK;
-            x[k] = -INFINITY;
-            if (i < n) {
-                x[k] = (float)l[i] * scaling;
-                if (mk)
-                    x[k] += mk[i];
-            }
-            mx = fmaxf(mx, x[k]);
-        }
-    } else {
-        for (int i = threadIdx.x; i < n; i += SM_BLOCK) {
-            float v = (float)l[i] * scaling;
-            if (mk)
-                v += mk[i];
-            mx = fmaxf(mx, v);
-        }
-    }
-    mx = block_reduce(mx, sm, true);
-    float sum = 0.0f;
-    if (fits) {
-#pragma unroll
-        for (int k = 0; k < KEEP; k++) {
+        for (int k = 0; k < SM_KEEP; k++) {
             x[k] = __expf(x[k] - mx);
             sum += x[k];
         }
-    } else {
-        for (int i = threadIdx.x; i < n; i += SM_BLOCK) {
-            float v = (float)l[i] * scaling;
-            if (mk)
-                v += mk[i];
-            sum += __expf(v - mx);
-        }
+        sum = block_reduce(sum, sm, false);
+        softmax_store_chunk(w, n, 0, x, 1.0f / sum);
+        return;
     }
+    auto at = [&](int i) {
+        float v = (float)l[i] * scaling;
+        if (mk)
+            v += mk[i];
+        return v;
+    };
+    float mx = -INFINITY;
+    for (int i = threadIdx.x; i < n; i += SM_BLOCK)
+        mx = fmaxf(mx, at(i));
+    mx = block_reduce(mx, sm, true);
+    float sum = 0.0f;
+    for (int i = threadIdx.x; i < n; i += SM_BLOCK)
+        sum += __expf(at(i) - mx);
     sum = block_reduce(sum, sm, false);
     const float inv = 1.0f / sum;
-    if (fits) {
-#pragma unroll
-        for (int k = 0; k < KEEP; k++) {
-            const int i = threadIdx.x + k * SM_BLOCK;
-            if (i < n)
-                w[i] = (h1)(x[k] * inv);
-        }
-    } else {
-        for (int i = threadIdx.x; i < n; i += SM_BLOCK) {
-            float v = (float)l[i] * scaling;
-            if (mk)
-                v += mk[i];
-            w[i] = (h1)(__expf(v - mx) * inv);
-        }
-    }
+    for (int i = threadIdx.x; i < n; i += SM_BLOCK)
+        w[i] = (h1)(__expf(at(i) - mx) * inv);
 }
 
 // Rows longer than one workgroup can hold in registers are cut into chunks of SM_CHUNK elements,
 // one workgroup each: the first pass leaves (max, sum of exp(x - max)) per chunk, the second
 // combines a row's chunks and normalises.  Each logit is read twice and nothing depends on the
 // order in which workgroups run.
-constexpr int SM_KEEP = SM_KEEP_FWD;
-constexpr int SM_CHUNK = SM_BLOCK * SM_KEEP;
-
-__device__ __forceinline__ void softmax_load_chunk(const h1 *l, const float *mk, int n, int base,
-                                                   float scaling, float *x, float &mx)
-{
-    mx = -INFINITY;
-#pragma unroll
-    for (int k = 0; k < SM_KEEP; k++) {
-        const int i = base + threadIdx.x + k * SM_BLOCK;
-        x[k] = -INFINITY;
-        if (i < n) {
-            x[k] = (float)l[i] * scaling;
-            if (mk)
-                x[k] += mk[i];
-        }
-        mx = fmaxf(mx, x[k]);
-    }
-}
-
 __global__ __launch_bounds__(SM_BLOCK) void softmax_part_kernel(
     const h1 *__restrict__ logits, const float *__restrict__ mask, float2 *__restrict__ part,
     int n, long ld, int nchunk, int rows_per_mask_row, float scaling)
@@ -948,15 +976,12 @@ __global__ __launch_bounds__(SM_BLOCK) void softmax_norm_kernel(
         if (p.x > -INFINITY)
             Z += p.y * __expf(p.x - M);
     }
-    const float inv = 1.0f / Z;
     float x[SM_KEEP], mx;
     softmax_load_chunk(l, mk, n, ck * SM_CHUNK, scaling, x, mx);
 #pragma unroll
-    for (int k = 0; k < SM_KEEP; k++) {
-        const int i = ck * SM_CHUNK + threadIdx.x + k * SM_BLOCK;
-        if (i < n)
-            w[i] = (h1)(__expf(x[k] - M) * inv);
-    }
+    for (int k = 0; k < SM_KEEP; k++)
+        x[k] = __expf(x[k] - M);
+    softmax_store_chunk(w, n, ck * SM_CHUNK, x, 1.0f / Z);
 }
 
 } // namespace adkv
