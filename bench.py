@@ -194,7 +194,9 @@ def encode_main(args):
         "codes_bit_exact_vs_oracle": exact,
         "roofline": {"kernel": "encode_kernel", "bound": "hbm", "achieved": achieved,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": None},
+                     # FETCH_SIZE/WRITE_SIZE per prefill launch, scaled by a 1 GiB copy
+                     # (profiles/encode_cfg3_and_decode_cfg5_pmc_traffic.md); default workload only
+                     "traffic": 2.7015e9 if (B, H, D, T, S) == (8, 32, 128, 32768, 256) else None},
     }
     if not args.no_cpu_baseline:
         hs, Ts = 2, 4096
@@ -411,7 +413,9 @@ def main():
             "frac": achieved / HBM_PEAK_GBPS,
             # HBM bytes per QK launch from rocprofv3 FETCH_SIZE/WRITE_SIZE scaled by a 1 GiB copy
             # (profiles/decode_cfg2_pmc_traffic.md); measured for the default workload only
-            "traffic": 1.1227e9 if (B, Hq, H, D, T, S, bits) == (128, 32, 32, 128, 4096, 256, 4) else None,
+            # (profiles/encode_cfg3_and_decode_cfg5_pmc_traffic.md for the grouped-query 2-bit shape)
+            "traffic": {(128, 32, 32, 128, 4096, 256, 4): 1.1227e9,
+                        (16, 32, 8, 128, 131072, 256, 2): 0.6911e9}.get((B, Hq, H, D, T, S, bits)),
         },
     }
     if not args.no_fp16_comparator and D == 128 and H == Hq and bits == 4:
