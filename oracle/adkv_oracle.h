@@ -8,9 +8,10 @@
  * smoke check and the bench's cpu_baseline leg do.
  *
  * Parity status: the reference holds no tests or golden vectors for this path; every function is
- * pinned by the independent checks in tests/test_oracle_*.py.  Parity unpinned on two points:
- * adkv_o_quant_f32 versus the reference's torch.compile'd chunk function (compiler-dependent),
- * and CUDA hardware behaviour at NaN/denormal corners beyond its intrinsics' documentation.
+ * pinned by the independent checks in tests/test_oracle_*.py, and adkv_o_quant_f32 additionally by
+ * vectors recorded from the reference's own (torch.compile'd) fp32 module
+ * (tests/golden/fp32_reference.npz, tests/test_golden_fp32_reference.py).  Parity unpinned on one
+ * point: CUDA hardware behaviour at NaN/denormal corners beyond its intrinsics' documentation.
  *
  * All fp16 values cross this interface as raw uint16_t bit patterns.
  */
