@@ -50,19 +50,6 @@ __device__ __forceinline__ void update_pair(Pair &p, h2 q, h2 qs)
     p.sc = p.sc * f;
 }
 
-// Byte row br of two channel words -> the two tokens' code pairs as exact fp16 integers.
-//   x = [0, B.byte[br], 0, A.byte[br]]
-//   low nibbles : 0x6400|n = 1024+n  -> minus 1032 = n-8   (gemv.cu:79-88)
-//   high nibbles: 0x5400|(n<<4) = 64+n -> minus 72 = n-8   (same trick one binade lower: no shift)
-template <int BR>
-__device__ __forceinline__ void unpack_row(uint32_t wa, uint32_t wb, h2 &q_even, h2 &q_odd)
-{
-    constexpr uint32_t sel = 0x0C000C00u | ((4u + BR) << 16) | (uint32_t)BR;
-    const uint32_t x = __builtin_amdgcn_perm(wb, wa, sel);
-    q_even = as_h2((x & 0x000F000Fu) | 0x64006400u) - splat((h1)1032.0f);
-    q_odd = as_h2((x & 0x00F000F0u) | 0x54005400u) - splat((h1)72.0f);
-}
-
 // ---------------------------------------------------------------------------------------------
 // Code-pair lookup table in LDS.
 //
@@ -139,21 +126,10 @@ __device__ __forceinline__ int quantize(h1 x, h1 zp, h1 sc)
     return (int)r;
 }
 
-// The encoder's form of quantize(): same value, fewer instructions.  x - zp as one fp32 fma with
-// fp16 operands (exactly the rounded fp32 difference), IEEE divide, round-half-even, then the
-// hardware float->int conversion, which saturates and maps NaN to 0 as CUDA's __float2int_rn does.
-template <int BITS = 4>
-__device__ __forceinline__ int quantize_enc(h1 x, h1 zp, h1 sc)
-{
-    const float d = __builtin_fmaf((float)x, 1.0f, -(float)zp);
-    const float r = __builtin_rintf(d / (float)sc);
-    int q;
-    asm("v_cvt_i32_f32 %0, %1" : "=v"(q) : "v"(r));
-    return q < Code<BITS>::QLO ? Code<BITS>::QLO : (q > Code<BITS>::QHI ? Code<BITS>::QHI : q);
-}
-
-// The same value with the IEEE divide off the token-to-token critical path.  rsc is the hardware
-// reciprocal of sc (1 ulp), taken as soon as sc is known.  r = d*rsc is within 2^-22 relative of
+// The encoder's form of quantize(): the same value with the IEEE divide off the token-to-token
+// critical path.  x - zp is one fp32 fma with fp16 operands (exactly the rounded fp32 difference);
+// the hardware float->int conversion saturates and maps NaN to 0 as CUDA's __float2int_rn does.
+// rsc is the hardware reciprocal of sc (1 ulp), taken as soon as sc is known.  r = d*rsc is within 2^-22 relative of
 // the exact quotient u, so for |r| < 16 it is within 2^-18 absolute: unless r lies closer than
 // 2^-16 to a rounding boundary k + 1/2, rint(r) == rint(u) (exact ties always land in that band).
 // For |r| >= 16 both u and r are beyond the clamp on the same side, whatever rint gives.  Inside
