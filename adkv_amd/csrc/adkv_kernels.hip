@@ -1022,7 +1022,11 @@ static inline int lanes_per_head(int D) { return D == 128 ? 32 : 64; }
 constexpr int WAVES_PER_SIMD_TARGET = 4;
 constexpr int N_SIMD = 256 * 4;
 
-// Segment plan for a decode launch: as few segments as give every SIMD its target of waves.
+// Segment plan for a decode launch.  Starting from the fewest segments that give every SIMD its
+// target of waves, finer splits are taken when they shorten the launch: 16-wave workgroups run one
+// per CU, so a launch is ceil(workgroups / 256) rounds of one segment's length each, and a batch
+// whose workgroup count falls just past a multiple of 256 (B = 352: 352 workgroups = 2 rounds for
+// 1.4 rounds of work) wastes most of a round unless it is cut finer.
 static Seg plan_segments(void *ckpt, int n_ckpt_cap, int ckpt_interval, int BH, int T, int D)
 {
     Seg s;
@@ -1035,19 +1039,44 @@ static Seg plan_segments(void *ckpt, int n_ckpt_cap, int ckpt_interval, int BH, 
     if (!ckpt || ckpt_interval <= 0 || T <= ckpt_interval)
         return s;
     const int avail = (T + ckpt_interval - 1) / ckpt_interval;               // finest split
-    const long units_target = (long)N_SIMD * WAVES_PER_SIMD_TARGET * (64 / lanes_per_head(D));
+    const int lph = lanes_per_head(D);
+    const long units_target = (long)N_SIMD * WAVES_PER_SIMD_TARGET * (64 / lph);
     long want = (units_target + BH - 1) / BH;
     if (want < 1)
         want = 1;
     if (want > avail)
         want = avail;
-    int m = (int)((avail + want - 1) / want);                                 // intervals per segment
+    const int m0 = (int)((avail + want - 1) / want);                          // intervals per segment
     // every segment start s*m*interval needs checkpoint s*m-1 < n_ckpt_cap
-    while (m < avail && ((avail - 1) / m) * m - 1 >= n_ckpt_cap)
-        m++;
-    if (m >= avail)
+    auto valid = [&](int m) { return m >= avail || ((avail - 1) / m) * m - 1 < n_ckpt_cap; };
+    // launch length in units of one checkpoint interval
+    auto cost = [&](int m) {
+        const int nseg = (avail + m - 1) / m;
+        const long threads = (long)BH * nseg * lph;
+        if (D == 512 || threads < 1024L * 256)
+            return (double)m;                        // small workgroups: no round structure to model
+        const long wgs = (threads + 1023) / 1024;
+        return (double)((wgs + 255) / 256) * m;
+    };
+    int best = -1;
+    double best_cost = 0.0;
+    for (int m = avail; m >= 1; m--) {
+        if (m > m0 && m < avail)
+            continue;                                // between "one segment" and the occupancy target: skip
+        if (!valid(m))
+            continue;
+        const double c = cost(m);
+        if (best < 0 || c < 0.97 * best_cost) {      // a finer split has to pay for its overheads
+            best = m;
+            best_cost = c;
+        }
+    }
+    // the occupancy target comes first: one segment is only kept when no split is possible
+    if (best >= avail && m0 < avail && valid(m0))
+        best = m0;
+    if (best < 0 || best >= avail)
         return s;
-    s.seg_tokens = m * ckpt_interval;
+    s.seg_tokens = best * ckpt_interval;
     s.nseg = (T + s.seg_tokens - 1) / s.seg_tokens;
     return s;
 }

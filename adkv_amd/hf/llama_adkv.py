@@ -79,6 +79,12 @@ class LlamaAttention_ADKV(LlamaAttention):
             return self.o_proj(ctx.reshape(*lead, -1).contiguous()), weights
 
         if layer_cache is not None:
+            if layer_cache.get_seq_length() > 0:
+                # the earlier tokens exist only as codes: a multi-token step would have to attend
+                # over dequantised history, which this deployment path does not keep (the cache
+                # object itself accepts prompt chunks; see KVCacheLayer_ADKV.prefill)
+                raise NotImplementedError(
+                    "ADKV attention takes the prompt in one call; multi-token steps after it are not supported")
             layer_cache.prefill(k, v, *self._adkv_params("key"), *self._adkv_params("value"))
 
         attend = eager_attention_forward

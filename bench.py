@@ -324,6 +324,8 @@ def main():
         del x
         kps.append(kp.astuple()); vps.append(vp.astuple()); kcs.append(kc); vcs.append(vc)
         kks.append(kk); vks.append(vk)
+        if NL > 8:
+            torch.cuda.empty_cache()   # many resident layer caches: keep the input scratch from fragmenting
     q = synth.make_q(B, Hq, D, device=dev)
     k_new = synth.make_k(B, H, 1, D, seed=11, dtype=torch.float16, device=dev, t0=T)
     v_new = synth.make_v(B, H, 1, D, seed=12, dtype=torch.float16, device=dev)
