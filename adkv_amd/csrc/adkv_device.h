@@ -126,26 +126,66 @@ __device__ __forceinline__ int quantize(h1 x, h1 zp, h1 sc)
     return (int)r;
 }
 
-// The encoder's form of quantize(): the same value with the IEEE divide off the token-to-token
-// critical path.  x - zp is one fp32 fma with fp16 operands (exactly the rounded fp32 difference);
-// the hardware float->int conversion saturates and maps NaN to 0 as CUDA's __float2int_rn does.
-// rsc is the hardware reciprocal of sc (1 ulp), taken as soon as sc is known.  r = d*rsc is within 2^-22 relative of
-// the exact quotient u, so for |r| < 16 it is within 2^-18 absolute: unless r lies closer than
-// 2^-16 to a rounding boundary k + 1/2, rint(r) == rint(u) (exact ties always land in that band).
-// For |r| >= 16 both u and r are beyond the clamp on the same side, whatever rint gives.  Inside
-// the band, and for NaN, the exact divide decides; that branch is taken by about one element in
-// 30 000.
-template <int BITS = 4>
-__device__ __forceinline__ int quantize_enc_fast(h1 x, h1 zp, h1 sc, float rsc)
+// The encoder's form of quantize(): the same value with as few dependent instructions between
+// one token's state and the next as the arithmetic allows.
+//  * x - zp is one mixed-precision fma on the fp16 halves in place (f32(x)*1 - f32(zp), rounded
+//    once: exactly the reference's fp32 difference) instead of two conversions and a subtract.
+//  * rsc is the hardware reciprocal of sc (1 ulp), taken as soon as sc is known.  r = d*rsc is
+//    within 2^-22 relative of the exact quotient u, so for |r| < 16 it is within 2^-18 absolute:
+//    unless r lies closer than 2^-16 to a rounding boundary k + 1/2, rint(r) == rint(u) (exact
+//    ties always land in that band).  For |r| >= 16 both u and r are beyond the clamp on the same
+//    side, whatever rint gives.  Inside the band, and for NaN (which ends as code 0, like CUDA's
+//    __float2int_rn), the exact divide decides; that branch is taken by about one element in
+//    30 000.
+//  * The result is the clamped code as a float (an integer in [QLO, QHI]): the fp16 operands of
+//    the state update are converted from it directly, the integer for the code word off the
+//    critical path.
+// xw / zpw hold the fp16 operands in their low (HI = false) or high (HI = true) halves.
+template <int BITS, bool HI>
+__device__ __forceinline__ float quantize_enc_fast(uint32_t xw, uint32_t zpw, h1 sc, float rsc)
 {
-    const float d = __builtin_fmaf((float)x, 1.0f, -(float)zp);
+    float d;
+    if (HI)
+        asm("v_fma_mix_f32 %0, %1, 1.0, -%2 op_sel:[1,0,1] op_sel_hi:[1,0,1]" : "=v"(d) : "v"(xw), "v"(zpw));
+    else
+        asm("v_fma_mix_f32 %0, %1, 1.0, -%2 op_sel_hi:[1,0,1]" : "=v"(d) : "v"(xw), "v"(zpw));
     const float r = d * rsc;
     float n = __builtin_rintf(r);
-    if (__builtin_expect(!(__builtin_fabsf(r - n) < 0.5f - 0x1p-16f), 0))
+    if (__builtin_expect(!(__builtin_fabsf(r - n) < 0.5f - 0x1p-16f), 0)) {
         n = __builtin_rintf(d / (float)sc);
-    int q;
-    asm("v_cvt_i32_f32 %0, %1" : "=v"(q) : "v"(n));
-    return q < Code<BITS>::QLO ? Code<BITS>::QLO : (q > Code<BITS>::QHI ? Code<BITS>::QHI : q);
+        n = (n != n) ? 0.0f : n;
+    }
+    return __builtin_amdgcn_fmed3f(n, (float)Code<BITS>::QLO, (float)Code<BITS>::QHI);
+}
+
+// quantize_enc_fast without its branch, for lanes whose wave is alone on its SIMD and pays every
+// dependent instruction in full: the code is taken from the reciprocal product unconditionally and
+// the squared distance of r from its integer is folded into `worst` as an unsigned maximum (a NaN
+// has the largest bit pattern of all).  A caller that finds worst >= ENC_SPEC_LIMIT afterwards
+// must discard the codes and the state derived from them and redo the tokens with
+// quantize_enc_fast.  Squaring is monotonic, so every |r - n| >= 0.5 - 2^-16 is caught.
+constexpr float ENC_SPEC_EDGE = 0.5f - 0x1p-16f;
+constexpr float ENC_SPEC_LIMIT = ENC_SPEC_EDGE * ENC_SPEC_EDGE;
+template <int BITS, bool HI>
+__device__ __forceinline__ float quantize_enc_spec(uint32_t xw, uint32_t zpw, float rsc, uint32_t &worst)
+{
+    float d;
+    if (HI)
+        asm("v_fma_mix_f32 %0, %1, 1.0, -%2 op_sel:[1,0,1] op_sel_hi:[1,0,1]" : "=v"(d) : "v"(xw), "v"(zpw));
+    else
+        asm("v_fma_mix_f32 %0, %1, 1.0, -%2 op_sel_hi:[1,0,1]" : "=v"(d) : "v"(xw), "v"(zpw));
+    const float r = d * rsc;
+    const float n = __builtin_rintf(r);
+    const float e = r - n;
+    const uint32_t e2 = __float_as_uint(e * e);
+    worst = worst > e2 ? worst : e2;
+    return __builtin_amdgcn_fmed3f(n, (float)Code<BITS>::QLO, (float)Code<BITS>::QHI);
+}
+
+// Two small integers held as floats -> fp16 pair (exact, so the rounding mode is irrelevant).
+__device__ __forceinline__ h2 pack_codes(float a, float b)
+{
+    return __builtin_bit_cast(h2, __builtin_amdgcn_cvt_pkrtz(a, b));
 }
 
 __device__ __forceinline__ h2 codes_to_h2(int q0, int q1) { return (h2){(h1)q0, (h1)q1}; }

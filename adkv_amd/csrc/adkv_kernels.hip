@@ -179,20 +179,22 @@ __device__ __forceinline__ void init_pairs(Pair *st, const h1 *zp, const h1 *sc,
 // encode_kv  (gemv.cu:168-308)
 // ---------------------------------------------------------------------------------------------
 // The state at token t depends on every code before it, so the encoder is one serial chain per
-// channel and nothing but B*H*D is parallel.  A lane owns CPL consecutive channels (1, 2 or 4: the
-// launcher picks the widest that still gives every SIMD work, because a wave that is alone on its
-// SIMD issues an instruction only every ~5 ns whatever it is).  Input rows for the next two
-// supergroups are in flight while the current one is quantised.  The eight codes of a channel are
-// summed as signed q << 4t and biased once by 0x8888... instead of being masked in one by one.
+// channel and nothing but B*H*D is parallel.  A lane owns CPL consecutive channels (1 or 2, the
+// launcher's choice).  With few channels every wave has a SIMD to itself and the time per token
+// is the length of its instruction stream, so that stream is kept short: the dependent chain from
+// one token's state to the next is mixed-precision fma -> mul -> rint -> med3 -> pack -> packed
+// mul -> packed fma, input rows are loaded two groups of 8 tokens ahead with nothing waiting on
+// them, codes are summed as signed q << 4t in floats (one fma each) and biased once by 0x8888...,
+// row pointers advance by addition, checkpoints are found by comparison.
 constexpr int ENC_PF = 3; // supergroup input buffers in rotation
 
 template <int BITS, int CPL, int BLK>
-__global__ __launch_bounds__(BLK) void encode_kernel(
+__device__ __forceinline__ void encode_body(
     uint32_t *__restrict__ cache, const h1 *__restrict__ kv_new,
     const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
     const h1 *__restrict__ be, const h1 *__restrict__ tg,
     int BH, int H, int T0, int T, int D, int n_super_cap, const h1 *__restrict__ state_in,
-    h1 *__restrict__ state_out, Seg sa)
+    h1 *__restrict__ state_out, const Seg &sa)
 {
     // Quantises tokens [T0, T) of a stream whose first T0 tokens are already in the cache; kv_new
     // holds the T - T0 new rows; state_in is the state after token T0-1 (ignored when T0 == 0).
@@ -233,14 +235,17 @@ __global__ __launch_bounds__(BLK) void encode_kernel(
     uint32_t *cw = cache + (size_t)bx * n_super_cap * D + c0;
     const h1 *xb = kv_new + (size_t)bx * (T - T0) * D + c0; // rows of tokens T0.. of this head
 
-    auto load_tok = [&](int t, h2 *x) {
-        if (CPL >= 2) {
+    // One token's CPL channels as NP aligned 32-bit words of the input row (an fp16 pair each; a
+    // one-channel lane takes the word its channel lies in and shifts at use).  The loads carry no
+    // arithmetic, and no 16-bit values the compiler would pack in pairs across the loop edge, so
+    // nothing waits for a load until its token is quantised.
+    using XW = uint32_t;
+    const h1 *xbw = xb - (CPL == 1 ? (c0 & 1) : 0);
+    const uint32_t xsh = CPL == 1 ? (uint32_t)(c0 & 1) * 16u : 0u;
+    auto load_tok = [&](int t, XW *x) {
 #pragma unroll
-            for (int p = 0; p < NP; p++)
-                x[p] = *reinterpret_cast<const h2 *>(xb + (size_t)(t - T0) * D + 2 * p);
-        } else {
-            x[0] = splat(xb[(size_t)(t - T0) * D]);
-        }
+        for (int p = 0; p < NP; p++)
+            x[p] = *reinterpret_cast<const XW *>(xbw + (size_t)(t - T0) * D + 2 * p);
     };
     // reciprocal of the current scale, refreshed right after every update (see quantize_enc_fast)
     float rs[NP][2];
@@ -251,23 +256,56 @@ __global__ __launch_bounds__(BLK) void encode_kernel(
 #pragma unroll
     for (int p = 0; p < NP; p++)
         refresh(p);
-    auto step = [&](const h2 *x, int tt, uint32_t *w) {
+    // quantise one token with the current state, advance the state; qf = the codes as floats.
+    // spec: branch-free speculative form (see quantize_enc_spec), the caller checks `worst`.
+    uint32_t worst = 0u;
+    auto advance = [&](auto spec, const XW *x, float *qf) {
 #pragma unroll
         for (int p = 0; p < NP; p++) {
-            const int q0 = quantize_enc_fast<BITS>(x[p].x, st[p].zp.x, st[p].sc.x, rs[p][0]);
-            w[CPL >= 2 ? 2 * p : 0] += (uint32_t)q0 << (BITS * tt);
-            int q1 = q0;
-            if (CPL >= 2) {
-                q1 = quantize_enc_fast<BITS>(x[p].y, st[p].zp.y, st[p].sc.y, rs[p][1]);
-                w[2 * p + 1] += (uint32_t)q1 << (BITS * tt);
+            const XW xw = CPL == 1 ? x[p] >> xsh : x[p];
+            const uint32_t zw = __builtin_bit_cast(uint32_t, st[p].zp);
+            float q0, q1;
+            if constexpr (decltype(spec)::value) {
+                q0 = quantize_enc_spec<BITS, false>(xw, zw, rs[p][0], worst);
+                q1 = CPL >= 2 ? quantize_enc_spec<BITS, true>(xw, zw, rs[p][1], worst) : q0;
+            } else {
+                q0 = quantize_enc_fast<BITS, false>(xw, zw, st[p].sc.x, rs[p][0]);
+                q1 = CPL >= 2 ? quantize_enc_fast<BITS, true>(xw, zw, st[p].sc.y, rs[p][1]) : q0;
             }
-            const h2 q = (h2){(h1)(short)q0, (h1)(short)q1};
-            update_pair(st[p], q, q * st[p].sc);
+            qf[CPL >= 2 ? 2 * p : 0] = q0;
+            if (CPL >= 2)
+                qf[2 * p + 1] = q1;
+            const h2 q = pack_codes(q0, q1);
+            update_pair_abs(st[p], pack_codes(__builtin_fabsf(q0), __builtin_fabsf(q1)), q * st[p].sc);
             refresh(p);
         }
     };
+    using Exact = std::integral_constant<bool, false>;
+    using Spec = std::integral_constant<bool, true>;
+    // partial words: token slot known at run time only
+    auto step = [&](const XW *x, int tt, uint32_t *w) {
+        float qf[CPL];
+        advance(Exact{}, x, qf);
+#pragma unroll
+        for (int c = 0; c < CPL; c++)
+            w[c] += (uint32_t)(int)qf[c] << (BITS * tt);
+    };
+    // Checkpoints: entry j is the state before token (j+1)*interval.  Words are stored in order,
+    // so the next boundary is tracked by comparison instead of a division per word.
+    int ck_next = -1, ck_j = 0;
+    if (sa.ckpt != nullptr) {
+        const int first_end = (T0 / TPW) * TPW + TPW;
+        ck_j = (first_end + sa.ckpt_interval - 1) / sa.ckpt_interval - 1;
+        ck_next = (ck_j + 1) * sa.ckpt_interval;
+    }
     // bias adds -QLO to the codes written now; keep selects codes of earlier tokens to preserve
     auto store_sg = [&](int sg, const uint32_t *w, uint32_t bias, uint32_t keep) {
+        const int tend = sg * TPW + TPW;
+        const bool ck_here = tend == ck_next;
+        if (ck_here) {
+            ck_next += sa.ckpt_interval;
+            ck_j++;
+        }
         if (!active)
             return;
         uint32_t *dst = cw + (size_t)sg * D;
@@ -286,13 +324,8 @@ __global__ __launch_bounds__(BLK) void encode_kernel(
             *reinterpret_cast<uint2 *>(dst) = make_uint2(o[0], o[1]);
         else
             dst[0] = o[0];
-        // state before token (j+1)*interval
-        const int tend = sg * TPW + TPW;
-        if (sa.ckpt != nullptr && tend <= T && tend % sa.ckpt_interval == 0) {
-            const int j = tend / sa.ckpt_interval - 1;
-            if (j < sa.n_ckpt_cap)
-                store_state_n<CPL>(sa.ckpt + (((size_t)bx * sa.n_ckpt_cap + j) * D + c0) * 2, st);
-        }
+        if (ck_here && tend <= T && ck_j - 1 < sa.n_ckpt_cap)
+            store_state_n<CPL>(sa.ckpt + (((size_t)bx * sa.n_ckpt_cap + (ck_j - 1)) * D + c0) * 2, st);
     };
 
     auto nib_mask = [](int k) { return k >= TPW ? 0xFFFFFFFFu : ((1u << (BITS * k)) - 1u); };
@@ -307,7 +340,7 @@ __global__ __launch_bounds__(BLK) void encode_kernel(
         for (int c = 0; c < CPL; c++)
             w[c] = 0u;
         for (; t < T && t / TPW == sg; t++) {
-            h2 x[NP];
+            XW x[NP];
             load_tok(t, x);
             step(x, t % TPW, w);
         }
@@ -315,44 +348,107 @@ __global__ __launch_bounds__(BLK) void encode_kernel(
         store_sg(sg, w, BIAS & nib_mask(hi) & ~nib_mask(lo), nib_mask(lo));
     }
 
-    // full words: no per-token conditions, inputs ENC_PF-1 groups of 8 tokens ahead
+    // full words: no per-token conditions, inputs ENC_PF-1 groups of 8 tokens ahead.  The loads
+    // are unconditional (index clamped to the last group): a load under a condition has to land
+    // before the code after the condition runs, which would expose the memory latency per group.
     const int sgb = t / TPW;                    // first full word
     const int nfull = (T - t) / TPW;
     const int ng = nfull * G8;
-    h2 xbuf[ENC_PF][8][NP];
+    XW xbuf[ENC_PF][8][NP];
     uint32_t w[CPL];
 #pragma unroll
     for (int c = 0; c < CPL; c++)
         w[c] = 0u;
+    // loads the next group of 8 rows; past the last group the same rows are loaded again
+    const h1 *xnext = xbw + (size_t)(t - T0) * D;
+    int gnext = 0;
+    auto load_next = [&](XW (*xg)[NP]) {
 #pragma unroll
-    for (int i = 0; i < ENC_PF - 1; i++)
-        if (i < ng) {
+        for (int tt = 0; tt < 8; tt++) {
 #pragma unroll
-            for (int tt = 0; tt < 8; tt++)
-                load_tok(t + i * 8 + tt, xbuf[i][tt]);
+            for (int p = 0; p < NP; p++)
+                xg[tt][p] = *reinterpret_cast<const XW *>(xnext + (size_t)tt * D + 2 * p);
         }
-    for (int g0 = 0; g0 < ng; g0 += ENC_PF) {
+        if (gnext < ng - 1) {
+            xnext += (size_t)8 * D;
+            gnext++;
+        }
+    };
+    // The codes of 16/BITS tokens fill 16 bits; their signed sum q << BITS*k is exact in one
+    // float (|sum| < 2^20), one fma per code, and two halves make the 32-bit word.
+    constexpr int TPA = 16 / BITS; // tokens per half word
+    constexpr int NA = 8 / TPA;    // half words an 8-token group fills
+    auto run_group = [&](auto spec, const XW (*xg)[NP], float (*acc)[NA]) {
 #pragma unroll
-        for (int i = 0; i < ENC_PF; i++) {
-            const int g = g0 + i;
-            if (g < ng) {
-                if (g + ENC_PF - 1 < ng) {
+        for (int tt = 0; tt < 8; tt++) {
+            float qf[CPL];
+            advance(spec, xg[tt], qf);
 #pragma unroll
-                    for (int tt = 0; tt < 8; tt++)
-                        load_tok(t + (g + ENC_PF - 1) * 8 + tt, xbuf[(i + ENC_PF - 1) % ENC_PF][tt]);
-                }
-                const int sub = G8 == 1 ? 0 : (g % G8) * 8;
-#pragma unroll
-                for (int tt = 0; tt < 8; tt++)
-                    step(xbuf[i][tt], sub + tt, w);
-                if (G8 == 1 || g % G8 == G8 - 1) {
-                    store_sg(sgb + g / G8, w, BIAS, 0u);
-#pragma unroll
-                    for (int c = 0; c < CPL; c++)
-                        w[c] = 0u;
-                }
+            for (int c = 0; c < CPL; c++) {
+                if (tt % TPA == 0)
+                    acc[c][tt / TPA] = qf[c];
+                else
+                    acc[c][tt / TPA] = __builtin_fmaf(qf[c], (float)(1u << (BITS * (tt % TPA))),
+                                                      acc[c][tt / TPA]);
             }
         }
+    };
+    // Lanes of one channel belong to waves that have a SIMD to themselves (that is when the
+    // launcher picks them), so they run a group speculatively without the per-token branch and
+    // repeat it exactly from the saved state when any lane of the wave came near a rounding
+    // boundary (about one group in sixty).
+    constexpr bool SPECULATE = CPL == 1;
+    auto do_group = [&](int g, const XW (*xg)[NP]) {
+        float acc[CPL][NA];
+        if (SPECULATE) {
+            Pair saved[NP];
+#pragma unroll
+            for (int p = 0; p < NP; p++)
+                saved[p] = st[p];
+            worst = 0u;
+            run_group(Spec{}, xg, acc);
+            if (__any(worst >= __float_as_uint(ENC_SPEC_LIMIT))) {
+#pragma unroll
+                for (int p = 0; p < NP; p++) {
+                    st[p] = saved[p];
+                    refresh(p);
+                }
+                run_group(Exact{}, xg, acc);
+            }
+        } else {
+            run_group(Exact{}, xg, acc);
+        }
+#pragma unroll
+        for (int c = 0; c < CPL; c++) {
+            uint32_t v = (uint32_t)(int)acc[c][0];
+            if (NA == 2)
+                v += (uint32_t)(int)acc[c][NA - 1] << 16;
+            w[c] += G8 == 1 ? v : v << (16 * (g % G8));
+        }
+        if (G8 == 1 || g % G8 == G8 - 1) {
+            store_sg(sgb + g / G8, w, BIAS, 0u);
+#pragma unroll
+            for (int c = 0; c < CPL; c++)
+                w[c] = 0u;
+        }
+    };
+    if (ng > 0) {
+#pragma unroll
+        for (int i = 0; i < ENC_PF - 1; i++)
+            load_next(xbuf[i]);
+        int g0 = 0;
+        for (; g0 + ENC_PF <= ng; g0 += ENC_PF) {
+#pragma unroll
+            for (int i = 0; i < ENC_PF; i++) {
+                load_next(xbuf[(i + ENC_PF - 1) % ENC_PF]);
+                do_group(g0 + i, xbuf[i]);
+            }
+        }
+        // at most ENC_PF-1 groups left; their inputs are already in xbuf[0 .. ENC_PF-2]
+#pragma unroll
+        for (int i = 0; i < ENC_PF - 1; i++)
+            if (g0 + i < ng)
+                do_group(g0 + i, xbuf[i]);
     }
     // ragged last word: codes of the tokens present, zero fields after them
     t += nfull * TPW;
@@ -362,7 +458,7 @@ __global__ __launch_bounds__(BLK) void encode_kernel(
         for (int c = 0; c < CPL; c++)
             w[c] = 0u;
         for (int tt = 0; tt < ntail; tt++) {
-            h2 x[NP];
+            XW x[NP];
             load_tok(t + tt, x);
             step(x, tt, w);
         }
@@ -370,6 +466,38 @@ __global__ __launch_bounds__(BLK) void encode_kernel(
     }
     if (state_out != nullptr && active)
         store_state_n<CPL>(state_out + ((size_t)bx * D + c0) * 2, st);
+}
+
+template <int BITS, int CPL, int BLK>
+__global__ __launch_bounds__(BLK) void encode_kernel(
+    uint32_t *__restrict__ cache, const h1 *__restrict__ kv_new,
+    const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
+    const h1 *__restrict__ be, const h1 *__restrict__ tg,
+    int BH, int H, int T0, int T, int D, int n_super_cap, const h1 *__restrict__ state_in,
+    h1 *__restrict__ state_out, Seg sa)
+{
+    encode_body<BITS, CPL, BLK>(cache, kv_new, zp, sc, al, be, tg, BH, H, T0, T, D, n_super_cap,
+                                state_in, state_out, sa);
+}
+
+// Two tensors of one shape (the K and V rows of the same tokens) in one launch: blockIdx.y picks
+// the tensor.  A prompt with few channels (small batch) leaves SIMDs idle when the tensors are
+// encoded one after the other; together they run in the time of one.
+struct EncTensor {
+    uint32_t *cache;
+    const h1 *kv_new, *zp, *sc, *al, *be, *tg, *state_in;
+    h1 *state_out, *ckpt;
+};
+
+template <int BITS, int CPL, int BLK>
+__global__ __launch_bounds__(BLK) void encode_pair_kernel(EncTensor k, EncTensor v, int BH, int H,
+                                                          int T0, int T, int D, int n_super_cap,
+                                                          Seg sa)
+{
+    const EncTensor e = blockIdx.y ? v : k;
+    sa.ckpt = e.ckpt;
+    encode_body<BITS, CPL, BLK>(e.cache, e.kv_new, e.zp, e.sc, e.al, e.be, e.tg, BH, H, T0, T, D,
+                                n_super_cap, e.state_in, e.state_out, sa);
 }
 
 // Shared tail of the two decode kernels: quantise the new token with the state after token T-1,
@@ -1168,7 +1296,7 @@ static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval, int b
 
 extern "C" {
 
-int adkv_abi_version(void) { return 7; }
+int adkv_abi_version(void) { return 8; }
 
 void adkv_set_mha_kernel(int use_matrix_cores) { g_mha_kernel = use_matrix_cores; }
 
@@ -1190,14 +1318,19 @@ const char *adkv_strerror(int code)
     }
 }
 
+// One tensor, or two of the same shape (v_cache != NULL) in one launch.
 static int encode_common(void *cache, const void *kv_new,
                          const void *zp, const void *sc, const void *alpha, const void *beta,
                          const void *tgt,
                          int B, int H, int T0, int T, int D, int n_super_cap,
                          const void *state_in, void *state_out, void *ckpt_out, int n_ckpt_cap,
-                         int ckpt_interval, void *stream, int bits = 4)
+                         int ckpt_interval, void *stream, int bits = 4,
+                         const EncTensor *second = nullptr)
 {
     if (!cache || !kv_new || !zp || !sc || !alpha || !beta || !tgt)
+        return ADKV_E_NULL;
+    if (second && (!second->cache || !second->kv_new || !second->zp || !second->sc || !second->al ||
+                   !second->be || !second->tg))
         return ADKV_E_NULL;
     if (bits != 2 && bits != 4)
         return ADKV_E_UNSUPPORTED;
@@ -1206,16 +1339,20 @@ static int encode_common(void *cache, const void *kv_new,
         return rc;
     if (T0 < 0 || T0 > T)
         return ADKV_E_SHAPE;
-    if (T0 > 0 && !state_in)
+    if (T0 > 0 && (!state_in || (second && !second->state_in)))
         return ADKV_E_NULL;
     const int tpw = 32 / bits;
     if ((T + tpw - 1) / tpw > n_super_cap)
         return ADKV_E_CAPACITY;
     if (((uintptr_t)cache & 15) || ((uintptr_t)kv_new & 3))
         return ADKV_E_ALIGN;
+    if (second && (((uintptr_t)second->cache & 15) || ((uintptr_t)second->kv_new & 3)))
+        return ADKV_E_ALIGN;
+    if (second && (ckpt_out == nullptr) != (second->ckpt == nullptr))
+        return ADKV_E_NULL; // both tensors keep checkpoints or neither does
     if ((rc = check_ckpt(ckpt_out, n_ckpt_cap, ckpt_interval, bits)))
         return rc;
-    if (T == T0 && (state_out == nullptr || state_out == state_in))
+    if (T == T0 && !second && (state_out == nullptr || state_out == state_in))
         return ADKV_OK;
     const int BH = B * H;
     hipStream_t st = (hipStream_t)stream;
@@ -1226,28 +1363,47 @@ static int encode_common(void *cache, const void *kv_new,
     seg.seg_tokens = T > 0 ? T : 1;
     seg.nseg = 1;
     seg.row_pitch = T + 1;
-    // widest lane that still leaves every SIMD with about two waves
+    // Lane width, measured on an MI355X (4096 tokens, ms for 65 536 / 131 072 / 196 608 / 262 144 /
+    // 524 288 channels): one channel per lane 0.29 / 0.44 / 0.60 / 0.74 / 1.38, two 0.43 / 0.44 /
+    // 0.55 / 0.60 / 1.17, four 0.78 / 0.78 / 0.78 / 0.79 / 1.18.  Up to two waves per SIMD the
+    // one-channel lanes win (each wave is paced by its own dependent chain, and only they run the
+    // branch-free speculative form); beyond that two channels share the packed fp16 updates.
+    // Four channels per lane never win and are not instantiated.
     const long channels = (long)BH * D;
-    int cpl = 4;
-    while (cpl > 1 && channels / (64L * cpl) < 2L * N_SIMD)
-        cpl >>= 1;
+    const long tensors = second ? 2 : 1;
+    int cpl = tensors * channels > 2L * 64 * N_SIMD + 32768 ? 2 : 1;
     if (const char *e = getenv("ADKV_ENCODE_CPL")) {
         const int v = atoi(e);
-        if (v == 1 || v == 2 || v == 4)
+        if (v == 1 || v == 2)
             cpl = v;
     }
     const long lanes = channels / cpl;
-    const dim3 grid((unsigned)((lanes + 255) / 256)), block(256);
+    const dim3 grid((unsigned)((lanes + 255) / 256), (unsigned)tensors), block(256);
+    EncTensor first;
+    first.cache = (uint32_t *)cache;
+    first.kv_new = (const h1 *)kv_new;
+    first.zp = (const h1 *)zp;
+    first.sc = (const h1 *)sc;
+    first.al = (const h1 *)alpha;
+    first.be = (const h1 *)beta;
+    first.tg = (const h1 *)tgt;
+    first.state_in = (const h1 *)state_in;
+    first.state_out = (h1 *)state_out;
+    first.ckpt = (h1 *)ckpt_out;
 #define ADKV_ENC(BB, C)                                                                          \
-    hipLaunchKernelGGL((encode_kernel<BB, C, 256>), grid, block, 0, st, (uint32_t *)cache,       \
-                       (const h1 *)kv_new, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,    \
-                       (const h1 *)beta, (const h1 *)tgt, BH, H, T0, T, D, n_super_cap,          \
-                       (const h1 *)state_in, (h1 *)state_out, seg)
+    do {                                                                                         \
+        if (second)                                                                              \
+            hipLaunchKernelGGL((encode_pair_kernel<BB, C, 256>), grid, block, 0, st, first,      \
+                               *second, BH, H, T0, T, D, n_super_cap, seg);                      \
+        else                                                                                     \
+            hipLaunchKernelGGL((encode_kernel<BB, C, 256>), grid, block, 0, st, first.cache,     \
+                               first.kv_new, first.zp, first.sc, first.al, first.be, first.tg,   \
+                               BH, H, T0, T, D, n_super_cap, first.state_in, first.state_out,    \
+                               seg);                                                             \
+    } while (0)
 #define ADKV_ENC_CPL(BB)                                                                         \
     do {                                                                                         \
-        if (cpl == 4)                                                                            \
-            ADKV_ENC(BB, 4);                                                                     \
-        else if (cpl == 2)                                                                       \
+        if (cpl == 2)                                                                            \
             ADKV_ENC(BB, 2);                                                                     \
         else                                                                                     \
             ADKV_ENC(BB, 1);                                                                     \
@@ -1287,6 +1443,34 @@ int adkv_append_kv(void *cache, const void *kv_new,
     return encode_common(cache, kv_new, zp, sc, alpha, beta, tgt, B, H, T0, T0 + n_new, D,
                          n_super_cap, state_io, state_io, ckpt, n_ckpt_cap, ckpt_interval, stream,
                          bits);
+}
+
+int adkv_append_kv_pair(void *k_cache, void *v_cache, const void *k_new, const void *v_new,
+                        const void *const *k_params, const void *const *v_params,
+                        int B, int H, int T0, int n_new, int D, int n_super_cap, int bits,
+                        void *k_state_io, void *v_state_io, void *k_ckpt, void *v_ckpt,
+                        int n_ckpt_cap, int ckpt_interval, void *stream)
+{
+    if (!k_params || !v_params || !k_state_io || !v_state_io)
+        return ADKV_E_NULL;
+    if (n_new < 0)
+        return ADKV_E_SHAPE;
+    if (n_new == 0)
+        return ADKV_OK;
+    EncTensor v;
+    v.cache = (uint32_t *)v_cache;
+    v.kv_new = (const h1 *)v_new;
+    v.zp = (const h1 *)v_params[0];
+    v.sc = (const h1 *)v_params[1];
+    v.al = (const h1 *)v_params[2];
+    v.be = (const h1 *)v_params[3];
+    v.tg = (const h1 *)v_params[4];
+    v.state_in = (const h1 *)v_state_io;
+    v.state_out = (h1 *)v_state_io;
+    v.ckpt = (h1 *)v_ckpt;
+    return encode_common(k_cache, k_new, k_params[0], k_params[1], k_params[2], k_params[3],
+                         k_params[4], B, H, T0, T0 + n_new, D, n_super_cap, k_state_io, k_state_io,
+                         k_ckpt, n_ckpt_cap, ckpt_interval, stream, bits, &v);
 }
 
 int adkv_encode_kv(void *cache, const void *kv_new,

@@ -21,7 +21,7 @@ import math
 
 import torch
 
-from ..kernel.gemv import append_kv, decode_fused, decode_fused_workspace_bytes
+from ..kernel.gemv import append_kv_pair, decode_fused, decode_fused_workspace_bytes
 
 SCALE_MIN = math.exp(-4.0)  # kept for API parity; the fp16 recurrence never clamps
 SCALE_MAX = math.exp(4.0)
@@ -153,14 +153,14 @@ class KVCacheLayer_ADKV:
         """Quantise ``[B, H, T, C]`` keys/values as tokens ``quant_len ..`` of the stream."""
         v = self._view
         S = self._ckpt_interval
-        append_kv(self._key_buf, key_states.to(torch.float16).contiguous(),
-                  v(key_zp_init), v(key_scale_init), v(key_alpha), v(key_beta), v(key_quant_target),
-                  self._quant_len, self._key_state, ckpt=self._key_ckpt, ckpt_interval=S, bits=self._bits)
-        append_kv(self._value_buf, value_states.to(torch.float16).contiguous(),
-                  v(value_zp_init), v(value_scale_init), v(value_alpha), v(value_beta),
-                  v(value_quant_target),
-                  self._quant_len, self._value_state, ckpt=self._value_ckpt, ckpt_interval=S,
-                  bits=self._bits)
+        append_kv_pair(
+            self._key_buf, self._value_buf,
+            key_states.to(torch.float16).contiguous(), value_states.to(torch.float16).contiguous(),
+            (v(key_zp_init), v(key_scale_init), v(key_alpha), v(key_beta), v(key_quant_target)),
+            (v(value_zp_init), v(value_scale_init), v(value_alpha), v(value_beta),
+             v(value_quant_target)),
+            self._quant_len, self._key_state, self._value_state,
+            k_ckpt=self._key_ckpt, v_ckpt=self._value_ckpt, ckpt_interval=S, bits=self._bits)
         self._quant_len += key_states.shape[2]
 
     def prefill(self, key_states, value_states,

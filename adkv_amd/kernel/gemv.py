@@ -336,6 +336,67 @@ def append_kv(
     return kv_cache
 
 
+def append_kv_pair(
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    k_new: torch.Tensor,
+    v_new: torch.Tensor,
+    k_params,
+    v_params,
+    T0: int,
+    k_state: torch.Tensor,
+    v_state: torch.Tensor,
+    *,
+    k_ckpt: torch.Tensor | None = None,
+    v_ckpt: torch.Tensor | None = None,
+    ckpt_interval: int = 0,
+    bits: int = 4,
+) -> None:
+    """``append_kv`` for the K and V rows of the same tokens in one launch (the two calls of
+    src/adkv/hf/llama_adkv.py:144-153 made together).  Results are byte-identical to two
+    ``append_kv`` calls; at small batch the pair takes the time of one tensor because channels are
+    the encoder's only parallel axis.  ``k_params`` / ``v_params``: the five ``[nh, DIM]`` fp16
+    tensors ``(zp, sc, alpha, beta, quant_target)``.
+    """
+    _chk(k_new.dtype == torch.float16 and v_new.dtype == torch.float16, "kv_new must be float16")
+    _chk(k_cache.dtype == torch.uint8 and v_cache.dtype == torch.uint8, "kv_cache must be uint8")
+    _chk(k_cache.is_contiguous() and v_cache.is_contiguous(),
+         "kv_cache must be contiguous (written in place)")
+    _chk(k_new.shape == v_new.shape and k_cache.shape == v_cache.shape,
+         "K and V must have the same shapes")
+    B, nh, n, DIM = k_new.shape
+    kp = _params(k_params, ("k_zp", "k_sc", "k_alpha", "k_beta", "k_t"), nh, DIM)
+    vp = _params(v_params, ("v_zp", "v_sc", "v_alpha", "v_beta", "v_t"), nh, DIM)
+    n_super_cap = k_cache.shape[2]
+    _chk(k_cache.shape[3] * _TILE == DIM, "kv_cache channel groups do not match kv_new head dim")
+    _chk(T0 >= 0, "T0 must be non-negative")
+    _chk(bits in (2, 4), "bits must be 2 or 4")
+    tps = 32 // bits
+    need = (T0 + n + tps - 1) // tps
+    _chk(need <= n_super_cap,
+         f"kv_cache capacity too small: need {need} supergroups for {T0 + n} tokens, have {n_super_cap}")
+    _chk(DIM in _DIMS, "DIM must be 128, 256 or 512")
+    for st in (k_state, v_state):
+        _chk(st.dtype == torch.float16 and st.is_contiguous() and st.numel() == B * nh * DIM * 2,
+             "state must be contiguous fp16 [B,nh,DIM,2]")
+    _chk((k_ckpt is None) == (v_ckpt is None), "give both checkpoint tensors or neither")
+    dev = _need_device(k_cache, v_cache, k_new, v_new, *kp, *vp, k_state, v_state)
+    kc, ccap, civ = _ckpt_args(k_ckpt, ckpt_interval, B, nh, DIM, bits)
+    vc, vcap, _ = _ckpt_args(v_ckpt, ckpt_interval, B, nh, DIM, bits)
+    _chk(ccap == vcap, "K and V checkpoint tensors must have the same capacity")
+    if n == 0:
+        return
+    xk, xv = k_new.contiguous(), v_new.contiguous()
+    arr = _lib.C.c_void_p * 5
+    with torch.cuda.device(dev):
+        rc = _lib.lib().adkv_append_kv_pair(
+            k_cache.data_ptr(), v_cache.data_ptr(), xk.data_ptr(), xv.data_ptr(),
+            arr(*[t.data_ptr() for t in kp]), arr(*[t.data_ptr() for t in vp]),
+            B, nh, T0, n, DIM, n_super_cap, bits, k_state.data_ptr(), v_state.data_ptr(),
+            kc, vc, ccap, civ, _lib.current_stream_ptr(dev))
+    _lib.check(rc, "append_kv_pair")
+
+
 def softmax_scale_mask(logits: torch.Tensor, scaling: float,
                        mask: torch.Tensor | None = None) -> torch.Tensor:
     """``softmax(logits.float()*scaling + mask) -> fp16`` in one launch.

@@ -170,6 +170,26 @@ def encode_main(args):
     a1.record(); torch.cuda.synchronize()
     append_us = a0.elapsed_time(a1) * 1e3 / n_app
 
+    # K and V rows of the same tokens in one launch (what the cache layer's prefill does)
+    pv = synth.make_params(H, D, seed=4).to(dev)
+    xv = synth.make_v(B, H, T, D, dtype=torch.float16, device=dev)
+    cache_v = synth.alloc_cache(B, H, T + 8, D, dev)
+    cache_k2 = synth.alloc_cache(B, H, T + 8, D, dev)
+    st_k, st_v = torch.zeros_like(state), torch.zeros_like(state)
+
+    def prefill_pair():
+        gemv.append_kv_pair(cache_k2, cache_v, xp, xv, p.astuple(), pv.astuple(), 0, st_k, st_v)
+
+    prefill_pair()
+    torch.cuda.synchronize()
+    p0, p1 = ev(), ev()
+    p0.record()
+    for _ in range(args.steps):
+        prefill_pair()
+    p1.record(); torch.cuda.synchronize()
+    pair_ms = p0.elapsed_time(p1) / args.steps
+    pair_same = bool(torch.equal(cache_k2[:, :, :T // 8], cache[:, :, :T // 8]))
+
     # bit-exactness of the codes: two sampled heads against the oracle, whole stream
     from oracle import oracle as O
     np16 = lambda t: t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.float16)
@@ -191,6 +211,9 @@ def encode_main(args):
                                f"then {n_app} single-token appends with carried state",
                    "batch": B, "heads": H, "head_dim": D, "ctx": T, "bits": 4, "ckpt_interval": S},
         "append_us_per_token_step": append_us,
+        "kv_pair": {"ms_per_prefill": pair_ms, "tokens_per_s": B * T / (pair_ms * 1e-3),
+                    "k_codes_equal_single_tensor_run": pair_same,
+                    "note": "K and V of every token in one launch (adkv_append_kv_pair)"},
         "codes_bit_exact_vs_oracle": exact,
         "roofline": {"kernel": "encode_kernel", "bound": "hbm", "achieved": achieved,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,

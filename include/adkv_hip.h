@@ -141,6 +141,21 @@ int adkv_append_kv(void *cache, const void *kv_new,
                    int B, int H, int T0, int n_new, int D, int n_super_cap, int bits,
                    void *state_io, void *ckpt, int n_ckpt_cap, int ckpt_interval, void *stream);
 
+/*
+ * adkv_append_kv for the K and the V rows of the same tokens in ONE launch: the two calls that
+ * KVCacheLayer_ADKV._append_tokens makes back to back (src/adkv/hf/llama_adkv.py:144-153).  Both
+ * tensors share every shape argument; k_params / v_params are host arrays of five device
+ * pointers {zp, sc, alpha, beta, tgt}; the checkpoint tensors are both given or both NULL.
+ * Results are byte-identical to two adkv_append_kv calls.  Channels are the only parallel axis
+ * of the encoder, so a long prompt at a small batch (B*H*D below ~130 000 channels) leaves half
+ * of the device idle per tensor; paired, both tensors finish in the time of one.
+ */
+int adkv_append_kv_pair(void *k_cache, void *v_cache, const void *k_new, const void *v_new,
+                        const void *const *k_params, const void *const *v_params,
+                        int B, int H, int T0, int n_new, int D, int n_super_cap, int bits,
+                        void *k_state_io, void *v_state_io, void *k_ckpt, void *v_ckpt,
+                        int n_ckpt_cap, int ckpt_interval, void *stream);
+
 int adkv_forward_qk_ex(const void *q, void *k_cache, const void *k_new, void *logits,
                        const void *zp, const void *sc, const void *alpha, const void *beta,
                        const void *tgt,

@@ -472,6 +472,46 @@ def _gqa_case(gpu, oracle, B, Hkv, G, T, S, seed=0, bits=4):
         assert torch.equal(ck.view(torch.int16), ckv.view(torch.int16))
 
 
+@pytest.mark.parametrize("bits,B,H,D,cuts,S", [
+    (4, 2, 3, 128, (0, 5, 8, 19, 64, 100), 16),   # one channel per lane (few channels)
+    (4, 1, 2, 512, (0, 3, 24), 0),
+    (4, 16, 32, 128, (0, 40), 8),                 # 65 536 channels per tensor: still one per lane
+    (4, 64, 32, 128, (0, 17), 0),                 # 262 144 channels per tensor: two per lane
+    (2, 2, 2, 128, (0, 33, 34, 64, 150), 32),
+])
+def test_paired_append_equals_oracle(gpu, oracle, bits, B, H, D, cuts, S):
+    """K and V rows of the same tokens quantised in one launch: both caches, both carried states
+    and both checkpoint tensors equal the oracle's for each tensor on its own."""
+    T = cuts[-1]
+    tps = 32 // bits
+    ncap = T // S + 1 if S else 0
+    data, want = [], []
+    for i in range(2):
+        x, p = _inputs(B, H, T, D, seed=11 + i, bits=bits)
+        pn = [_np16(t) for t in p.astuple()]
+        with oracle.code_bits(bits):
+            c = oracle.alloc_cache(B, H, T + tps, D)
+            st = oracle.encode_kv_f16(c, _np16(x), *pn)
+            ck = _oracle_ckpts(oracle, c, pn, T, S, ncap) if S else None
+        data.append((x.to(gpu), [t.to(gpu) for t in p.astuple()]))
+        want.append((c, st, ck))
+    caches = [synth.alloc_cache(B, H, T + tps, D, gpu, bits=bits) for _ in range(2)]
+    states = [torch.zeros(B, H, D, 2, dtype=torch.float16, device=gpu) for _ in range(2)]
+    cks = [torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=gpu) if S else None
+           for _ in range(2)]
+    for a, b in zip(cuts[:-1], cuts[1:]):
+        gemv.append_kv_pair(caches[0], caches[1], data[0][0][:, :, a:b], data[1][0][:, :, a:b],
+                            data[0][1], data[1][1], a, states[0], states[1],
+                            k_ckpt=cks[0], v_ckpt=cks[1], ckpt_interval=S, bits=bits)
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert np.array_equal(caches[i].cpu().numpy(), want[i][0]), i
+        assert np.array_equal(_np16(states[i]).view(np.uint16), want[i][1]), i
+        if S:
+            n = T // S
+            assert np.array_equal(_np16(cks[i]).view(np.uint16)[:, :, :n], want[i][2][:, :, :n]), i
+
+
 @pytest.mark.parametrize("B,Hkv,G,T,S", [
     (1, 2, 4, 0, 0), (2, 2, 4, 5, 0), (1, 3, 2, 8, 0), (2, 2, 4, 71, 0), (1, 2, 8, 40, 0),
     (2, 3, 4, 530, 64), (1, 2, 2, 256, 64), (1, 1, 8, 200, 16), (1, 5, 4, 1025, 0)])
