@@ -7,6 +7,8 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <type_traits>
+#include <utility>
 #include <stdint.h>
 
 #pragma clang fp contract(off)
@@ -21,6 +23,34 @@ __device__ __forceinline__ uint32_t as_u32(h2 h) { return __builtin_bit_cast(uin
 __device__ __forceinline__ h2 pk_fma(h2 a, h2 b, h2 c) { return __builtin_elementwise_fma(a, b, c); }
 __device__ __forceinline__ h2 pk_abs(h2 a) { return as_h2(as_u32(a) & 0x7FFF7FFFu); }
 __device__ __forceinline__ h2 splat(h1 x) { return (h2){x, x}; }
+
+// f(integral_constant<int, 0>), ..., f(integral_constant<int, N-1>): a loop whose index is a
+// compile-time constant inside the body (register arrays indexed by it stay in registers).
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>)
+{
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// A decode loop over n items whose buffers rotate with period P: whole rotations without a
+// single condition in them (conditions around loads or stores make the compiler wait for every
+// load in flight), then the up to P-1 items left.  body(item, integral_constant slot).
+template <int P, typename F>
+__device__ __forceinline__ void rotate_over(int n, F &&body)
+{
+    int i0 = 0;
+    for (; i0 + P <= n; i0 += P)
+        static_for<P>([&](auto ic) { body(i0 + decltype(ic)::value, ic); });
+    static_for<P - 1>([&](auto ic) {
+        if (i0 + decltype(ic)::value < n)
+            body(i0 + decltype(ic)::value, ic);
+    });
+}
 
 // One channel pair's filter state and fixed parameters (two channels packed per register).
 struct Pair {

@@ -231,7 +231,7 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
 
     uint4 buf[GPF];
     uint32_t nbc[G::NP][2], nbn[G::NP][2]; // byte streams of the current / the next supergroup
-    uint2 areg[8];
+    uint2 areg[8] = {}; // read (and discarded) once before the first unit has filled it
 #pragma unroll
     for (int i = 0; i < GPF; i++)
         buf[i] = (i < nfull) ? cb[(size_t)i * G::VPS] : make_uint4(0, 0, 0, 0);
@@ -239,41 +239,38 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
         code_bytes<BITS>(buf[0], nbc);
         lk.fill(lut, nbc, lane_copy, 0);
     }
-    for (int sg0 = 0; sg0 < nfull; sg0 += GPF) {
+    // one supergroup, nothing conditional in it; i = its buffer in the rotation
+    auto body = [&](int sg, auto ic) {
+        constexpr int i = decltype(ic)::value;
+        // bytes of supergroup sg+1 (stale data past the end: looked up, never used)
+        code_bytes<BITS>(buf[(i + 1) % GPF], nbn);
+        // unconditional, clamped to the segment's last supergroup: a load inside a branch makes
+        // the next wait cover every load in flight, this one included
+        buf[i] = cb[(size_t)min(sg + GPF, nfull - 1) * G::VPS];
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < GPF; i++) {
-            const int sg = sg0 + i;
-            if (sg < nfull) {
-                // bytes of supergroup sg+1 (stale data past the end: looked up, never used)
-                code_bytes<BITS>(buf[(i + 1) % GPF], nbn);
-                // unconditional, clamped to the segment's last supergroup: a load inside a branch
-                // makes the next wait cover every load in flight, this one included
-                buf[i] = cb[(size_t)min(sg + GPF, nfull - 1) * G::VPS];
-                __builtin_amdgcn_sched_barrier(0);
+        for (int hf = 0; hf < UPS; hf++) {
+            const int unit = sg * UPS + hf;
+            const bool into_next_sg = hf == UPS - 1;
 #pragma unroll
-                for (int hf = 0; hf < UPS; hf++) {
-                    const int unit = sg * UPS + hf;
-                    const bool into_next_sg = hf == UPS - 1;
+            for (int t = 0; t < 3; t++)
+                token(t, into_next_sg ? nbn : nbc, into_next_sg ? 0 : hf + 1);
+            // the tile reads of the previous unit were issued before these three tokens overwrote
+            // its first rows (LDS operations of a wave execute in order); nothing is stored for
+            // the unit before the first
+            emit_finish(areg, unit - 1, unit > 0 ? 8 : 0);
 #pragma unroll
-                    for (int t = 0; t < 3; t++)
-                        token(t, into_next_sg ? nbn : nbc, into_next_sg ? 0 : hf + 1);
-                    // the tile reads of the previous unit were issued before these three tokens
-                    // overwrote its first rows (LDS operations of a wave execute in order)
-                    if (unit > 0)
-                        emit_finish(areg, unit - 1, 8);
-#pragma unroll
-                    for (int t = 3; t < 8; t++)
-                        token(t, into_next_sg ? nbn : nbc, into_next_sg ? 0 : hf + 1);
-                    emit_read(areg);
-                }
-#pragma unroll
-                for (int p = 0; p < G::NP; p++) {
-                    nbc[p][0] = nbn[p][0];
-                    nbc[p][1] = nbn[p][1];
-                }
-            }
+            for (int t = 3; t < 8; t++)
+                token(t, into_next_sg ? nbn : nbc, into_next_sg ? 0 : hf + 1);
+            emit_read(areg);
         }
-    }
+#pragma unroll
+        for (int p = 0; p < G::NP; p++) {
+            nbc[p][0] = nbn[p][0];
+            nbc[p][1] = nbn[p][1];
+        }
+    };
+    rotate_over<GPF>(nfull, body);
     if (nfull > 0)
         emit_finish(areg, nfull * UPS - 1, 8);
     if (!last)
@@ -422,43 +419,38 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
         code_bytes<BITS>(buf[0], nbc);
         lk.fill(lut, nbc, lane_copy, 0);
     }
-    for (int sg0 = 0; sg0 < nfull; sg0 += GPF) {
+    // one supergroup, nothing conditional in it; i = its buffer in the rotation
+    auto body = [&](int sg, auto ic) {
+        constexpr int i = decltype(ic)::value;
+        code_bytes<BITS>(buf[(i + 1) % GPF], nbn);
+        buf[i] = cb[(size_t)min(sg + GPF, nfull - 1) * G::VPS]; // unconditional: see qk_gqa_kernel
 #pragma unroll
-        for (int i = 0; i < GPF; i++) {
-            const int sg = sg0 + i;
-            if (sg < nfull) {
-                code_bytes<BITS>(buf[(i + 1) % GPF], nbn);
-                buf[i] = cb[(size_t)min(sg + GPF, nfull - 1) * G::VPS]; // unconditional: see qk_gqa_kernel
+        for (int hf = 0; hf < UPS; hf++) {
+            const int unit = sg * UPS + hf;
+            const int ws = (i * UPS + hf) % WPF; // compile-time after unrolling
+            __builtin_amdgcn_sched_barrier(0);
+            const bool into_next_sg = hf == UPS - 1;
 #pragma unroll
-                for (int hf = 0; hf < UPS; hf++) {
-                    const int unit = sg * UPS + hf;
-                    const int ws = (i * UPS + hf) % WPF; // compile-time after unrolling
-                    uint4 wcur[NB];
+            for (int t = 0; t < 4; t++)
+                token(t, into_next_sg ? nbn : nbc, into_next_sg ? 0 : hf + 1);
+            contract(kh, wbuf[ws], 0);
 #pragma unroll
-                    for (int n = 0; n < NB; n++)
-                        wcur[n] = wbuf[ws][n];
+            for (int t = 4; t < 8; t++)
+                token(t, into_next_sg ? nbn : nbc, into_next_sg ? 0 : hf + 1);
+            contract(kh, wbuf[ws], 1);
+            // reloaded once used: an earlier load into a second register set costs copies at the
+            // loop edge, which wait for the load they move
 #pragma unroll
-                    for (int n = 0; n < NB; n++)
-                        wbuf[ws][n] = load_w(n, min(unit + WPF, nunits - 1));
-                    __builtin_amdgcn_sched_barrier(0);
-                    const bool into_next_sg = hf == UPS - 1;
-#pragma unroll
-                    for (int t = 0; t < 4; t++)
-                        token(t, into_next_sg ? nbn : nbc, into_next_sg ? 0 : hf + 1);
-                    contract(kh, wcur, 0);
-#pragma unroll
-                    for (int t = 4; t < 8; t++)
-                        token(t, into_next_sg ? nbn : nbc, into_next_sg ? 0 : hf + 1);
-                    contract(kh, wcur, 1);
-                }
-#pragma unroll
-                for (int p = 0; p < G::NP; p++) {
-                    nbc[p][0] = nbn[p][0];
-                    nbc[p][1] = nbn[p][1];
-                }
-            }
+            for (int n = 0; n < NB; n++)
+                wbuf[ws][n] = load_w(n, min(unit + WPF, nunits - 1));
         }
-    }
+#pragma unroll
+        for (int p = 0; p < G::NP; p++) {
+            nbc[p][0] = nbn[p][0];
+            nbc[p][1] = nbn[p][1];
+        }
+    };
+    rotate_over<GPF>(nfull, body);
 
     if (last) {
         // ragged tail, then the appended token: a handful of tokens, plain fp32 multiply-adds

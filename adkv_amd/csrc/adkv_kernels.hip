@@ -139,8 +139,18 @@ __device__ __forceinline__ void store_state_n(h1 *dst, const Pair *st)
         *reinterpret_cast<h2 *>(dst) = (h2){st[0].zp.x, st[0].sc.x};
 }
 
-// Which (head, segment) this lane works on.  Units beyond the end are clamped to the last one and
+// Which (head, segment) this lane works on.  Units are ordered segment-major and every segment's
+// run of units is padded to whole waves, so all lanes of a wave work on the same segment and
+// everything derived from it (token range, trip counts) is wave-uniform: the decode loops then
+// branch on scalars instead of masking lanes.  Units past the end are clamped to a valid one and
 // flagged inactive: they compute but never store.
+template <int LPH>
+static inline long padded_units(int BH, int nseg)
+{
+    constexpr int UPW = 64 / LPH; // units per wave
+    return (long)nseg * (((long)BH + UPW - 1) / UPW * UPW);
+}
+
 template <int D, int CPL, int BLK>
 struct Unit {
     int bx, seg, lh, c0;
@@ -148,14 +158,16 @@ struct Unit {
     __device__ __forceinline__ Unit(int BH, int nseg)
     {
         using G = Geo<D, CPL>;
+        constexpr int UPW = 64 / G::LPH;
+        const int per_seg = (BH + UPW - 1) / UPW * UPW;
         const long gl = (long)blockIdx.x * BLK + threadIdx.x;
-        long u = gl / G::LPH;
+        const long slot = gl / G::LPH;
         lh = (int)(gl % G::LPH);
-        active = u < (long)BH * nseg;
-        if (!active)
-            u = (long)BH * nseg - 1;
-        bx = (int)(u / nseg);
-        seg = (int)(u % nseg);
+        const int sg = __builtin_amdgcn_readfirstlane((int)(slot / per_seg));
+        const int b = (int)(slot % per_seg);
+        active = sg < nseg && b < BH;
+        seg = sg < nseg ? sg : nseg - 1;
+        bx = b < BH ? b : BH - 1;
         c0 = lh * CPL;
     }
 };
@@ -660,37 +672,34 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
             for (int p = 0; p < G::NP; p++)
                 lk[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
     }
-    for (int sg0 = 0; sg0 < nfull; sg0 += PF) {
+    // One supergroup; i = its buffer in the rotation (compile-time).  Nothing in here is
+    // conditional: the trip count is wave-uniform, the prefetch index is clamped, and the
+    // reduction of the previous supergroup stores nothing when there is none (sg == 0).
+    auto body = [&](int sg, auto ic) {
+        constexpr int i = decltype(ic)::value;
+        float tmp[8], part[8];
+        // bytes of supergroup sg+1 (stale data past the end: looked up, never used)
+        pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
+        red_read(tmp);
+        {
+            // unconditional, clamped to the segment's last supergroup: a load inside a branch
+            // makes the next wait cover every load in flight, this one included
+            const int sgp = min(sg + PF, nfull - 1);
 #pragma unroll
-        for (int i = 0; i < PF; i++) {
-            const int sg = sg0 + i;
-            if (sg < nfull) {
-                float tmp[8], part[8];
-                // bytes of supergroup sg+1 (stale data past the end: looked up, never used)
-                pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
-                if (sg > 0)
-                    red_read(tmp);
-                {
-                    // unconditional, clamped to the segment's last supergroup: a load inside a
-                    // branch makes the next wait cover every load in flight, this one included
-                    const int sgp = min(sg + PF, nfull - 1);
-#pragma unroll
-                    for (int v = 0; v < G::NV; v++)
-                        buf[i][v] = cb[(size_t)sgp * G::VPS + v];
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int t = 0; t < 3; t++)
-                    token(t, lk, nb, part[t]);
-                if (sg > 0)
-                    red_finish(tmp, sg - 1, 8); // early, so tmp[] is dead while part[] fills up
-#pragma unroll
-                for (int t = 3; t < 8; t++)
-                    token(t, lk, nb, part[t]);
-                red_write(part);
-            }
+            for (int v = 0; v < G::NV; v++)
+                buf[i][v] = cb[(size_t)sgp * G::VPS + v];
         }
-    }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < 3; t++)
+            token(t, lk, nb, part[t]);
+        red_finish(tmp, sg - 1, sg > 0 ? 8 : 0); // early, so tmp[] is dead while part[] fills up
+#pragma unroll
+        for (int t = 3; t < 8; t++)
+            token(t, lk, nb, part[t]);
+        red_write(part);
+    };
+    rotate_over<PF>(nfull, body);
     if (nfull > 0) {
         float tmp[8];
         red_read(tmp);
@@ -831,27 +840,23 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
             for (int p = 0; p < G::NP; p++)
                 lk[p][t] = lut_get(lut, nb[p][t & 1], lane_copy, t >> 1);
     }
-    for (int sg0 = 0; sg0 < nfull; sg0 += PF) {
+    // one supergroup, nothing conditional in it (see qk_kernel); i = its buffer in the rotation
+    auto body = [&](int sg, auto ic) {
+        constexpr int i = decltype(ic)::value;
+        pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
+        const int sgp = min(sg + PF, nfull - 1);
 #pragma unroll
-        for (int i = 0; i < PF; i++) {
-            const int sg = sg0 + i;
-            if (sg < nfull) {
-                pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
-                const uint4 wcur = wbuf[i];
-                {
-                    const int sgp = min(sg + PF, nfull - 1); // unconditional: see qk_kernel
+        for (int v = 0; v < G::NV; v++)
+            buf[i][v] = cb[(size_t)sgp * G::VPS + v];
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int v = 0; v < G::NV; v++)
-                        buf[i][v] = cb[(size_t)sgp * G::VPS + v];
-                    wbuf[i] = load_w(sgp);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int t = 0; t < 8; t++)
-                    token(t, lk, nb, wcur);
-            }
-        }
-    }
+        for (int t = 0; t < 8; t++)
+            token(t, lk, nb, wbuf[i]);
+        // the weights are reloaded once their last token is done: loading them earlier into a
+        // second register set costs copies at the loop edge, which wait for the load they move
+        wbuf[i] = load_w(sgp);
+    };
+    rotate_over<PF>(nfull, body);
 
     if (last) {
         const int ntail = (t1 - t0) & 7;
@@ -1180,7 +1185,7 @@ static Seg plan_segments(void *ckpt, int n_ckpt_cap, int ckpt_interval, int BH, 
     // launch length in units of one checkpoint interval
     auto cost = [&](int m) {
         const int nseg = (avail + m - 1) / m;
-        const long threads = (long)BH * nseg * lph;
+        const long threads = (lph == 32 ? padded_units<32>(BH, nseg) : padded_units<64>(BH, nseg)) * lph;
         if (D == 512 || threads < 1024L * 256)
             return (double)m;                        // small workgroups: no round structure to model
         const long wgs = (threads + 1023) / 1024;
@@ -1222,7 +1227,7 @@ static void launch_units(long threads, int big, F256 f256, FBIG fbig)
 
 #define ADKV_LAUNCH(KERNEL, DD, CC, BIG, ...)                                                   \
     launch_units(                                                                               \
-        (long)BH * seg.nseg * (DD / CC), BIG,                                                   \
+        padded_units<DD / CC>(BH, seg.nseg) * (DD / CC), BIG,                                                  \
         [&](dim3 g, dim3 b) { hipLaunchKernelGGL((KERNEL<DD, CC, 256>), g, b, 0, st, __VA_ARGS__); }, \
         [&](dim3 g, dim3 b) { hipLaunchKernelGGL((KERNEL<DD, CC, BIG>), g, b, 0, st, __VA_ARGS__); })
 
@@ -1243,7 +1248,7 @@ static void launch_units(long threads, int big, F256 f256, FBIG fbig)
 // (their LDS tile leaves room for one workgroup per CU either way).
 #define ADKV_LAUNCH_GQA(KERNEL, BB, GQV, ...)                                                      \
     do {                                                                                            \
-        const long threads = (long)BH * seg.nseg * 32;                                              \
+        const long threads = padded_units<32>(BH, seg.nseg) * 32;                                            \
         /* eight heads per KV head need more registers than a 16-wave workgroup leaves a lane */   \
         if (GQV <= 4 && threads >= 1024L * 256)                                                     \
             hipLaunchKernelGGL((KERNEL<BB, (GQV <= 4 ? GQV : 1), 1024>), dim3((unsigned)((threads + 1023) / 1024)),  \

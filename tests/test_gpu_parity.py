@@ -221,6 +221,7 @@ def _oracle_ckpts(oracle, cache_np, pn, T, S, ncap):
 @pytest.mark.parametrize("B,H,T,D,S", [
     (1, 2, 100, 128, 16), (2, 3, 64, 128, 16), (1, 2, 63, 128, 8), (1, 1, 257, 128, 64),
     (2, 2, 48, 256, 16), (1, 2, 40, 512, 8), (3, 2, 15, 128, 16), (1, 2, 1024, 128, 256),
+    (1, 3, 100, 128, 16), (1, 5, 70, 128, 8),   # odd head counts: a wave's second half is padding
 ])
 def test_checkpointed_segments(gpu, oracle, B, H, T, D, S):
     """Encoder checkpoints are the oracle's replayed states; decode over independently replayed
@@ -514,7 +515,7 @@ def test_paired_append_equals_oracle(gpu, oracle, bits, B, H, D, cuts, S):
 
 @pytest.mark.parametrize("B,Hkv,G,T,S", [
     (1, 2, 4, 0, 0), (2, 2, 4, 5, 0), (1, 3, 2, 8, 0), (2, 2, 4, 71, 0), (1, 2, 8, 40, 0),
-    (2, 3, 4, 530, 64), (1, 2, 2, 256, 64), (1, 1, 8, 200, 16), (1, 5, 4, 1025, 0)])
+    (2, 3, 4, 530, 64), (1, 2, 2, 256, 64), (1, 1, 8, 200, 16), (1, 5, 4, 1025, 0), (1, 3, 4, 200, 16)])
 def test_grouped_query_kernels(gpu, oracle, B, Hkv, G, T, S):
     _gqa_case(gpu, oracle, B, Hkv, G, T, S, seed=T % 7)
 
