@@ -50,6 +50,84 @@ def test_quant_f32_bit_exact(gpu, oracle, B, T, C, bits):
         assert np.array_equal(_bits(got).numpy(), want[key].view(np.int32)), key
 
 
+def _run_no_seq(gpu, x, p, bits, dtype=torch.float32):
+    from adkv_amd.train import quant_f32
+    B, T, C = x.shape
+    ql, qu = -2 ** (bits - 1), 2 ** (bits - 1) - 1
+    zp = torch.empty(B, C, device=gpu)
+    sc = torch.empty(B, C, device=gpu)
+    xhat, codes, _, _ = quant_f32(
+        x.to(dtype).to(gpu), p["alpha"].to(gpu), p["beta"].to(gpu), p["tgt"].to(gpu), ql, qu,
+        math.exp(-4.0), math.exp(4.0), zp_state=zp, sc_state=sc,
+        zp_init=p["zp"].to(gpu), sc_init=p["sc"].to(gpu), want_codes=True)
+    torch.cuda.synchronize()
+    return xhat, codes, zp, sc
+
+
+def _same_bits_or_both_nan(got, want):
+    g, w = got.detach().cpu().float().numpy(), np.asarray(want, dtype=np.float32)
+    both_nan = np.isnan(g) & np.isnan(w)
+    return np.array_equal(np.where(both_nan, 0, g.view(np.int32)), np.where(both_nan, 0, w.view(np.int32)))
+
+
+@pytest.mark.parametrize("B,T,C,bits", [(1, 7, 64, 4), (2, 8, 100, 4), (2, 37, 100, 4), (3, 257, 130, 2),
+                                        (1, 100, 512, 8), (1, 1024, 4096, 4)])
+def test_quant_f32_without_state_sequence_bit_exact(gpu, oracle, B, T, C, bits):
+    """The production form (no state sequence recorded) runs groups of 8 tokens speculatively and
+    repeats the ones that came near a rounding boundary: same codes, values and state as the oracle."""
+    p = _params(C, 7 + T, bits)
+    g = torch.Generator().manual_seed(T)
+    x = torch.randn(B, T, C, generator=g) * 2.0
+    x[:, :, ::17] += 6.0 * torch.sin(0.02 * torch.arange(T, dtype=torch.float32))[None, :, None]
+    want = oracle.quant_f32(x.numpy(), *[p[k].numpy() for k in ("zp", "sc", "alpha", "beta", "tgt")], bits=bits)
+    xhat, codes, zp, sc = _run_no_seq(gpu, x, p, bits)
+    assert np.array_equal(codes.cpu().numpy(), want["codes"])
+    for got, key in ((xhat, "xhat"), (zp, "zp"), (sc, "sc")):
+        assert np.array_equal(_bits(got).numpy(), want[key].view(np.int32)), key
+
+
+def test_quant_f32_rounding_boundaries_and_non_finite_inputs(gpu, oracle):
+    """First tokens placed on rounding boundaries (x - zp = (k + 1/2) * sc and its fp32 neighbours),
+    and NaN / infinite / huge inputs scattered over the stream: the speculative path has to notice
+    all of them and fall back; NaN handling follows torch.clamp (NaN stays NaN, its code is 0)."""
+    B, T, C, bits = 2, 64, 256, 4
+    p = _params(C, 11, bits)
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(B, T, C, generator=g) * 2.0
+    k = torch.arange(C, dtype=torch.float32) % 16 - 8.0
+    tie = p["zp"] + (k + 0.5) * p["sc"]
+    x[0, 0] = tie
+    x[1, 0] = torch.nextafter(tie, torch.full_like(tie, 1e9))
+    x[1, 8] = torch.nextafter(x[1, 8], torch.full_like(tie, -1e9))
+    x[0, 5, 3] = float("nan")
+    x[0, 17, 40] = float("inf")
+    x[1, 30, 41] = float("-inf")
+    x[1, 9, 100] = 3.0e38
+    x[0, 33, 101] = -1.0e30
+    want = oracle.quant_f32(x.numpy(), *[p[k].numpy() for k in ("zp", "sc", "alpha", "beta", "tgt")], bits=bits)
+    xhat, codes, zp, sc = _run_no_seq(gpu, x, p, bits)
+    assert np.array_equal(codes.cpu().numpy(), want["codes"])
+    assert _same_bits_or_both_nan(xhat, want["xhat"])
+    assert _same_bits_or_both_nan(zp, want["zp"])
+    assert _same_bits_or_both_nan(sc, want["sc"])
+    assert np.isnan(want["zp"]).any()            # the NaN really reached the state of its channel
+
+
+@pytest.mark.parametrize("dtype,C", [(torch.float16, 130), (torch.bfloat16, 129), (torch.float16, 65)])
+def test_quant_f32_half_inputs_odd_and_even_widths(gpu, oracle, dtype, C):
+    """16-bit inputs take aligned 32-bit loads when rows allow it (even C) and plain 16-bit loads
+    otherwise (odd C): both give the oracle's result on the values as read."""
+    B, T = 2, 50
+    p = _params(C, 3, 4)
+    x = (torch.randn(B, T, C, generator=torch.Generator().manual_seed(C)) * 1.5).to(dtype)
+    want = oracle.quant_f32(x.float().numpy(), *[p[k].numpy() for k in ("zp", "sc", "alpha", "beta", "tgt")])
+    xhat, codes, zp, sc = _run_no_seq(gpu, x.float(), p, 4, dtype=dtype)
+    assert np.array_equal(codes.cpu().numpy(), want["codes"])
+    assert torch.equal(xhat.cpu(), torch.from_numpy(want["xhat"]).to(dtype))
+    assert np.array_equal(_bits(zp).numpy(), want["zp"].view(np.int32))
+    assert np.array_equal(_bits(sc).numpy(), want["sc"].view(np.int32))
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_quant_f32_half_inputs_in_place_and_chunked(gpu, oracle, dtype):
     """16-bit buffers are read up to fp32 and written back rounded (as the reference's Triton kernel
