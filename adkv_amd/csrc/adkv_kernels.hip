@@ -1149,9 +1149,9 @@ static int check_common(int B, int H, int T, int D, int n_super_cap)
 
 static inline int lanes_per_head(int D) { return D == 128 ? 32 : 64; }
 
-// Waves a SIMD should hold for packed-f16 issue to run near full rate, and SIMDs on the device.
 #include "adkv_gqa_kernels.h"
 
+// Waves a SIMD should hold for packed-f16 issue to run near full rate, and SIMDs on the device.
 constexpr int WAVES_PER_SIMD_TARGET = 4;
 constexpr int N_SIMD = 256 * 4;
 
