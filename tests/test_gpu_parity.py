@@ -420,6 +420,68 @@ def test_decode_fused_equals_three_calls(gpu, B, H, T, D, S, masked):
         assert torch.equal(vk.view(torch.int16), vk2.view(torch.int16))
 
 
+@pytest.mark.parametrize("H,Hq,T,S,bits", [(4, 4, 300, 64, 4), (2, 8, 530, 64, 4), (2, 8, 200, 32, 2)])
+def test_decode_step_replays_from_a_captured_graph(gpu, H, Hq, T, S, bits):
+    """The library never allocates, clears memory or synchronises, so a decode step can be captured
+    in a HIP graph by a serving loop.  Every replay (with eager work and synchronisations between
+    replays) must reproduce the eager step: outputs, weights and the caches with the appended token."""
+    B, D = 2, 128
+    tps = 32 // bits
+    kp = [t.to(gpu) for t in synth.make_params(H, D, seed=3, bits=bits).astuple()]
+    vp = [t.to(gpu) for t in synth.make_params(H, D, seed=4, bits=bits).astuple()]
+    k = synth.make_k(B, H, T + 1, D, dtype=torch.float16).to(gpu)
+    v = synth.make_v(B, H, T + 1, D, dtype=torch.float16).to(gpu)
+    q = synth.make_q(B, Hq, D).to(gpu)
+    scaling = D ** -0.5
+    ncap = (T + tps) // S + 1
+
+    def fresh():
+        kc = synth.alloc_cache(B, H, T + tps, D, gpu, bits=bits)
+        vc = synth.alloc_cache(B, H, T + tps, D, gpu, bits=bits)
+        kk = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=gpu)
+        vk = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=gpu)
+        ks = torch.zeros(B, H, D, 2, dtype=torch.float16, device=gpu)
+        vs = torch.zeros(B, H, D, 2, dtype=torch.float16, device=gpu)
+        gemv.append_kv_pair(kc, vc, k[:, :, :T], v[:, :, :T], kp, vp, 0, ks, vs,
+                            k_ckpt=kk, v_ckpt=vk, ckpt_interval=S, bits=bits)
+        return kc, vc, kk, vk
+
+    ws_bytes = gemv.decode_fused_workspace_bytes(B, Hq, H, T, D, ncap, S)
+    ws = torch.empty(ws_bytes + 256, dtype=torch.uint8, device=gpu)
+    ws = ws[(-ws.data_ptr()) % 256:][:ws_bytes]
+
+    def step(kc, vc, kk, vk):
+        return gemv.decode_fused(q, kc, vc, k[:, :, T:], v[:, :, T:], kp, vp, T, scaling, None,
+                                 k_ckpt=kk, v_ckpt=vk, ckpt_interval=S, bits=bits, workspace=ws)
+
+    e = fresh()
+    out_e, w_e = step(*e)
+    torch.cuda.synchronize()
+    out_e, w_e = out_e.clone(), w_e.clone()
+
+    gbuf = fresh()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(*gbuf)                                  # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g, w_g = step(*gbuf)
+    for rep in range(4):
+        out_g.zero_()
+        w_g.zero_()
+        graph.replay()
+        junk = (k.float() * 1.5).sum()               # the program's own eager work between replays
+        torch.cuda.synchronize()
+        assert torch.isfinite(junk)
+        assert torch.equal(out_g.view(torch.int16), out_e.view(torch.int16)), rep
+        assert torch.equal(w_g.view(torch.int16), w_e.view(torch.int16)), rep
+        for a, b in zip(gbuf, e):
+            assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), rep
+
+
 # ------------------------------------------------------------------ grouped-query / matrix-core kernels
 def _gqa_case(gpu, oracle, B, Hkv, G, T, S, seed=0, bits=4):
     """One QK + OV pass with G query heads per KV head against the oracle run once per group member
