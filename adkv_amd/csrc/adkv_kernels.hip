@@ -1245,33 +1245,37 @@ static void launch_units(long threads, int big, F256 f256, FBIG fbig)
     }
 
 // Matrix-core kernels (head dim 128): 16-wave workgroups for big launches, 8-wave ones otherwise
-// (their LDS tile leaves room for one workgroup per CU either way).
-#define ADKV_LAUNCH_GQA(KERNEL, BB, GQV, ...)                                                      \
+// (their LDS tile leaves room for one workgroup per CU either way).  Eight query heads per KV head
+// need ~138 registers per lane, more than the 128 a 16-wave workgroup leaves: qk_gqa_kernel still
+// gains from four waves per SIMD with a dozen cold values spilled (cfg5 KV shape, 64 query heads:
+// 563 -> 530 us with 4-bit codes, 518 -> 425 us with 2-bit ones), ov_gqa_kernel spills
+// accumulators and loses (421 -> 533 us, 346 -> 747 us), so BIG8 says which of the two this is.
+#define ADKV_LAUNCH_GQA(KERNEL, BIG8, BB, GQV, ...)                                                \
     do {                                                                                            \
-        const long threads = padded_units<32>(BH, seg.nseg) * 32;                                            \
-        /* eight heads per KV head need more registers than a 16-wave workgroup leaves a lane */   \
-        if (GQV <= 4 && threads >= 1024L * 256)                                                     \
-            hipLaunchKernelGGL((KERNEL<BB, (GQV <= 4 ? GQV : 1), 1024>), dim3((unsigned)((threads + 1023) / 1024)),  \
+        const long threads = padded_units<32>(BH, seg.nseg) * 32;                                   \
+        constexpr int GBIG = (GQV <= 4 || BIG8) ? GQV : 1; /* unused instantiation otherwise */     \
+        if ((GQV <= 4 || BIG8) && threads >= 1024L * 256)                                           \
+            hipLaunchKernelGGL((KERNEL<BB, GBIG, 1024>), dim3((unsigned)((threads + 1023) / 1024)), \
                                dim3(1024), 0, st, __VA_ARGS__);                                     \
         else                                                                                        \
             hipLaunchKernelGGL((KERNEL<BB, GQV, 512>), dim3((unsigned)((threads + 511) / 512)),     \
                                dim3(512), 0, st, __VA_ARGS__);                                      \
     } while (0)
 
-#define ADKV_DISPATCH_GQ_BITS(KERNEL, BB, ...)                                                     \
+#define ADKV_DISPATCH_GQ_BITS(KERNEL, BIG8, BB, ...)                                               \
     switch (GQ) {                                                                                   \
-    case 1: ADKV_LAUNCH_GQA(KERNEL, BB, 1, __VA_ARGS__); break;                                     \
-    case 2: ADKV_LAUNCH_GQA(KERNEL, BB, 2, __VA_ARGS__); break;                                     \
-    case 4: ADKV_LAUNCH_GQA(KERNEL, BB, 4, __VA_ARGS__); break;                                     \
-    case 8: ADKV_LAUNCH_GQA(KERNEL, BB, 8, __VA_ARGS__); break;                                     \
+    case 1: ADKV_LAUNCH_GQA(KERNEL, BIG8, BB, 1, __VA_ARGS__); break;                               \
+    case 2: ADKV_LAUNCH_GQA(KERNEL, BIG8, BB, 2, __VA_ARGS__); break;                               \
+    case 4: ADKV_LAUNCH_GQA(KERNEL, BIG8, BB, 4, __VA_ARGS__); break;                               \
+    case 8: ADKV_LAUNCH_GQA(KERNEL, BIG8, BB, 8, __VA_ARGS__); break;                               \
     default: return ADKV_E_UNSUPPORTED;                                                             \
     }
 
-#define ADKV_DISPATCH_GQ(KERNEL, ...)                                                              \
+#define ADKV_DISPATCH_GQ(KERNEL, BIG8, ...)                                                        \
     if (bits == 4) {                                                                                \
-        ADKV_DISPATCH_GQ_BITS(KERNEL, 4, __VA_ARGS__)                                               \
+        ADKV_DISPATCH_GQ_BITS(KERNEL, BIG8, 4, __VA_ARGS__)                                         \
     } else {                                                                                        \
-        ADKV_DISPATCH_GQ_BITS(KERNEL, 2, __VA_ARGS__)                                               \
+        ADKV_DISPATCH_GQ_BITS(KERNEL, BIG8, 2, __VA_ARGS__)                                         \
     }
 
 // Whether single-query-head launches (GQ == 1, head dim 128) also take the matrix-core kernels:
@@ -1521,7 +1525,7 @@ int adkv_forward_qk_gqa(const void *q, void *k_cache, const void *k_new, void *l
     if (ld)
         seg.row_pitch = ld;
     if (D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha())) {
-        ADKV_DISPATCH_GQ(qk_gqa_kernel, (const h1 *)q, (uint4 *)k_cache, (const h1 *)k_new,
+        ADKV_DISPATCH_GQ(qk_gqa_kernel, true, (const h1 *)q, (uint4 *)k_cache, (const h1 *)k_new,
                          (h1 *)logits, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,
                          (const h1 *)beta, (const h1 *)tgt, BH, H, T, n_super_cap, (h1 *)state_out,
                          seg);
@@ -1602,7 +1606,7 @@ int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void
             return ADKV_E_ALIGN;
     }
     if (D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha())) {
-        ADKV_DISPATCH_GQ(ov_gqa_kernel, (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new,
+        ADKV_DISPATCH_GQ(ov_gqa_kernel, false, (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new,
                          (h1 *)out, (float *)workspace, (const h1 *)zp, (const h1 *)sc,
                          (const h1 *)alpha, (const h1 *)beta, (const h1 *)tgt, BH, H, T, n_super_cap,
                          (h1 *)state_out, seg);

@@ -582,6 +582,55 @@ def test_grouped_query_kernels(gpu, oracle, B, Hkv, G, T, S):
     _gqa_case(gpu, oracle, B, Hkv, G, T, S, seed=T % 7)
 
 
+@pytest.mark.parametrize("G,bits", [(4, 4), (8, 4), (2, 2), (8, 2)])
+def test_grouped_query_kernels_in_16_wave_workgroups(gpu, oracle, G, bits):
+    """A launch big enough for the 16-wave workgroups (128 KV heads x 64 segments = 8192 units):
+    the instantiations the small cases above never reach, including the eight-head QK kernel
+    that runs them with spilled registers.  The GPU does the whole problem; the oracle (far too
+    slow for all of it) replays three sampled (sequence, KV head) pairs from the GPU-encoded cache."""
+    B, Hkv, D, S = 16, 8, 128, 16
+    T = 64 * S + 5
+    Hq = Hkv * G
+    tps = 32 // bits
+    x, p = _inputs(B, Hkv, T + 1, D, seed=G, bits=bits)
+    pg = [t.to(gpu) for t in p.astuple()]
+    g = torch.Generator().manual_seed(50 + G)
+    q = torch.randn(B, Hq, 1, D, generator=g).half()
+    attn = torch.softmax(2.0 * torch.randn(B, Hq, T + 1, generator=g), dim=-1).half()
+    ncap = (T + tps) // S + 1
+    cache = synth.alloc_cache(B, Hkv, T + tps, D, gpu, bits=bits)
+    st = torch.zeros(B, Hkv, D, 2, dtype=torch.float16, device=gpu)
+    ck = torch.zeros(B, Hkv, ncap, D, 2, dtype=torch.float16, device=gpu)
+    gemv.append_kv(cache, x[:, :, :T].to(gpu), *pg, 0, st, ckpt=ck, ckpt_interval=S, bits=bits)
+    torch.cuda.synchronize()
+    cache0 = cache.cpu().numpy()
+    kc, vc, ckv = cache.clone(), cache.clone(), ck.clone()
+    xnew = x[:, :, T:T + 1].to(gpu)
+    logits = gemv.forward_qk(q.to(gpu), kc, xnew, *pg, T, SMIN, SMAX, ckpt=ck, ckpt_interval=S, bits=bits)
+    out = gemv.forward_ov(attn.to(gpu), vc, xnew, *pg, SMIN, SMAX, ckpt=ckv, ckpt_interval=S, bits=bits)
+    torch.cuda.synchronize()
+    lg = _np16(logits).astype(np.float64).reshape(B, Hkv, G, T + 1)
+    og = _np16(out).astype(np.float64).reshape(B, Hkv, G, D)
+    qn, an = _np16(q).reshape(B, Hkv, G, D), _np16(attn).reshape(B, Hkv, G, T + 1)
+    for (b, h) in [(0, 0), (B - 1, Hkv - 1), (7, 3)]:
+        pn = [_np16(t)[h:h + 1] for t in p.astuple()]
+        xn = _np16(x)[b:b + 1, h:h + 1, T:T + 1]
+        with oracle.code_bits(bits):
+            want = oracle.alloc_cache(1, 1, T + tps, D)
+            oracle.encode_kv_f16(want, _np16(x)[b:b + 1, h:h + 1, :T], *pn)
+            assert np.array_equal(cache0[b:b + 1, h:h + 1], want), (b, h)
+            for j in range(G):
+                c = want.copy()
+                l, _ = oracle.forward_qk_f16(qn[b:b + 1, h:h + 1, j], c, xn, *pn, T)
+                c2 = want.copy()
+                o, _ = oracle.forward_ov_f16(an[b:b + 1, h:h + 1, j], c2, xn, *pn)
+                assert np.all(np.abs(lg[b, h, j] - l[0, 0]) <= _ulp16(l[0, 0]) + 1e-3), (b, h, j)
+                assert np.all(np.abs(og[b, h, j] - o[0, 0]) <= _ulp16(o[0, 0]) + 1e-3), (b, h, j)
+        assert np.array_equal(kc[b:b + 1, h:h + 1].cpu().numpy(), c), (b, h)
+        assert np.array_equal(vc[b:b + 1, h:h + 1].cpu().numpy(), c2), (b, h)
+    assert torch.equal(ck.view(torch.int16), ckv.view(torch.int16))
+
+
 @pytest.mark.parametrize("B,H,T,S", [(2, 3, 0, 0), (1, 2, 7, 0), (2, 2, 130, 0), (2, 3, 530, 64)])
 def test_matrix_core_kernels_for_equal_heads(gpu, oracle, B, H, T, S):
     """The same matrix-core kernels with one query head per KV head (selected by the tuning knob)
