@@ -84,5 +84,29 @@ def check(rc: int, what: str) -> None:
         raise RuntimeError(f"{what}: {msg}")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def current_stream_ptr(device) -> int:
+    """The device's current stream as a ``hipStream_t`` value."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)          # one C call instead of building a Stream object
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def device_guard(device):
+    """Context that makes ``device`` current for a launch; free when it already is."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(device)

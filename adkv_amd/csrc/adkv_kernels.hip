@@ -953,13 +953,15 @@ __device__ __forceinline__ float block_reduce(float v, float *sm, bool is_max)
 // x[k] = logits*scaling + mask for the SM_KEEP elements of this thread in the chunk that starts at
 // `base` (-inf past the end of the row); 16-byte accesses wherever a whole vector lies inside the
 // row (rows are only 2-byte aligned: the hardware takes unaligned vector accesses).
+template <int NV = SM_NV, int NT = SM_BLOCK>
 __device__ __forceinline__ void softmax_load_chunk(const h1 *l, const float *mk, int n, int base,
-                                                   float scaling, float *x, float &mx)
+                                                   float scaling, float *x, float &mx,
+                                                   int tid = (int)threadIdx.x)
 {
     mx = -INFINITY;
 #pragma unroll
-    for (int v = 0; v < SM_NV; v++) {
-        const int i0 = base + (v * SM_BLOCK + (int)threadIdx.x) * SM_VEC;
+    for (int v = 0; v < NV; v++) {
+        const int i0 = base + (v * NT + tid) * SM_VEC;
         float *xv = x + v * SM_VEC;
         if (i0 + SM_VEC <= n) {
             uint4 raw;
@@ -997,11 +999,13 @@ __device__ __forceinline__ void softmax_load_chunk(const h1 *l, const float *mk,
 }
 
 // w[i] = fp16(x[k] * inv) for the same elements
-__device__ __forceinline__ void softmax_store_chunk(h1 *w, int n, int base, const float *x, float inv)
+template <int NV = SM_NV, int NT = SM_BLOCK>
+__device__ __forceinline__ void softmax_store_chunk(h1 *w, int n, int base, const float *x, float inv,
+                                                    int tid = (int)threadIdx.x)
 {
 #pragma unroll
-    for (int v = 0; v < SM_NV; v++) {
-        const int i0 = base + (v * SM_BLOCK + (int)threadIdx.x) * SM_VEC;
+    for (int v = 0; v < NV; v++) {
+        const int i0 = base + (v * NT + tid) * SM_VEC;
         const float *xv = x + v * SM_VEC;
         if (i0 + SM_VEC <= n) {
             uint32_t o[4];
@@ -1017,6 +1021,38 @@ __device__ __forceinline__ void softmax_store_chunk(h1 *w, int n, int base, cons
                     w[i0 + k] = (h1)(xv[k] * inv);
         }
     }
+}
+
+// Short rows: one wave per row (four rows per workgroup), the row in registers, reductions across
+// the wave only.  A workgroup per row would spend most of its time on two barriers for a handful of
+// elements per thread; rows of a few hundred tokens are the common decode case.
+template <int NV>
+__global__ __launch_bounds__(SM_BLOCK) void softmax_wave_kernel(
+    const h1 *__restrict__ logits, h1 *__restrict__ weights, const float *__restrict__ mask,
+    int rows, int n, long ld, int rows_per_mask_row, float scaling)
+{
+    const int row = blockIdx.x * (SM_BLOCK / 64) + (threadIdx.x >> 6);
+    if (row >= rows)
+        return;
+    const int lane = threadIdx.x & 63;
+    const h1 *l = logits + (size_t)row * ld;
+    h1 *w = weights + (size_t)row * ld;
+    const float *mk = mask ? mask + (size_t)(row / rows_per_mask_row) * n : nullptr;
+    float x[NV * SM_VEC], mx;
+    softmax_load_chunk<NV, 64>(l, mk, n, 0, scaling, x, mx, lane);
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1)
+        mx = fmaxf(mx, __shfl_xor(mx, m, 64));
+    float sum = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NV * SM_VEC; k++) {
+        x[k] = __expf(x[k] - mx);
+        sum += x[k];
+    }
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1)
+        sum += __shfl_xor(sum, m, 64);
+    softmax_store_chunk<NV, 64>(w, n, 0, x, 1.0f / sum, lane);
 }
 
 // One workgroup per row.  A row of up to SM_CHUNK elements is read once and kept in registers;
@@ -1676,6 +1712,22 @@ int adkv_softmax_ex(const void *logits, void *weights, const void *mask,
         return ADKV_E_SHAPE;
     if (ld == 0)
         ld = n;
+    if (n <= 64 * SM_VEC * 4) {
+        // short rows: a wave per row, the row in 8, 16 or 32 registers per lane
+        const dim3 grid((unsigned)((rows + SM_BLOCK / 64 - 1) / (SM_BLOCK / 64)));
+#define ADKV_SM_WAVE(NVW)                                                                           \
+    hipLaunchKernelGGL(softmax_wave_kernel<NVW>, grid, dim3(SM_BLOCK), 0, (hipStream_t)stream,      \
+                       (const h1 *)logits, (h1 *)weights, (const float *)mask, rows, n, (long)ld,   \
+                       mask ? rows_per_mask_row : 1, scaling)
+        if (n <= 64 * SM_VEC)
+            ADKV_SM_WAVE(1);
+        else if (n <= 64 * SM_VEC * 2)
+            ADKV_SM_WAVE(2);
+        else
+            ADKV_SM_WAVE(4);
+#undef ADKV_SM_WAVE
+        return check_launch();
+    }
     const int64_t need = adkv_softmax_workspace_bytes(rows, n);
     if (need == 0 || !workspace || rows > 65535) {
         // one workgroup per row; rows that do not fit in its registers are read three times

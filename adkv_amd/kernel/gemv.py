@@ -29,6 +29,12 @@ def _chk(cond: bool, msg: str) -> None:
 
 def _need_device(*tensors: torch.Tensor) -> torch.device:
     dev = tensors[0].device
+    if dev.type == "cuda":
+        for t in tensors:
+            if t.device != dev:
+                break
+        else:
+            return dev
     for t in tensors:
         _chk(t.is_cuda, "ADKV kernels need every tensor on a HIP device; there is no CPU path")
         _chk(t.device == dev, "ADKV kernels need all tensors on the same device")
@@ -36,15 +42,19 @@ def _need_device(*tensors: torch.Tensor) -> torch.device:
 
 
 def _params(tensors, names, nh, dim):
-    out = []
-    for t, n in zip(tensors, names):
-        _chk(t.dtype == torch.float16, f"{n} must be float16")
-        out.append(t)
+    want = nh * dim
     res = []
-    for t, n in zip(out, names):
-        _chk(t.numel() == nh * dim, f"{n} must have nh*DIM = {nh * dim} elements")
-        res.append(t.contiguous())
-    return res
+    for t in tensors:
+        if t.dtype != torch.float16 or t.numel() != want:
+            break
+        res.append(t if t.is_contiguous() else t.contiguous())
+    else:
+        return res
+    for t, n in zip(tensors, names):      # same order of complaints as the reference's checks
+        _chk(t.dtype == torch.float16, f"{n} must be float16")
+    for t, n in zip(tensors, names):
+        _chk(t.numel() == want, f"{n} must have nh*DIM = {want} elements")
+    raise AssertionError("unreachable")
 
 
 def _pitch(n: int) -> int:
@@ -150,7 +160,7 @@ def forward_qk(
         _chk(state_out.dtype == torch.float16 and state_out.is_contiguous()
              and state_out.numel() == B * nh * DIM * 2, "state_out must be contiguous fp16 [B,nh,DIM,2]")
     cp, ccap, civ = _ckpt_args(ckpt, ckpt_interval, B, nh, DIM, bits)
-    with torch.cuda.device(dev):
+    with _lib.device_guard(dev):
         rc = _lib.lib().adkv_forward_qk_gqa(
             q_flat.data_ptr(), k_cache.data_ptr(), k_new_flat.data_ptr(), o.data_ptr(),
             zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
@@ -220,7 +230,7 @@ def forward_ov(
         ws_bytes = L.adkv_forward_ov_gqa_workspace_bytes(B, nq, nh, T, DIM, ccap, civ)
         if ws_bytes:
             ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.device_guard(dev):
         rc = L.adkv_forward_ov_gqa(
             attn_flat.data_ptr(), v_cache.data_ptr(), v_new_flat.data_ptr(), o.data_ptr(),
             zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
@@ -272,7 +282,7 @@ def encode_kv(
     if B * nh * T == 0 and state_out is None:
         return kv_cache
     cp, ccap, civ = _ckpt_args(ckpt, ckpt_interval, B, nh, DIM)
-    with torch.cuda.device(dev):
+    with _lib.device_guard(dev):
         rc = _lib.lib().adkv_encode_kv_ex(
             kv_cache.data_ptr(), kv_new_flat.data_ptr(),
             zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
@@ -326,7 +336,7 @@ def append_kv(
     if n == 0:
         return kv_cache
     x = kv_new.contiguous()
-    with torch.cuda.device(dev):
+    with _lib.device_guard(dev):
         rc = _lib.lib().adkv_append_kv(
             kv_cache.data_ptr(), x.data_ptr(),
             zp.data_ptr(), sc.data_ptr(), al.data_ptr(), be.data_ptr(), tg.data_ptr(),
@@ -388,7 +398,7 @@ def append_kv_pair(
         return
     xk, xv = k_new.contiguous(), v_new.contiguous()
     arr = _lib.C.c_void_p * 5
-    with torch.cuda.device(dev):
+    with _lib.device_guard(dev):
         rc = _lib.lib().adkv_append_kv_pair(
             k_cache.data_ptr(), v_cache.data_ptr(), xk.data_ptr(), xv.data_ptr(),
             arr(*[t.data_ptr() for t in kp]), arr(*[t.data_ptr() for t in vp]),
@@ -423,7 +433,7 @@ def softmax_scale_mask(logits: torch.Tensor, scaling: float,
     L = _lib.lib()
     wsb = L.adkv_softmax_workspace_bytes(B * nh, n)
     ws = torch.empty(wsb, dtype=torch.uint8, device=dev) if wsb else None
-    with torch.cuda.device(dev):
+    with _lib.device_guard(dev):
         rc = L.adkv_softmax_ex(lg.data_ptr(), out.data_ptr(), mptr, B * nh, n, ld, rpm, float(scaling),
                                _ptr(ws), wsb, _lib.current_stream_ptr(dev))
     _lib.check(rc, "softmax_scale_mask")
@@ -502,7 +512,7 @@ def decode_fused(
     wld = int(L.adkv_row_pitch(n))
     weights = torch.empty((B, nq, wld), dtype=torch.float16, device=dev)
     arr = _lib.C.c_void_p * 5
-    with torch.cuda.device(dev):
+    with _lib.device_guard(dev):
         rc = L.adkv_decode_fused(
             qf.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), knf.data_ptr(), vnf.data_ptr(),
             arr(*[t.data_ptr() for t in kp]), arr(*[t.data_ptr() for t in vp]),

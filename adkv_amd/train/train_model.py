@@ -63,7 +63,7 @@ def quant_f32(x: torch.Tensor, alpha: torch.Tensor, beta: torch.Tensor, target: 
     p = lambda t: None if t is None else t.data_ptr()
     sb = x.stride(0) if B > 1 else T * max(x.stride(1), C)
     st = x.stride(1) if T > 1 else C
-    with torch.cuda.device(dev):
+    with _lib.device_guard(dev):
         rc = _lib.lib().adkv_quant_f32(
             x.data_ptr(), out.data_ptr(), p(codes), zp_state.data_ptr(), sc_state.data_ptr(),
             p(zi), p(si), al.data_ptr(), be.data_ptr(), tg.data_ptr(), p(zs), p(ss),
