@@ -38,11 +38,30 @@ constexpr int PF = ADKV_PF; // supergroups in flight per lane
 template <int D, int CPL>
 struct Geo {
     static constexpr int LPH = D / CPL;       // lanes per head
-    static constexpr int NV = CPL / 4;        // 16-byte vectors per lane per supergroup
     static constexpr int NP = CPL / 2;        // channel pairs per lane
-    static constexpr int VPS = D / 4;         // 16-byte vectors per supergroup of one head
+    // a lane's CPL code words of one supergroup, loaded as 16-byte vectors (8 bytes when the lane
+    // owns only two channels)
+    using Vec = typename std::conditional<CPL >= 4, uint4, uint2>::type;
+    static constexpr int WPV = sizeof(Vec) / 4; // 32-bit channel words per vector
+    static constexpr int NV = CPL / WPV;        // vectors per lane per supergroup
+    static constexpr int VPS = D / WPV;         // vectors per supergroup of one head
     static_assert(LPH == 32 || LPH == 64, "a head must fit in one wave");
+    static_assert(CPL == 2 || CPL % 4 == 0, "two channels per lane, or a multiple of four");
 };
+
+__device__ __forceinline__ void vec_words(const uint4 &u, uint32_t *w)
+{
+    w[0] = u.x; w[1] = u.y; w[2] = u.z; w[3] = u.w;
+}
+__device__ __forceinline__ void vec_words(const uint2 &u, uint32_t *w)
+{
+    w[0] = u.x; w[1] = u.y;
+}
+__device__ __forceinline__ void words_vec(const uint32_t *w, uint4 &u) { u = make_uint4(w[0], w[1], w[2], w[3]); }
+__device__ __forceinline__ void words_vec(const uint32_t *w, uint2 &u) { u = make_uint2(w[0], w[1]); }
+template <typename V> __device__ __forceinline__ V vec_zero();
+template <> __device__ __forceinline__ uint4 vec_zero<uint4>() { return make_uint4(0, 0, 0, 0); }
+template <> __device__ __forceinline__ uint2 vec_zero<uint2>() { return make_uint2(0, 0); }
 
 // How the time axis is cut.  seg_tokens is a multiple of ckpt_interval (itself a multiple of 8);
 // segment s covers tokens [s*seg_tokens, min((s+1)*seg_tokens, T)) and starts from checkpoint
@@ -516,25 +535,28 @@ __global__ __launch_bounds__(BLK) void encode_pair_kernel(EncTensor k, EncTensor
 // patch it into slot T, return the fused dequant r16(q*sc + zp) per pair (gemv.cu:744-798,
 // 1105-1157).  The state is NOT advanced.
 template <int D, int CPL, int BITS = 4>
-__device__ __forceinline__ void append_new_token(uint4 *cb, int T, const h1 *xnew, const Pair *st,
+__device__ __forceinline__ void append_new_token(typename Geo<D, CPL>::Vec *cb, int T, const h1 *xnew, const Pair *st,
                                                  h2 *deq, bool active)
 {
     using G = Geo<D, CPL>;
     const int sg = T / Code<BITS>::TPW, tt = T % Code<BITS>::TPW;
 #pragma unroll
     for (int v = 0; v < G::NV; v++) {
-        uint4 *slot = cb + (size_t)sg * G::VPS + v;
-        uint4 u = *slot;
-        uint32_t w[4] = {u.x, u.y, u.z, u.w};
+        typename G::Vec *slot = cb + (size_t)sg * G::VPS + v;
+        typename G::Vec u = *slot;
+        uint32_t w[G::WPV];
+        vec_words(u, w);
 #pragma unroll
-        for (int pp = 0; pp < 2; pp++) {
-            const int p = 2 * v + pp;
+        for (int pp = 0; pp < G::WPV / 2; pp++) {
+            const int p = (G::WPV / 2) * v + pp;
             const h2 x = *reinterpret_cast<const h2 *>(xnew + 2 * p);
             const h2 q = append_pair<BITS>(w[2 * pp], w[2 * pp + 1], tt, x, st[p]);
             deq[p] = pk_fma(q, st[p].sc, st[p].zp);
         }
-        if (active)
-            *slot = make_uint4(w[0], w[1], w[2], w[3]);
+        if (active) {
+            words_vec(w, u);
+            *slot = u;
+        }
     }
 }
 
@@ -554,12 +576,16 @@ __device__ __forceinline__ void publish_state(const Pair *st, h1 *state_out, con
 }
 
 template <int D, int CPL>
-__device__ __forceinline__ void pair_bytes_of(const uint4 *u, uint32_t (*nb)[2])
+__device__ __forceinline__ void pair_bytes_of(const typename Geo<D, CPL>::Vec *u, uint32_t (*nb)[2])
 {
+    using G = Geo<D, CPL>;
 #pragma unroll
-    for (int v = 0; v < CPL / 4; v++) {
-        pair_bytes(u[v].x, u[v].y, nb[2 * v][0], nb[2 * v][1]);
-        pair_bytes(u[v].z, u[v].w, nb[2 * v + 1][0], nb[2 * v + 1][1]);
+    for (int v = 0; v < G::NV; v++) {
+        uint32_t w[G::WPV];
+        vec_words(u[v], w);
+#pragma unroll
+        for (int pp = 0; pp < G::WPV / 2; pp++)
+            pair_bytes(w[2 * pp], w[2 * pp + 1], nb[(G::WPV / 2) * v + pp][0], nb[(G::WPV / 2) * v + pp][1]);
     }
 }
 
@@ -604,8 +630,9 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
 
     const int t0 = un.seg * sa.seg_tokens;
     const int t1 = last ? T : t0 + sa.seg_tokens;
-    uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV; // this head, this lane
-    const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;                  // this segment
+    using Vec = typename G::Vec;
+    Vec *cbh = reinterpret_cast<Vec *>(cache) + (size_t)bx * n_super_cap * G::VPS + lh * G::NV; // this head, this lane
+    const Vec *cb = cbh + (size_t)(t0 >> 3) * G::VPS;                                           // this segment
     h1 *ob = out + (size_t)bx * sa.row_pitch + t0;
     const int nfull = (t1 - t0) >> 3;
     const int tk = lane & 7, g8 = lane >> 3;
@@ -655,14 +682,14 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    uint4 buf[PF][G::NV];
+    Vec buf[PF][G::NV];
     uint2 lk[G::NP][8];
     uint32_t nb[G::NP][2];
 #pragma unroll
     for (int i = 0; i < PF; i++) {
 #pragma unroll
         for (int v = 0; v < G::NV; v++)
-            buf[i][v] = (i < nfull) ? cb[(size_t)i * G::VPS + v] : make_uint4(0, 0, 0, 0);
+            buf[i][v] = (i < nfull) ? cb[(size_t)i * G::VPS + v] : vec_zero<Vec>();
     }
     if (nfull > 0) {
         pair_bytes_of<D, CPL>(buf[0], nb);
@@ -715,17 +742,17 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
         float part[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int v = 0; v < G::NV; v++) {
-            const uint4 u = cb[(size_t)nfull * G::VPS + v];
-            const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+            uint32_t w[G::WPV];
+            vec_words(cb[(size_t)nfull * G::VPS + v], w);
 #pragma unroll
-            for (int pp = 0; pp < 2; pp++) {
-                Pair &s = st[2 * v + pp];
+            for (int pp = 0; pp < G::WPV / 2; pp++) {
+                Pair &s = st[(G::WPV / 2) * v + pp];
                 for (int tt = 0; tt < ntail; tt++) {
                     const uint32_t na = (w[2 * pp] >> (4 * tt)) & 0xFu;
                     const uint32_t nbb = (w[2 * pp + 1] >> (4 * tt)) & 0xFu;
                     const h2 qc = codes_to_h2((int)na - 8, (int)nbb - 8);
                     const h2 qs = qc * s.sc;
-                    const float d = __builtin_amdgcn_fdot2(qv[2 * v + pp], qs + s.zp, 0.0f, false);
+                    const float d = __builtin_amdgcn_fdot2(qv[(G::WPV / 2) * v + pp], qs + s.zp, 0.0f, false);
 #pragma unroll
                     for (int k = 0; k < 8; k++)
                         part[k] += (k == tt) ? d : 0.0f;
@@ -789,8 +816,9 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
 
     const int t0 = un.seg * sa.seg_tokens;
     const int t1 = last ? T : t0 + sa.seg_tokens;
-    uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV;
-    const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;
+    using Vec = typename G::Vec;
+    Vec *cbh = reinterpret_cast<Vec *>(cache) + (size_t)bx * n_super_cap * G::VPS + lh * G::NV;
+    const Vec *cb = cbh + (size_t)(t0 >> 3) * G::VPS;
     const h1 *wrow = attn + (size_t)bx * sa.row_pitch;
     const h1 *wb = wrow + t0;
     const int nfull = (t1 - t0) >> 3;
@@ -821,7 +849,7 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    uint4 buf[PF][G::NV];
+    Vec buf[PF][G::NV];
     uint4 wbuf[PF];
     uint2 lk[G::NP][8];
     uint32_t nb[G::NP][2];
@@ -829,7 +857,7 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
     for (int i = 0; i < PF; i++) {
 #pragma unroll
         for (int v = 0; v < G::NV; v++)
-            buf[i][v] = (i < nfull) ? cb[(size_t)i * G::VPS + v] : make_uint4(0, 0, 0, 0);
+            buf[i][v] = (i < nfull) ? cb[(size_t)i * G::VPS + v] : vec_zero<Vec>();
         wbuf[i] = (i < nfull) ? load_w(i) : make_uint4(0, 0, 0, 0);
     }
     if (nfull > 0) {
@@ -863,11 +891,11 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
         if (ntail) {
 #pragma unroll
             for (int v = 0; v < G::NV; v++) {
-                const uint4 u = cb[(size_t)nfull * G::VPS + v];
-                const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+                uint32_t w[G::WPV];
+                vec_words(cb[(size_t)nfull * G::VPS + v], w);
 #pragma unroll
-                for (int pp = 0; pp < 2; pp++) {
-                    Pair &s = st[2 * v + pp];
+                for (int pp = 0; pp < G::WPV / 2; pp++) {
+                    Pair &s = st[(G::WPV / 2) * v + pp];
                     for (int tt = 0; tt < ntail; tt++) {
                         const uint32_t na = (w[2 * pp] >> (4 * tt)) & 0xFu;
                         const uint32_t nbb = (w[2 * pp + 1] >> (4 * tt)) & 0xFu;
@@ -875,8 +903,9 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
                         const h2 qs = qc * s.sc;
                         const h2 vd = qs + s.zp;
                         const float wt = (float)wb[nfull * 8 + tt];
-                        acc[4 * v + 2 * pp] = __builtin_fmaf(wt, (float)vd.x, acc[4 * v + 2 * pp]);
-                        acc[4 * v + 2 * pp + 1] = __builtin_fmaf(wt, (float)vd.y, acc[4 * v + 2 * pp + 1]);
+                        const int c = G::WPV * v + 2 * pp;
+                        acc[c] = __builtin_fmaf(wt, (float)vd.x, acc[c]);
+                        acc[c + 1] = __builtin_fmaf(wt, (float)vd.y, acc[c + 1]);
                         update_pair(s, qc, qs);
                     }
                 }
@@ -902,10 +931,10 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
         for (int p = 0; p < G::NP; p++)
             o[p] = (h2){(h1)acc[2 * p], (h1)acc[2 * p + 1]};
     } else {
-        float4 *o = reinterpret_cast<float4 *>(partial + ((size_t)un.seg * BH + bx) * D + c0);
+        float2 *o = reinterpret_cast<float2 *>(partial + ((size_t)un.seg * BH + bx) * D + c0);
 #pragma unroll
-        for (int v = 0; v < G::NV; v++)
-            o[v] = make_float4(acc[4 * v], acc[4 * v + 1], acc[4 * v + 2], acc[4 * v + 3]);
+        for (int p = 0; p < G::NP; p++)
+            o[p] = make_float2(acc[2 * p], acc[2 * p + 1]);
     }
 }
 
@@ -1267,10 +1296,17 @@ static void launch_units(long threads, int big, F256 f256, FBIG fbig)
         [&](dim3 g, dim3 b) { hipLaunchKernelGGL((KERNEL<DD, CC, 256>), g, b, 0, st, __VA_ARGS__); }, \
         [&](dim3 g, dim3 b) { hipLaunchKernelGGL((KERNEL<DD, CC, BIG>), g, b, 0, st, __VA_ARGS__); })
 
+// Head dim 128 has a second shape, two channels per lane (a head per wave): twice the waves, each
+// with half the instruction stream per token.  It pays when every wave has a SIMD to itself and
+// the launch is bound by the length of that stream (small batches, or no checkpoints to cut the
+// context with); with more waves per SIMD the four-channel lanes do less work in total.
 #define ADKV_DISPATCH_D(KERNEL, ...)                  \
     switch (D) {                                      \
     case 128:                                         \
-        ADKV_LAUNCH(KERNEL, 128, 4, 1024, __VA_ARGS__); \
+        if (padded_units<32>(BH, seg.nseg) / 2 <= N_SIMD) \
+            ADKV_LAUNCH(KERNEL, 128, 2, 256, __VA_ARGS__); \
+        else                                          \
+            ADKV_LAUNCH(KERNEL, 128, 4, 1024, __VA_ARGS__); \
         break;                                        \
     case 256:                                         \
         ADKV_LAUNCH(KERNEL, 256, 4, 1024, __VA_ARGS__); \

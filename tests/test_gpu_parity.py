@@ -222,6 +222,8 @@ def _oracle_ckpts(oracle, cache_np, pn, T, S, ncap):
     (1, 2, 100, 128, 16), (2, 3, 64, 128, 16), (1, 2, 63, 128, 8), (1, 1, 257, 128, 64),
     (2, 2, 48, 256, 16), (1, 2, 40, 512, 8), (3, 2, 15, 128, 16), (1, 2, 1024, 128, 256),
     (1, 3, 100, 128, 16), (1, 5, 70, 128, 8),   # odd head counts: a wave's second half is padding
+    (24, 32, 41, 128, 8),    # 3840 units: past the two-channel-per-lane shape, still 4-wave workgroups
+    (9, 32, 20, 128, 16),    # 576 units: two channels per lane with every SIMD of a few CUs busy
 ])
 def test_checkpointed_segments(gpu, oracle, B, H, T, D, S):
     """Encoder checkpoints are the oracle's replayed states; decode over independently replayed
