@@ -12,6 +12,8 @@ by hand-written gfx950 kernels behind ``libadkv_hip.so``.  Differences, all on t
 """
 from __future__ import annotations
 
+import functools
+
 import torch
 
 from .. import _lib
@@ -57,11 +59,17 @@ def _params(tensors, names, nh, dim):
     raise AssertionError("unreachable")
 
 
+@functools.lru_cache(maxsize=4096)
+def _row_pitch(n: int) -> int:
+    """The library's row pitch for rows of ``n`` elements (a pure function of ``n``)."""
+    return int(_lib.lib().adkv_row_pitch(n))
+
+
 def _pitch(n: int) -> int:
     """Row pitch for a ``[rows, n]`` logits / weights matrix.  Long rows are padded to the library's
     recommended pitch (an odd multiple of 128 elements) so that rows of different heads do not all
     start in one memory channel; short rows stay packed."""
-    return int(_lib.lib().adkv_row_pitch(n)) if n >= 1024 else n
+    return _row_pitch(n) if n >= 1024 else n
 
 
 def _rows_view(t: torch.Tensor):
@@ -467,11 +475,14 @@ def decode_fused(
     weights [B,nh,T+1] fp16)``.  ``workspace`` (uint8, 256-byte aligned, sized by
     ``decode_fused_workspace_bytes``) may be passed to avoid the per-call allocation.
     """
-    for t, n in ((q, "q"), (k_new, "k_new"), (v_new, "v_new")):
-        _chk(t.dtype == torch.float16, f"{n} must be float16")
-    for t, n in ((k_cache, "k_cache"), (v_cache, "v_cache")):
-        _chk(t.dtype == torch.uint8, f"{n} must be uint8")
-        _chk(t.is_contiguous(), f"{n} must be contiguous (appended in place)")
+    f16, u8 = torch.float16, torch.uint8
+    if not (q.dtype == f16 and k_new.dtype == f16 and v_new.dtype == f16 and k_cache.dtype == u8
+            and v_cache.dtype == u8 and k_cache.is_contiguous() and v_cache.is_contiguous()):
+        for t, n in ((q, "q"), (k_new, "k_new"), (v_new, "v_new")):
+            _chk(t.dtype == f16, f"{n} must be float16")
+        for t, n in ((k_cache, "k_cache"), (v_cache, "v_cache")):
+            _chk(t.dtype == u8, f"{n} must be uint8")
+            _chk(t.is_contiguous(), f"{n} must be contiguous (appended in place)")
     _chk(k_cache.shape == v_cache.shape, "k_cache and v_cache shapes differ")
     B, nq, nh = q.shape[0], q.shape[1], k_cache.shape[1]
     n_super_cap, DIM = k_cache.shape[2], k_cache.shape[3] * _TILE
@@ -483,7 +494,8 @@ def decode_fused(
     _chk(T >= 0, "T must be non-negative")
     _chk(bits in (2, 4), "bits must be 2 or 4")
     _chk(bits == 4 or DIM == 128, "2-bit codes need DIM == 128")
-    _chk(T // (32 // bits) < n_super_cap, f"k_cache has no free supergroup to append token {T}")
+    if not T // (32 // bits) < n_super_cap:
+        raise RuntimeError(f"k_cache has no free supergroup to append token {T}")
     _chk(DIM in _DIMS, "DIM must be 128, 256 or 512")
     dev = _need_device(q, k_cache, v_cache, k_new, v_new, *kp, *vp)
     n = T + 1
@@ -500,16 +512,16 @@ def decode_fused(
     _chk((k_ckpt is None) == (v_ckpt is None) and ccap == vcap,
          "k_ckpt and v_ckpt must both be given, with the same capacity, or both omitted")
     L = _lib.lib()
-    need = L.adkv_decode_fused_workspace_bytes(B, nq, nh, T, DIM, ccap, civ)
     if workspace is None:
+        need = L.adkv_decode_fused_workspace_bytes(B, nq, nh, T, DIM, ccap, civ)
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
-    _chk(workspace.dtype == torch.uint8 and workspace.is_cuda and workspace.numel() >= need,
-         "workspace too small")
+    # a caller's workspace is sized against the launch by the library itself ("workspace too small")
+    _chk(workspace.dtype == torch.uint8 and workspace.is_cuda, "workspace must be a uint8 device tensor")
     qf = q.contiguous()
     knf = k_new.reshape(B * nh, DIM).contiguous()
     vnf = v_new.reshape(B * nh, DIM).contiguous()
     out = torch.empty((B, nq, DIM), dtype=torch.float16, device=dev)
-    wld = int(L.adkv_row_pitch(n))
+    wld = _row_pitch(n)
     weights = torch.empty((B, nq, wld), dtype=torch.float16, device=dev)
     arr = _lib.C.c_void_p * 5
     with _lib.device_guard(dev):
