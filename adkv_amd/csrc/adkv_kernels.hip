@@ -951,6 +951,43 @@ __global__ __launch_bounds__(256) void ov_finalize_kernel(const float *__restric
     out[i] = (h1)s;
 }
 
+// The same sum for many segments (long contexts at small batch: 128 segments of a 32 768-token
+// context leave the kernel above with 128 dependent additions per thread and few threads).  A
+// workgroup owns 64 consecutive outputs: thread (r, j) adds the segments r, r+16, ... of outputs
+// 4j..4j+3 in ascending order, then thread (0, j) adds the 16 subtotals in ascending r.  The order
+// is fixed, so results are reproducible from run to run.
+__global__ __launch_bounds__(256) void ov_finalize_wide_kernel(const float *__restrict__ partial,
+                                                                h1 *__restrict__ out, long n, int nseg)
+{
+    __shared__ float4 sub[16][16];
+    const int j = threadIdx.x & 15, r = threadIdx.x >> 4;
+    const long i = ((long)blockIdx.x * 16 + j) * 4; // n is a multiple of 4 (whole heads)
+    float4 a = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (i < n) {
+        for (int k = r; k < nseg; k += 16) {
+            const float4 p = *reinterpret_cast<const float4 *>(partial + (size_t)k * n + i);
+            a.x += p.x;
+            a.y += p.y;
+            a.z += p.z;
+            a.w += p.w;
+        }
+    }
+    sub[r][j] = a;
+    __syncthreads();
+    if (r == 0 && i < n) {
+#pragma unroll
+        for (int k = 1; k < 16; k++) {
+            const float4 p = sub[k][j];
+            a.x += p.x;
+            a.y += p.y;
+            a.z += p.z;
+            a.w += p.w;
+        }
+        *reinterpret_cast<h2 *>(out + i) = (h2){(h1)a.x, (h1)a.y};
+        *reinterpret_cast<h2 *>(out + i + 2) = (h2){(h1)a.z, (h1)a.w};
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // softmax(float(logits)*scaling + mask) -> fp16   (llama_adkv.py:266-271)
 // ---------------------------------------------------------------------------------------------
@@ -1692,8 +1729,12 @@ int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void
         return rc;
     if (seg.nseg > 1) {
         const long n = (long)BH * GQ * D;
-        hipLaunchKernelGGL(ov_finalize_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
-                           (const float *)workspace, (h1 *)out, n, seg.nseg);
+        if (seg.nseg > 8)
+            hipLaunchKernelGGL(ov_finalize_wide_kernel, dim3((unsigned)((n + 63) / 64)), dim3(256), 0, st,
+                               (const float *)workspace, (h1 *)out, n, seg.nseg);
+        else
+            hipLaunchKernelGGL(ov_finalize_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                               (const float *)workspace, (h1 *)out, n, seg.nseg);
         rc = check_launch();
     }
     return rc;
