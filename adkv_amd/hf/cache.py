@@ -70,6 +70,7 @@ class KVCacheLayer_ADKV:
         self._B = self._H = self._C = 0
         self._device = None
         self._ckpt_interval = CKPT_INTERVAL
+        self._views: dict = {}    # id(parameter) -> (parameter, its [H, C] view)
 
     # ------------------------------------------------------------------ HF cache protocol
     def get_seq_length(self) -> int:
@@ -144,7 +145,15 @@ class KVCacheLayer_ADKV:
             raise ValueError("cache was created for a different (B, H, C)")
 
     def _view(self, p: torch.Tensor) -> torch.Tensor:
-        return p.view(self._H, self._C)
+        # the module passes the same parameter buffers at every step: keep their [H, C] views
+        hit = self._views.get(id(p))
+        if hit is not None and hit[0] is p:
+            return hit[1]
+        v = p.view(self._H, self._C)
+        if len(self._views) > 64:
+            self._views.clear()
+        self._views[id(p)] = (p, v)
+        return v
 
     # ------------------------------------------------------------------ quantise
     def _append_tokens(self, key_states, value_states,
