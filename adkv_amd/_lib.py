@@ -13,7 +13,7 @@ import torch  # noqa: F401  (loads libamdhip64 first)
 
 _DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_DIR, "libadkv_hip.so")
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 _vp, _i, _f = C.c_void_p, C.c_int, C.c_float
 
@@ -32,7 +32,7 @@ PROTOTYPES = {
     "adkv_softmax_ex": (_i, [_vp] * 3 + [_i, _i, C.c_int64, _i, _f, _vp, C.c_int64, _vp]),
     "adkv_encode_kv_ex": (_i, [_vp] * 7 + [_i] * 5 + [_vp, _vp, _i, _i, _vp]),
     "adkv_append_kv": (_i, [_vp] * 7 + [_i] * 7 + [_vp, _vp, _i, _i, _vp]),
-    "adkv_append_kv_pair": (_i, [_vp] * 6 + [_i] * 7 + [_vp] * 4 + [_i, _i, _vp]),
+    "adkv_append_kv_pair": (_i, [_vp] * 4 + [_i, _vp, _vp] + [_vp] * 2 + [_i] * 7 + [_vp] * 4 + [_i, _i, _vp]),
     "adkv_forward_qk_ex": (_i, [_vp] * 9 + [_i] * 5 + [_vp, _vp, _i, _i, _vp]),
     "adkv_forward_ov_workspace_bytes": (C.c_int64, [_i] * 6),
     "adkv_forward_ov_ex": (_i, [_vp] * 9 + [_i] * 5 + [_vp, _vp, _i, _i, _vp, C.c_int64, _vp]),

@@ -21,6 +21,8 @@
 
 #include <stdlib.h>
 
+#include <initializer_list>
+
 #include <type_traits>
 
 #pragma clang fp contract(off)
@@ -219,9 +221,16 @@ __device__ __forceinline__ void init_pairs(Pair *st, const h1 *zp, const h1 *sc,
 // row pointers advance by addition, checkpoints are found by comparison.
 constexpr int ENC_PF = 3; // supergroup input buffers in rotation
 
-template <int BITS, int CPL, int BLK>
+// Where the new rows are: element strides between batches, heads and tokens (channels are
+// contiguous).  The encoder reads each row once, 256 bytes per head, so a [B, T, H, D] projection
+// output viewed as [B, H, T, D] can be quantised in place without a packed copy.
+struct RowStrides {
+    long b, h, t;
+};
+
+template <int BITS, int CPL, int BLK, bool BF16 = false>
 __device__ __forceinline__ void encode_body(
-    uint32_t *__restrict__ cache, const h1 *__restrict__ kv_new,
+    uint32_t *__restrict__ cache, const h1 *__restrict__ kv_new, RowStrides xs,
     const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
     const h1 *__restrict__ be, const h1 *__restrict__ tg,
     int BH, int H, int T0, int T, int D, int n_super_cap, const h1 *__restrict__ state_in,
@@ -264,7 +273,7 @@ __device__ __forceinline__ void encode_body(
     }
 
     uint32_t *cw = cache + (size_t)bx * n_super_cap * D + c0;
-    const h1 *xb = kv_new + (size_t)bx * (T - T0) * D + c0; // rows of tokens T0.. of this head
+    const h1 *xb = kv_new + (long)(bx / H) * xs.b + (long)h * xs.h + c0; // rows of tokens T0.. of this head
 
     // One token's CPL channels as NP aligned 32-bit words of the input row (an fp16 pair each; a
     // one-channel lane takes the word its channel lies in and shifts at use).  The loads carry no
@@ -276,7 +285,7 @@ __device__ __forceinline__ void encode_body(
     auto load_tok = [&](int t, XW *x) {
 #pragma unroll
         for (int p = 0; p < NP; p++)
-            x[p] = *reinterpret_cast<const XW *>(xbw + (size_t)(t - T0) * D + 2 * p);
+            x[p] = *reinterpret_cast<const XW *>(xbw + (long)(t - T0) * xs.t + 2 * p);
     };
     // reciprocal of the current scale, refreshed right after every update (see quantize_enc_fast)
     float rs[NP][2];
@@ -293,7 +302,13 @@ __device__ __forceinline__ void encode_body(
     auto advance = [&](auto spec, const XW *x, float *qf) {
 #pragma unroll
         for (int p = 0; p < NP; p++) {
-            const XW xw = CPL == 1 ? x[p] >> xsh : x[p];
+            XW xw = CPL == 1 ? x[p] >> xsh : x[p];
+            if (BF16) {
+                // bf16 -> fp32 is exact, fp32 -> fp16 rounds to nearest even: torch's .to(float16)
+                const h1 lo = (h1)__uint_as_float(xw << 16);
+                const h1 hi = CPL == 1 ? lo : (h1)__uint_as_float(xw & 0xFFFF0000u);
+                xw = as_u32((h2){lo, hi});
+            }
             const uint32_t zw = __builtin_bit_cast(uint32_t, st[p].zp);
             float q0, q1;
             if constexpr (decltype(spec)::value) {
@@ -391,17 +406,17 @@ __device__ __forceinline__ void encode_body(
     for (int c = 0; c < CPL; c++)
         w[c] = 0u;
     // loads the next group of 8 rows; past the last group the same rows are loaded again
-    const h1 *xnext = xbw + (size_t)(t - T0) * D;
+    const h1 *xnext = xbw + (long)(t - T0) * xs.t;
     int gnext = 0;
     auto load_next = [&](XW (*xg)[NP]) {
 #pragma unroll
         for (int tt = 0; tt < 8; tt++) {
 #pragma unroll
             for (int p = 0; p < NP; p++)
-                xg[tt][p] = *reinterpret_cast<const XW *>(xnext + (size_t)tt * D + 2 * p);
+                xg[tt][p] = *reinterpret_cast<const XW *>(xnext + (long)tt * xs.t + 2 * p);
         }
         if (gnext < ng - 1) {
-            xnext += (size_t)8 * D;
+            xnext += 8 * xs.t;
             gnext++;
         }
     };
@@ -507,7 +522,8 @@ __global__ __launch_bounds__(BLK) void encode_kernel(
     int BH, int H, int T0, int T, int D, int n_super_cap, const h1 *__restrict__ state_in,
     h1 *__restrict__ state_out, Seg sa)
 {
-    encode_body<BITS, CPL, BLK>(cache, kv_new, zp, sc, al, be, tg, BH, H, T0, T, D, n_super_cap,
+    const RowStrides packed = {(long)H * (T - T0) * D, (long)(T - T0) * D, (long)D};
+    encode_body<BITS, CPL, BLK>(cache, kv_new, packed, zp, sc, al, be, tg, BH, H, T0, T, D, n_super_cap,
                                 state_in, state_out, sa);
 }
 
@@ -518,17 +534,19 @@ struct EncTensor {
     uint32_t *cache;
     const h1 *kv_new, *zp, *sc, *al, *be, *tg, *state_in;
     h1 *state_out, *ckpt;
+    RowStrides xs;
 };
 
-template <int BITS, int CPL, int BLK>
+// BF16: the new rows are bfloat16 (same strides, in elements) and are rounded to fp16 on the fly.
+template <int BITS, int CPL, int BLK, bool BF16>
 __global__ __launch_bounds__(BLK) void encode_pair_kernel(EncTensor k, EncTensor v, int BH, int H,
                                                           int T0, int T, int D, int n_super_cap,
                                                           Seg sa)
 {
     const EncTensor e = blockIdx.y ? v : k;
     sa.ckpt = e.ckpt;
-    encode_body<BITS, CPL, BLK>(e.cache, e.kv_new, e.zp, e.sc, e.al, e.be, e.tg, BH, H, T0, T, D,
-                                n_super_cap, e.state_in, e.state_out, sa);
+    encode_body<BITS, CPL, BLK, BF16>(e.cache, e.kv_new, e.xs, e.zp, e.sc, e.al, e.be, e.tg, BH, H, T0,
+                                      T, D, n_super_cap, e.state_in, e.state_out, sa);
 }
 
 // Shared tail of the two decode kernels: quantise the new token with the state after token T-1,
@@ -1414,7 +1432,7 @@ static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval, int b
 
 extern "C" {
 
-int adkv_abi_version(void) { return 8; }
+int adkv_abi_version(void) { return 9; }
 
 void adkv_set_mha_kernel(int use_matrix_cores) { g_mha_kernel = use_matrix_cores; }
 
@@ -1443,7 +1461,8 @@ static int encode_common(void *cache, const void *kv_new,
                          int B, int H, int T0, int T, int D, int n_super_cap,
                          const void *state_in, void *state_out, void *ckpt_out, int n_ckpt_cap,
                          int ckpt_interval, void *stream, int bits = 4,
-                         const EncTensor *second = nullptr)
+                         const EncTensor *second = nullptr, const RowStrides *first_strides = nullptr,
+                         bool bf16 = false)
 {
     if (!cache || !kv_new || !zp || !sc || !alpha || !beta || !tgt)
         return ADKV_E_NULL;
@@ -1468,6 +1487,13 @@ static int encode_common(void *cache, const void *kv_new,
         return ADKV_E_ALIGN;
     if (second && (ckpt_out == nullptr) != (second->ckpt == nullptr))
         return ADKV_E_NULL; // both tensors keep checkpoints or neither does
+    const RowStrides packed = {(long)H * (T - T0) * D, (long)(T - T0) * D, (long)D};
+    const RowStrides xs1 = first_strides ? *first_strides : packed;
+    for (const RowStrides *xs : {&xs1, second ? &second->xs : &xs1}) {
+        // rows are read as aligned 32-bit words
+        if (xs->b < 0 || xs->h < 0 || xs->t < D || (xs->b | xs->h | xs->t) & 1)
+            return ADKV_E_SHAPE;
+    }
     if ((rc = check_ckpt(ckpt_out, n_ckpt_cap, ckpt_interval, bits)))
         return rc;
     if (T == T0 && !second && (state_out == nullptr || state_out == state_in))
@@ -1508,11 +1534,15 @@ static int encode_common(void *cache, const void *kv_new,
     first.state_in = (const h1 *)state_in;
     first.state_out = (h1 *)state_out;
     first.ckpt = (h1 *)ckpt_out;
+    first.xs = xs1;
 #define ADKV_ENC(BB, C)                                                                          \
     do {                                                                                         \
-        if (second)                                                                              \
-            hipLaunchKernelGGL((encode_pair_kernel<BB, C, 256>), grid, block, 0, st, first,      \
-                               *second, BH, H, T0, T, D, n_super_cap, seg);                      \
+        if (second && bf16)                                                                      \
+            hipLaunchKernelGGL((encode_pair_kernel<BB, C, 256, true>), grid, block, 0, st,       \
+                               first, *second, BH, H, T0, T, D, n_super_cap, seg);               \
+        else if (second)                                                                         \
+            hipLaunchKernelGGL((encode_pair_kernel<BB, C, 256, false>), grid, block, 0, st,      \
+                               first, *second, BH, H, T0, T, D, n_super_cap, seg);               \
         else                                                                                     \
             hipLaunchKernelGGL((encode_kernel<BB, C, 256>), grid, block, 0, st, first.cache,     \
                                first.kv_new, first.zp, first.sc, first.al, first.be, first.tg,   \
@@ -1564,6 +1594,7 @@ int adkv_append_kv(void *cache, const void *kv_new,
 }
 
 int adkv_append_kv_pair(void *k_cache, void *v_cache, const void *k_new, const void *v_new,
+                        int kv_dtype, const int64_t *k_strides, const int64_t *v_strides,
                         const void *const *k_params, const void *const *v_params,
                         int B, int H, int T0, int n_new, int D, int n_super_cap, int bits,
                         void *k_state_io, void *v_state_io, void *k_ckpt, void *v_ckpt,
@@ -1571,10 +1602,14 @@ int adkv_append_kv_pair(void *k_cache, void *v_cache, const void *k_new, const v
 {
     if (!k_params || !v_params || !k_state_io || !v_state_io)
         return ADKV_E_NULL;
+    if (kv_dtype != ADKV_DT_F16 && kv_dtype != ADKV_DT_BF16)
+        return ADKV_E_UNSUPPORTED;
     if (n_new < 0)
         return ADKV_E_SHAPE;
     if (n_new == 0)
         return ADKV_OK;
+    const RowStrides packed = {(long)H * n_new * D, (long)n_new * D, (long)D};
+    const RowStrides ks = k_strides ? RowStrides{(long)k_strides[0], (long)k_strides[1], (long)k_strides[2]} : packed;
     EncTensor v;
     v.cache = (uint32_t *)v_cache;
     v.kv_new = (const h1 *)v_new;
@@ -1586,9 +1621,11 @@ int adkv_append_kv_pair(void *k_cache, void *v_cache, const void *k_new, const v
     v.state_in = (const h1 *)v_state_io;
     v.state_out = (h1 *)v_state_io;
     v.ckpt = (h1 *)v_ckpt;
+    v.xs = v_strides ? RowStrides{(long)v_strides[0], (long)v_strides[1], (long)v_strides[2]} : packed;
     return encode_common(k_cache, k_new, k_params[0], k_params[1], k_params[2], k_params[3],
                          k_params[4], B, H, T0, T0 + n_new, D, n_super_cap, k_state_io, k_state_io,
-                         k_ckpt, n_ckpt_cap, ckpt_interval, stream, bits, &v);
+                         k_ckpt, n_ckpt_cap, ckpt_interval, stream, bits, &v, &ks,
+                         kv_dtype == ADKV_DT_BF16);
 }
 
 int adkv_encode_kv(void *cache, const void *kv_new,

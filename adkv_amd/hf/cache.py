@@ -144,6 +144,12 @@ class KVCacheLayer_ADKV:
         elif (B, H, C) != (self._B, self._H, self._C):
             raise ValueError("cache was created for a different (B, H, C)")
 
+    @staticmethod
+    def _rows(x: torch.Tensor) -> torch.Tensor:
+        # fp16 and bf16 rows go to the encoder as they are (it rounds bf16 to fp16 and follows the
+        # strides of a [B, T, H, C] projection output itself); anything else is converted first
+        return x if x.dtype in (torch.float16, torch.bfloat16) else x.to(torch.float16)
+
     def _view(self, p: torch.Tensor) -> torch.Tensor:
         # the module passes the same parameter buffers at every step: keep their [H, C] views
         hit = self._views.get(id(p))
@@ -164,7 +170,7 @@ class KVCacheLayer_ADKV:
         S = self._ckpt_interval
         append_kv_pair(
             self._key_buf, self._value_buf,
-            key_states.to(torch.float16).contiguous(), value_states.to(torch.float16).contiguous(),
+            self._rows(key_states), self._rows(value_states),
             (v(key_zp_init), v(key_scale_init), v(key_alpha), v(key_beta), v(key_quant_target)),
             (v(value_zp_init), v(value_scale_init), v(value_alpha), v(value_beta),
              v(value_quant_target)),

@@ -354,6 +354,23 @@ def append_kv(
     return kv_cache
 
 
+_DT_F16, _DT_BF16 = 1, 2     # ADKV_DT_F16 / ADKV_DT_BF16 of include/adkv_hip.h
+
+
+def _row_strides(t: torch.Tensor):
+    """``(tensor, strides)`` for new rows ``[B, nh, n, DIM]``: ``strides`` is None for a packed
+    tensor, a ctypes array of the (batch, head, token) element strides when the library can read
+    the rows where they lie (contiguous channels, even strides, 4-byte aligned), else the tensor
+    is packed first."""
+    if t.is_contiguous():
+        return t, None
+    sb, sh, st, sc = t.stride()
+    if sc == 1 and st >= t.shape[3] and not ((sb | sh | st) & 1) and not (t.data_ptr() & 3) \
+            and min(sb, sh) >= 0:
+        return t, (_lib.C.c_int64 * 3)(sb, sh, st)
+    return t.contiguous(), None
+
+
 def append_kv_pair(
     k_cache: torch.Tensor,
     v_cache: torch.Tensor,
@@ -375,8 +392,14 @@ def append_kv_pair(
     ``append_kv`` calls; at small batch the pair takes the time of one tensor because channels are
     the encoder's only parallel axis.  ``k_params`` / ``v_params``: the five ``[nh, DIM]`` fp16
     tensors ``(zp, sc, alpha, beta, quant_target)``.
+
+    ``k_new`` / ``v_new`` ``[B, nh, n, DIM]`` may be float16 or bfloat16 (rounded to fp16 as they
+    are read, like the reference's ``.to(torch.float16)``, llama_adkv.py:141-142) and need not be
+    packed: a ``[B, n, nh, DIM]`` projection output viewed with the head axis first is read in
+    place.
     """
-    _chk(k_new.dtype == torch.float16 and v_new.dtype == torch.float16, "kv_new must be float16")
+    _chk(k_new.dtype == v_new.dtype and k_new.dtype in (torch.float16, torch.bfloat16),
+         "kv_new must be float16 or bfloat16 (K and V alike)")
     _chk(k_cache.dtype == torch.uint8 and v_cache.dtype == torch.uint8, "kv_cache must be uint8")
     _chk(k_cache.is_contiguous() and v_cache.is_contiguous(),
          "kv_cache must be contiguous (written in place)")
@@ -404,11 +427,13 @@ def append_kv_pair(
     _chk(ccap == vcap, "K and V checkpoint tensors must have the same capacity")
     if n == 0:
         return
-    xk, xv = k_new.contiguous(), v_new.contiguous()
+    xk, ks = _row_strides(k_new)
+    xv, vs = _row_strides(v_new)
     arr = _lib.C.c_void_p * 5
     with _lib.device_guard(dev):
         rc = _lib.lib().adkv_append_kv_pair(
             k_cache.data_ptr(), v_cache.data_ptr(), xk.data_ptr(), xv.data_ptr(),
+            _DT_BF16 if k_new.dtype == torch.bfloat16 else _DT_F16, ks, vs,
             arr(*[t.data_ptr() for t in kp]), arr(*[t.data_ptr() for t in vp]),
             B, nh, T0, n, DIM, n_super_cap, bits, k_state.data_ptr(), v_state.data_ptr(),
             kc, vc, ccap, civ, _lib.current_stream_ptr(dev))

@@ -143,14 +143,24 @@ int adkv_append_kv(void *cache, const void *kv_new,
 
 /*
  * adkv_append_kv for the K and the V rows of the same tokens in ONE launch: the two calls that
- * KVCacheLayer_ADKV._append_tokens makes back to back (src/adkv/hf/llama_adkv.py:144-153).  Both
- * tensors share every shape argument; k_params / v_params are host arrays of five device
+ * KVCacheLayer_ADKV._append_tokens makes back to back (src/adkv/hf/llama_adkv.py:144-153), with
+ * the conversion and packing that precede them there (`.to(torch.float16).contiguous()`,
+ * llama_adkv.py:141-142) folded in:
+ *   kv_dtype   ADKV_DT_F16, or ADKV_DT_BF16: bfloat16 rows are rounded to fp16 (nearest even, as
+ *              torch's .to(float16)) as they are read;
+ *   k_strides / v_strides   NULL for packed [B,H,n_new,D] rows, else host arrays of three element
+ *              strides {batch, head, token} (channels contiguous, all three even, token stride
+ *              >= D, base pointers 4-byte aligned): a projection output laid out [B,T,H,D] is
+ *              quantised where it lies.
+ * Both tensors share every shape argument; k_params / v_params are host arrays of five device
  * pointers {zp, sc, alpha, beta, tgt}; the checkpoint tensors are both given or both NULL.
- * Results are byte-identical to two adkv_append_kv calls.  Channels are the only parallel axis
- * of the encoder, so a long prompt at a small batch (B*H*D below ~130 000 channels) leaves half
- * of the device idle per tensor; paired, both tensors finish in the time of one.
+ * Results are byte-identical to two adkv_append_kv calls on packed fp16 copies.  Channels are the
+ * only parallel axis of the encoder, so a long prompt at a small batch (B*H*D below ~130 000
+ * channels) leaves half of the device idle per tensor; paired, both tensors finish in the time of
+ * one.
  */
 int adkv_append_kv_pair(void *k_cache, void *v_cache, const void *k_new, const void *v_new,
+                        int kv_dtype, const int64_t *k_strides, const int64_t *v_strides,
                         const void *const *k_params, const void *const *v_params,
                         int B, int H, int T0, int n_new, int D, int n_super_cap, int bits,
                         void *k_state_io, void *v_state_io, void *k_ckpt, void *v_ckpt,

@@ -584,6 +584,46 @@ def test_grouped_query_kernels(gpu, oracle, B, Hkv, G, T, S):
     _gqa_case(gpu, oracle, B, Hkv, G, T, S, seed=T % 7)
 
 
+@pytest.mark.parametrize("dtype,strided,bits,B,H,D,cuts", [
+    (torch.float16, True, 4, 2, 3, 128, (0, 5, 8, 19, 64, 100)),
+    (torch.bfloat16, False, 4, 2, 3, 128, (0, 7, 40)),
+    (torch.bfloat16, True, 4, 1, 2, 256, (0, 16, 17, 33)),
+    (torch.bfloat16, True, 2, 2, 2, 128, (0, 33, 34, 64, 150)),
+    (torch.bfloat16, True, 4, 48, 32, 128, (0, 21)),        # 196 608 channels per tensor: two per lane
+])
+def test_paired_append_reads_projection_outputs_in_place(gpu, oracle, dtype, strided, bits, B, H, D, cuts):
+    """The K/V rows as an attention module has them: bfloat16 or float16, laid out [B, T, H, D] and
+    viewed head-first.  The paired append rounds bf16 to fp16 (nearest even) and follows the
+    strides itself; the result equals the oracle on a packed fp16 copy."""
+    T = cuts[-1]
+    tps = 32 // bits
+    caches = [synth.alloc_cache(B, H, T + tps, D, gpu, bits=bits) for _ in range(2)]
+    states = [torch.zeros(B, H, D, 2, dtype=torch.float16, device=gpu) for _ in range(2)]
+    rows, pars, want = [], [], []
+    for i in range(2):
+        x, p = _inputs(B, H, T, D, seed=21 + i, bits=bits)
+        x = (x.float() * 1.01).to(dtype)                      # values that are not fp16 numbers in bf16
+        if strided:
+            xg = x.permute(0, 2, 1, 3).contiguous().to(gpu).permute(0, 2, 1, 3)   # memory [B, T, H, D]
+            assert not xg.is_contiguous()
+        else:
+            xg = x.to(gpu)
+        rows.append(xg)
+        pars.append([t.to(gpu) for t in p.astuple()])
+        pn = [_np16(t) for t in p.astuple()]
+        with oracle.code_bits(bits):
+            c = oracle.alloc_cache(B, H, T + tps, D)
+            st = oracle.encode_kv_f16(c, _np16(x.to(torch.float16)), *pn)
+        want.append((c, st))
+    for a, b in zip(cuts[:-1], cuts[1:]):
+        gemv.append_kv_pair(caches[0], caches[1], rows[0][:, :, a:b], rows[1][:, :, a:b],
+                            pars[0], pars[1], a, states[0], states[1], bits=bits)
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert np.array_equal(caches[i].cpu().numpy(), want[i][0]), i
+        assert np.array_equal(_np16(states[i]).view(np.uint16), want[i][1]), i
+
+
 @pytest.mark.parametrize("G,bits", [(4, 4), (8, 4), (2, 2), (8, 2)])
 def test_grouped_query_kernels_in_16_wave_workgroups(gpu, oracle, G, bits):
     """A launch big enough for the 16-wave workgroups (128 KV heads x 64 segments = 8192 units):
