@@ -735,6 +735,47 @@ def test_decode_kernels_2bit(gpu, oracle, B, Hkv, G, T, S):
     _gqa_case(gpu, oracle, B, Hkv, G, T, S, seed=T % 7, bits=2)
 
 
+def test_non_finite_inputs_and_runaway_state(gpu, oracle):
+    """Parameters that make the scale run away to infinity or zero within a few tokens, large
+    inputs and a few infinite / NaN elements: codes, the carried state (NaN in the same places)
+    and the state replayed by the decode kernel still equal the oracle's."""
+    B, H, D, T = 1, 2, 128, 200
+    p = synth.make_params(H, D, seed=1)
+    g = torch.Generator().manual_seed(0)
+    p.beta = (0.9 * torch.rand(H, D, generator=g)).half()
+    p.alpha = (2.0 * torch.rand(H, D, generator=g)).half()
+    x = (50.0 * torch.randn(B, H, T + 1, D, generator=g)).half()
+    x[0, 0, 5, 3] = float("inf")
+    x[0, 1, 9, 7] = float("nan")
+    x[0, 1, 30, 8] = -float("inf")
+    pn = [_np16(t) for t in p.astuple()]
+    pg = [t.to(gpu) for t in p.astuple()]
+    want = oracle.alloc_cache(B, H, T + 8, D)
+    st_want = oracle.encode_kv_f16(want, _np16(x)[:, :, :T], *pn)
+    wf = st_want.view(np.float16).astype(np.float32)
+    assert np.isinf(wf).any() and np.isnan(wf).any() and (wf[..., 1] == 0).any()   # it did run away
+
+    def same(a, b):
+        nan = np.isnan(a.view(np.float16).astype(np.float32)) & np.isnan(b.view(np.float16).astype(np.float32))
+        return np.array_equal(np.where(nan, 0, a), np.where(nan, 0, b))
+
+    cache = synth.alloc_cache(B, H, T + 8, D, gpu)
+    st = torch.zeros(B, H, D, 2, dtype=torch.float16, device=gpu)
+    gemv.append_kv(cache, x[:, :, :T].to(gpu), *pg, 0, st)
+    torch.cuda.synchronize()
+    assert np.array_equal(cache.cpu().numpy(), want)
+    assert same(_np16(st).view(np.uint16), st_want)
+
+    q = torch.randn(B, H, 1, D, generator=g).half()
+    kc, st2 = cache.clone(), torch.zeros_like(st)
+    gemv.forward_qk(q.to(gpu), kc, x[:, :, T:].to(gpu), *pg, T, SMIN, SMAX, state_out=st2)
+    torch.cuda.synchronize()
+    assert same(_np16(st2).view(np.uint16), st_want)
+    kw = want.copy()
+    oracle.forward_qk_f16(_np16(q), kw, _np16(x)[:, :, T:T + 1], *pn, T)
+    assert np.array_equal(kc.cpu().numpy(), kw)
+
+
 @pytest.mark.parametrize("bits", [4, 2])
 def test_encode_rounding_boundaries(gpu, oracle, bits):
     """Inputs on and next to the quantiser's rounding boundaries: (x - zp) / sc = k + 1/2 exactly
