@@ -78,13 +78,26 @@ class LlamaAttention_ADKV(LlamaAttention):
                 attention_mask=attention_mask, scaling=self.scaling)
             return self.o_proj(ctx.reshape(*lead, -1).contiguous()), weights
 
+        if layer_cache is not None and layer_cache.get_seq_length() > 0:
+            # Several new tokens on top of a cache that already holds codes (a follow-up turn, a
+            # prompt fed in pieces).  The earlier tokens exist only as codes, so the new ones are
+            # taken one decode step at a time: token i attends over the cache and the new tokens
+            # before it, exactly as if they had arrived singly.  (The reference refuses this call,
+            # llama_adkv.py:195-197; the first prompt still goes through the dense path below.)
+            past = layer_cache.get_seq_length()
+            key_p, value_p = self._adkv_params("key"), self._adkv_params("value")
+            steps = []
+            for i in range(q.shape[2]):
+                mask = None
+                if attention_mask is not None:
+                    mask = attention_mask[:, :, i:i + 1, :past + i + 1]
+                o, _ = layer_cache.decode(q[:, :, i:i + 1], k[:, :, i:i + 1], v[:, :, i:i + 1],
+                                          *key_p, *value_p, attention_mask=mask, scaling=self.scaling)
+                steps.append(o)
+            ctx = torch.stack(steps, dim=1)                      # [B, Tq, Hq, C]
+            return self.o_proj(ctx.reshape(*lead, -1)), None
+
         if layer_cache is not None:
-            if layer_cache.get_seq_length() > 0:
-                # the earlier tokens exist only as codes: a multi-token step would have to attend
-                # over dequantised history, which this deployment path does not keep (the cache
-                # object itself accepts prompt chunks; see KVCacheLayer_ADKV.prefill)
-                raise NotImplementedError(
-                    "ADKV attention takes the prompt in one call; multi-token steps after it are not supported")
             layer_cache.prefill(k, v, *self._adkv_params("key"), *self._adkv_params("value"))
 
         attend = eager_attention_forward

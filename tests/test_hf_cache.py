@@ -156,6 +156,47 @@ def test_tiny_llama_generate(gpu):
 
 
 @pytest.mark.gpu
+def test_tiny_llama_follow_up_chunk_equals_single_token_steps(gpu):
+    """A second multi-token call on top of a cache that already holds codes (a follow-up turn):
+    the module takes it as successive decode steps, so the cache ends up byte-identical to
+    feeding the same tokens one call at a time and the logits agree (the projections run as one
+    GEMM instead of five, hence a small tolerance)."""
+    pytest.importorskip("transformers")
+    from transformers import LlamaConfig
+    from adkv_amd.hf.llama_adkv import ADKVConfig, LlamaForCausalLM_ADKV
+
+    cfg = LlamaConfig(vocab_size=128, hidden_size=256, intermediate_size=512, num_hidden_layers=2,
+                      num_attention_heads=2, num_key_value_heads=2, max_position_embeddings=256,
+                      attn_implementation="eager")
+    torch.manual_seed(0)
+    model = LlamaForCausalLM_ADKV(cfg).to(gpu).half().eval()
+    n = 2 * 128
+    mk = lambda: ADKVConfig(zp_init=torch.zeros(n), scale_init=torch.full((n,), 0.05),
+                            alpha=torch.full((n,), 0.95), beta=torch.full((n,), 0.05),
+                            quant_target=torch.full((n,), 3.5))
+    model.load_adkv_config([(mk(), mk()) for _ in range(2)])
+    g = torch.Generator().manual_seed(5)
+    prompt = torch.randint(0, 128, (2, 12), generator=g).to(gpu)
+    more = torch.randint(0, 128, (2, 5), generator=g).to(gpu)
+    with torch.no_grad():
+        a = model(prompt, use_cache=True)
+        chunk = model(more, past_key_values=a.past_key_values, use_cache=True)
+        b = model(prompt, use_cache=True)
+        singles = []
+        cache = b.past_key_values
+        for i in range(5):
+            r = model(more[:, i:i + 1], past_key_values=cache, use_cache=True)
+            cache = r.past_key_values
+            singles.append(r.logits)
+    assert chunk.past_key_values.get_seq_length() == 17 and cache.get_seq_length() == 17
+    for la, lb in zip(chunk.past_key_values, cache):
+        assert torch.equal(la._key_buf, lb._key_buf) and torch.equal(la._value_buf, lb._value_buf)
+    got, want = chunk.logits.float(), torch.cat(singles, dim=1).float()
+    assert got.shape == want.shape == (2, 5, 128)
+    assert torch.allclose(got, want, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("interval", [0, 16])
 def test_cache_save_and_restore_continues_identically(gpu, tmp_path, monkeypatch, interval):
     """A cache saved after prefill + decode steps and restored from the file continues exactly like
