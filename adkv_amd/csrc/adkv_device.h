@@ -52,6 +52,36 @@ __device__ __forceinline__ void rotate_over(int n, F &&body)
     });
 }
 
+// Activations (q, the new K / V token, the attention output) may be stored as bfloat16 instead of
+// fp16: they are rounded to fp16 as they are read (bf16 -> fp32 is exact, fp32 -> fp16 rounds to
+// nearest even: torch's .to(float16)) and the fp16 result is rounded to bf16 as it is written
+// (torch's .to(bfloat16)), so values are those of the reference's conversions around its kernels
+// (src/adkv/hf/llama_adkv.py:248-250, 274).  `bf16` is uniform over the launch.
+__device__ __forceinline__ h2 load_act2(const h1 *p, int bf16)
+{
+    const uint32_t w = *reinterpret_cast<const uint32_t *>(p);
+    if (bf16)
+        return (h2){(h1)__uint_as_float(w << 16), (h1)__uint_as_float(w & 0xFFFF0000u)};
+    return as_h2(w);
+}
+
+__device__ __forceinline__ uint32_t bf16_bits(h1 v)
+{
+    const uint32_t u = __float_as_uint((float)v);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u)
+        return (u >> 16) | 0x40u; // NaN stays NaN
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+
+__device__ __forceinline__ void store_act2(h1 *p, float a, float b, int bf16)
+{
+    const h2 v = {(h1)a, (h1)b};
+    if (bf16)
+        *reinterpret_cast<uint32_t *>(p) = bf16_bits(v.x) | (bf16_bits(v.y) << 16);
+    else
+        *reinterpret_cast<h2 *>(p) = v;
+}
+
 // One channel pair's filter state and fixed parameters (two channels packed per register).
 struct Pair {
     h2 zp, sc, al, be, omt;

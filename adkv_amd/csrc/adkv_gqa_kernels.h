@@ -168,10 +168,13 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
 #pragma unroll
     for (int n = 0; n < NB; n++) {
         const int g = 4 * n + r;
-        const uint2 *src = reinterpret_cast<const uint2 *>(q + ((size_t)bx * GQ + (g < GQ ? g : 0)) * D) + qd * 8;
+        const h1 *src = q + ((size_t)bx * GQ + (g < GQ ? g : 0)) * D + qd * 32;
 #pragma unroll
-        for (int m = 0; m < 8; m++)
-            qb[n][m] = (g < GQ) ? src[m] : make_uint2(0u, 0u);
+        for (int m = 0; m < 8; m++) {
+            const uint2 four = make_uint2(as_u32(load_act2(src + 4 * m, sa.act_bf16)),
+                                          as_u32(load_act2(src + 4 * m + 2, sa.act_bf16)));
+            qb[n][m] = (g < GQ) ? four : make_uint2(0u, 0u);
+        }
     }
     const uint2 *arow = tile + (tg4 * 4 + r) * TILE_ROW64 + (lane >> 5) * 32 + qd * 8;
 
@@ -304,7 +307,7 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
     if (active)
         publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
     h2 deq[G::NP];
-    append_new_token<D, CPL, BITS>(cbh, T, k_new + (size_t)bx * D + c0, st, deq, active);
+    append_new_token<D, CPL, BITS>(cbh, T, k_new + (size_t)bx * D + c0, st, deq, active, sa.act_bf16);
     tile[row * TILE_ROW64 + lane] = make_uint2(as_u32(deq[0]), as_u32(deq[1]));
     emit_read(areg);
     emit_finish(areg, unit, row + 1);
@@ -486,7 +489,7 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
         if (active)
             publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
         h2 deq[G::NP];
-        append_new_token<D, CPL, BITS>(cbh, T, v_new + (size_t)bx * D + c0, st, deq, active);
+        append_new_token<D, CPL, BITS>(cbh, T, v_new + (size_t)bx * D + c0, st, deq, active, sa.act_bf16);
         add_token(deq, T);
     }
     if (!active)
@@ -497,9 +500,8 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
         const float o0 = acc[g >> 2][0][g & 3], o1 = acc[g >> 2][1][g & 3];
         const float o2 = acc[g >> 2][2][g & 3], o3 = acc[g >> 2][3][g & 3];
         if (sa.nseg == 1) {
-            h2 *o = reinterpret_cast<h2 *>(out + row * D + c0);
-            o[0] = (h2){(h1)o0, (h1)o1};
-            o[1] = (h2){(h1)o2, (h1)o3};
+            store_act2(out + row * D + c0, o0, o1, sa.act_bf16);
+            store_act2(out + row * D + c0 + 2, o2, o3, sa.act_bf16);
         } else {
             *reinterpret_cast<float4 *>(partial + ((size_t)un.seg * BH * GQ + row) * D + c0) =
                 make_float4(o0, o1, o2, o3);

@@ -75,6 +75,7 @@ struct Seg {
     int seg_tokens;     // >= T when there is one segment
     int nseg;
     long row_pitch;     // elements between rows of the logits / attention-weight matrix (>= T + 1)
+    int act_bf16;       // q, the new token and the output are bfloat16 (see load_act2 / store_act2)
 };
 
 __device__ __forceinline__ float wave_xor_add(float v, int mask)
@@ -554,7 +555,7 @@ __global__ __launch_bounds__(BLK) void encode_pair_kernel(EncTensor k, EncTensor
 // 1105-1157).  The state is NOT advanced.
 template <int D, int CPL, int BITS = 4>
 __device__ __forceinline__ void append_new_token(typename Geo<D, CPL>::Vec *cb, int T, const h1 *xnew, const Pair *st,
-                                                 h2 *deq, bool active)
+                                                 h2 *deq, bool active, int act_bf16 = 0)
 {
     using G = Geo<D, CPL>;
     const int sg = T / Code<BITS>::TPW, tt = T % Code<BITS>::TPW;
@@ -567,7 +568,7 @@ __device__ __forceinline__ void append_new_token(typename Geo<D, CPL>::Vec *cb, 
 #pragma unroll
         for (int pp = 0; pp < G::WPV / 2; pp++) {
             const int p = (G::WPV / 2) * v + pp;
-            const h2 x = *reinterpret_cast<const h2 *>(xnew + 2 * p);
+            const h2 x = load_act2(xnew + 2 * p, act_bf16);
             const h2 q = append_pair<BITS>(w[2 * pp], w[2 * pp + 1], tt, x, st[p]);
             deq[p] = pk_fma(q, st[p].sc, st[p].zp);
         }
@@ -644,7 +645,7 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
     init_pairs<D, CPL>(st, zp, sc, al, be, tg, h, bx, c0, un.seg, sa);
 #pragma unroll
     for (int p = 0; p < G::NP; p++)
-        qv[p] = *reinterpret_cast<const h2 *>(q + (size_t)bx * D + c0 + 2 * p);
+        qv[p] = load_act2(q + (size_t)bx * D + c0 + 2 * p, sa.act_bf16);
 
     const int t0 = un.seg * sa.seg_tokens;
     const int t1 = last ? T : t0 + sa.seg_tokens;
@@ -788,7 +789,7 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
         publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
 
     h2 deq[G::NP];
-    append_new_token<D, CPL>(cbh, T, k_new + (size_t)bx * D + c0, st, deq, active);
+    append_new_token<D, CPL>(cbh, T, k_new + (size_t)bx * D + c0, st, deq, active, sa.act_bf16);
     float self = 0.0f;
 #pragma unroll
     for (int p = 0; p < G::NP; p++)
@@ -933,7 +934,7 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
             publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
 
         h2 deq[G::NP];
-        append_new_token<D, CPL>(cbh, T, v_new + (size_t)bx * D + c0, st, deq, active);
+        append_new_token<D, CPL>(cbh, T, v_new + (size_t)bx * D + c0, st, deq, active, sa.act_bf16);
         const float wT = (float)wrow[T];
 #pragma unroll
         for (int p = 0; p < G::NP; p++) {
@@ -944,10 +945,10 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
     if (!active)
         return;
     if (sa.nseg == 1) {
-        h2 *o = reinterpret_cast<h2 *>(out + (size_t)bx * D + c0);
+        h1 *o = out + (size_t)bx * D + c0;
 #pragma unroll
         for (int p = 0; p < G::NP; p++)
-            o[p] = (h2){(h1)acc[2 * p], (h1)acc[2 * p + 1]};
+            store_act2(o + 2 * p, acc[2 * p], acc[2 * p + 1], sa.act_bf16);
     } else {
         float2 *o = reinterpret_cast<float2 *>(partial + ((size_t)un.seg * BH + bx) * D + c0);
 #pragma unroll
@@ -958,15 +959,19 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
 
 // out[i] = fp16(sum over segments, in segment order, of partial[s][i])
 __global__ __launch_bounds__(256) void ov_finalize_kernel(const float *__restrict__ partial,
-                                                           h1 *__restrict__ out, long n, int nseg)
+                                                           h1 *__restrict__ out, long n, int nseg,
+                                                           int act_bf16)
 {
-    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 2; // n is even (whole heads)
     if (i >= n)
         return;
-    float s = 0.0f;
-    for (int k = 0; k < nseg; k++)
-        s += partial[(size_t)k * n + i];
-    out[i] = (h1)s;
+    float2 s = make_float2(0.0f, 0.0f);
+    for (int k = 0; k < nseg; k++) {
+        const float2 p = *reinterpret_cast<const float2 *>(partial + (size_t)k * n + i);
+        s.x += p.x;
+        s.y += p.y;
+    }
+    store_act2(out + i, s.x, s.y, act_bf16);
 }
 
 // The same sum for many segments (long contexts at small batch: 128 segments of a 32 768-token
@@ -975,7 +980,8 @@ __global__ __launch_bounds__(256) void ov_finalize_kernel(const float *__restric
 // 4j..4j+3 in ascending order, then thread (0, j) adds the 16 subtotals in ascending r.  The order
 // is fixed, so results are reproducible from run to run.
 __global__ __launch_bounds__(256) void ov_finalize_wide_kernel(const float *__restrict__ partial,
-                                                                h1 *__restrict__ out, long n, int nseg)
+                                                                h1 *__restrict__ out, long n, int nseg,
+                                                                int act_bf16)
 {
     __shared__ float4 sub[16][16];
     const int j = threadIdx.x & 15, r = threadIdx.x >> 4;
@@ -1001,8 +1007,8 @@ __global__ __launch_bounds__(256) void ov_finalize_wide_kernel(const float *__re
             a.z += p.z;
             a.w += p.w;
         }
-        *reinterpret_cast<h2 *>(out + i) = (h2){(h1)a.x, (h1)a.y};
-        *reinterpret_cast<h2 *>(out + i + 2) = (h2){(h1)a.z, (h1)a.w};
+        store_act2(out + i, a.x, a.y, act_bf16);
+        store_act2(out + i + 2, a.z, a.w, act_bf16);
     }
 }
 
@@ -1289,6 +1295,7 @@ static Seg plan_segments(void *ckpt, int n_ckpt_cap, int ckpt_interval, int BH, 
     s.seg_tokens = T > 0 ? T : 1;
     s.nseg = 1;
     s.row_pitch = T + 1;
+    s.act_bf16 = 0;
     if (!ckpt || ckpt_interval <= 0 || T <= ckpt_interval)
         return s;
     const int avail = (T + ckpt_interval - 1) / ckpt_interval;               // finest split
@@ -1432,7 +1439,7 @@ static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval, int b
 
 extern "C" {
 
-int adkv_abi_version(void) { return 9; }
+int adkv_abi_version(void) { return 10; }
 
 void adkv_set_mha_kernel(int use_matrix_cores) { g_mha_kernel = use_matrix_cores; }
 
@@ -1507,6 +1514,7 @@ static int encode_common(void *cache, const void *kv_new,
     seg.seg_tokens = T > 0 ? T : 1;
     seg.nseg = 1;
     seg.row_pitch = T + 1;
+    seg.act_bf16 = 0;
     // Lane width, measured on an MI355X (4096 tokens, ms for 65 536 / 131 072 / 196 608 / 262 144 /
     // 524 288 channels): one channel per lane 0.29 / 0.44 / 0.60 / 0.74 / 1.38, two 0.43 / 0.44 /
     // 0.55 / 0.60 / 1.17, four 0.78 / 0.78 / 0.78 / 0.79 / 1.18.  Up to two waves per SIMD the
@@ -1638,12 +1646,15 @@ int adkv_encode_kv(void *cache, const void *kv_new,
                              state_out, nullptr, 0, 0, stream);
 }
 
-int adkv_forward_qk_gqa(const void *q, void *k_cache, const void *k_new, void *logits,
-                        const void *zp, const void *sc, const void *alpha, const void *beta,
-                        const void *tgt,
-                        int B, int Hq, int H, int T, int D, int n_super_cap, int bits, int64_t ld,
-                        void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
-                        void *stream)
+} // extern "C"
+
+// act_bf16: q, k_new / v_new and the output are bfloat16 (only adkv_decode_fused asks for it)
+static int forward_qk_impl(const void *q, void *k_cache, const void *k_new, void *logits,
+                           const void *zp, const void *sc, const void *alpha, const void *beta,
+                           const void *tgt,
+                           int B, int Hq, int H, int T, int D, int n_super_cap, int bits, int64_t ld,
+                           void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
+                           void *stream, int act_bf16)
 {
     if (ld != 0 && ld < (int64_t)T + 1)
         return ADKV_E_SHAPE;
@@ -1668,6 +1679,7 @@ int adkv_forward_qk_gqa(const void *q, void *k_cache, const void *k_new, void *l
     const int BH = B * H;
     hipStream_t st = (hipStream_t)stream;
     Seg seg = plan_segments(ckpt, n_ckpt_cap, ckpt_interval, BH, T, D);
+    seg.act_bf16 = act_bf16;
     if (ld)
         seg.row_pitch = ld;
     if (D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha())) {
@@ -1681,6 +1693,19 @@ int adkv_forward_qk_gqa(const void *q, void *k_cache, const void *k_new, void *l
                     (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha, (const h1 *)beta,
                     (const h1 *)tgt, BH, H, T, n_super_cap, (h1 *)state_out, seg);
     return check_launch();
+}
+
+extern "C" {
+
+int adkv_forward_qk_gqa(const void *q, void *k_cache, const void *k_new, void *logits,
+                        const void *zp, const void *sc, const void *alpha, const void *beta,
+                        const void *tgt,
+                        int B, int Hq, int H, int T, int D, int n_super_cap, int bits, int64_t ld,
+                        void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
+                        void *stream)
+{
+    return forward_qk_impl(q, k_cache, k_new, logits, zp, sc, alpha, beta, tgt, B, Hq, H, T, D,
+                           n_super_cap, bits, ld, state_out, ckpt, n_ckpt_cap, ckpt_interval, stream, 0);
 }
 
 int adkv_forward_qk_ex(const void *q, void *k_cache, const void *k_new, void *logits,
@@ -1713,12 +1738,14 @@ int64_t adkv_forward_ov_workspace_bytes(int B, int H, int T, int D, int n_ckpt_c
     return seg.nseg > 1 ? (int64_t)seg.nseg * B * H * D * 4 : 0;
 }
 
-int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void *out,
-                        const void *zp, const void *sc, const void *alpha, const void *beta,
-                        const void *tgt,
-                        int B, int Hq, int H, int T, int D, int n_super_cap, int bits, int64_t ld,
-                        void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
-                        void *workspace, int64_t workspace_bytes, void *stream)
+} // extern "C"
+
+static int forward_ov_impl(const void *attn, void *v_cache, const void *v_new, void *out,
+                           const void *zp, const void *sc, const void *alpha, const void *beta,
+                           const void *tgt,
+                           int B, int Hq, int H, int T, int D, int n_super_cap, int bits, int64_t ld,
+                           void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
+                           void *workspace, int64_t workspace_bytes, void *stream, int act_bf16)
 {
     if (ld != 0 && ld < (int64_t)T + 1)
         return ADKV_E_SHAPE;
@@ -1743,6 +1770,7 @@ int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void
     const int BH = B * H;
     hipStream_t st = (hipStream_t)stream;
     Seg seg = plan_segments(ckpt, n_ckpt_cap, ckpt_interval, BH, T, D);
+    seg.act_bf16 = act_bf16;
     if (ld)
         seg.row_pitch = ld;
     if (seg.nseg > 1) {
@@ -1768,13 +1796,27 @@ int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void
         const long n = (long)BH * GQ * D;
         if (seg.nseg > 8)
             hipLaunchKernelGGL(ov_finalize_wide_kernel, dim3((unsigned)((n + 63) / 64)), dim3(256), 0, st,
-                               (const float *)workspace, (h1 *)out, n, seg.nseg);
+                               (const float *)workspace, (h1 *)out, n, seg.nseg, seg.act_bf16);
         else
-            hipLaunchKernelGGL(ov_finalize_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
-                               (const float *)workspace, (h1 *)out, n, seg.nseg);
+            hipLaunchKernelGGL(ov_finalize_kernel, dim3((unsigned)((n + 511) / 512)), dim3(256), 0, st,
+                               (const float *)workspace, (h1 *)out, n, seg.nseg, seg.act_bf16);
         rc = check_launch();
     }
     return rc;
+}
+
+extern "C" {
+
+int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void *out,
+                        const void *zp, const void *sc, const void *alpha, const void *beta,
+                        const void *tgt,
+                        int B, int Hq, int H, int T, int D, int n_super_cap, int bits, int64_t ld,
+                        void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
+                        void *workspace, int64_t workspace_bytes, void *stream)
+{
+    return forward_ov_impl(attn, v_cache, v_new, out, zp, sc, alpha, beta, tgt, B, Hq, H, T, D,
+                           n_super_cap, bits, ld, state_out, ckpt, n_ckpt_cap, ckpt_interval, workspace,
+                           workspace_bytes, stream, 0);
 }
 
 int adkv_forward_ov_ex(const void *attn, void *v_cache, const void *v_new, void *out,
@@ -1897,12 +1939,15 @@ int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k
                       const void *const *k_params, const void *const *v_params,
                       const void *mask, int rows_per_mask_row, float scaling,
                       void *out, void *weights_out, int64_t weights_ld,
-                      int B, int Hq, int H, int T, int D, int n_super_cap, int bits,
+                      int B, int Hq, int H, int T, int D, int n_super_cap, int bits, int act_dtype,
                       void *k_ckpt, void *v_ckpt, int n_ckpt_cap, int ckpt_interval,
                       void *workspace, int64_t workspace_bytes, void *stream)
 {
     if (!k_params || !v_params || !workspace)
         return workspace ? ADKV_E_NULL : ADKV_E_WORKSPACE;
+    if (act_dtype != ADKV_DT_F16 && act_dtype != ADKV_DT_BF16)
+        return ADKV_E_UNSUPPORTED;
+    const int act_bf16 = act_dtype == ADKV_DT_BF16;
     if (B <= 0 || H <= 0 || Hq <= 0 || Hq % H || T < 0)
         return ADKV_E_SHAPE;
     if (workspace_bytes < adkv_decode_fused_workspace_bytes(B, Hq, H, T, D, n_ckpt_cap, ckpt_interval))
@@ -1919,9 +1964,9 @@ int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k
     char *ws = (char *)workspace;
     void *logits = ws;
     void *weights = weights_out ? weights_out : (void *)(ws + mat);
-    int rc = adkv_forward_qk_gqa(q, k_cache, k_new, logits, k_params[0], k_params[1], k_params[2],
-                                 k_params[3], k_params[4], B, Hq, H, T, D, n_super_cap, bits, ld,
-                                 nullptr, k_ckpt, n_ckpt_cap, ckpt_interval, stream);
+    int rc = forward_qk_impl(q, k_cache, k_new, logits, k_params[0], k_params[1], k_params[2],
+                             k_params[3], k_params[4], B, Hq, H, T, D, n_super_cap, bits, ld,
+                             nullptr, k_ckpt, n_ckpt_cap, ckpt_interval, stream, act_bf16);
     if (rc)
         return rc;
     const int64_t smb = pad256(adkv_softmax_workspace_bytes(B * Hq, T + 1));
@@ -1929,10 +1974,10 @@ int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k
                          smb ? ws + 2 * mat : nullptr, smb, stream);
     if (rc)
         return rc;
-    return adkv_forward_ov_gqa(weights, v_cache, v_new, out, v_params[0], v_params[1], v_params[2],
-                               v_params[3], v_params[4], B, Hq, H, T, D, n_super_cap, bits, ld,
-                               nullptr, v_ckpt, n_ckpt_cap, ckpt_interval, ws + 2 * mat + smb,
-                               workspace_bytes - 2 * mat - smb, stream);
+    return forward_ov_impl(weights, v_cache, v_new, out, v_params[0], v_params[1], v_params[2],
+                           v_params[3], v_params[4], B, Hq, H, T, D, n_super_cap, bits, ld,
+                           nullptr, v_ckpt, n_ckpt_cap, ckpt_interval, ws + 2 * mat + smb,
+                           workspace_bytes - 2 * mat - smb, stream, act_bf16);
 }
 
 } // extern "C"

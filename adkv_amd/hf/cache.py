@@ -220,7 +220,10 @@ class KVCacheLayer_ADKV:
         ctx = self._quant_len
         self._cap_buffers(ctx + 1)
 
-        f16 = lambda t: t.to(torch.float16).contiguous()
+        # fp16 and bf16 activations go in as they are; the kernels convert (see decode_fused)
+        same = query_states.dtype in (torch.float16, torch.bfloat16) \
+            and key_states.dtype == query_states.dtype == value_states.dtype
+        f16 = (lambda t: t.contiguous()) if same else (lambda t: t.to(torch.float16).contiguous())
         v = self._view
         S = self._ckpt_interval
         dev = query_states.device
@@ -236,7 +239,7 @@ class KVCacheLayer_ADKV:
             workspace=ws)
         self._quant_len = ctx + 1
         self._state_valid = False
-        return out.to(query_states.dtype), weights
+        return (out if out.dtype == query_states.dtype else out.to(query_states.dtype)), weights
 
     # ------------------------------------------------------------------ save / restore
     def state_dict(self) -> dict:

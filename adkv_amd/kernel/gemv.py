@@ -497,14 +497,20 @@ def decode_fused(
     ``forward_qk`` -> ``softmax(logits*scaling + mask)`` -> ``forward_ov``, with ``k_new`` / ``v_new``
     appended at slot ``T`` of both caches.  ``k_params`` / ``v_params`` are the five ``[nh, DIM]``
     fp16 tensors ``(zp, sc, alpha, beta, quant_target)``.  Returns ``(out [B,nh,DIM] fp16,
-    weights [B,nh,T+1] fp16)``.  ``workspace`` (uint8, 256-byte aligned, sized by
+    weights [B,nh,T+1] fp16)``.  ``q``, ``k_new`` and ``v_new`` may all be bfloat16: the kernels
+    round them to fp16 as they read them and return ``out`` in bfloat16, with the values of the
+    reference's ``.to(torch.float16)`` / ``.to(q.dtype)`` around its kernels
+    (llama_adkv.py:248-250, 274) but without those launches.  ``workspace`` (uint8, 256-byte aligned, sized by
     ``decode_fused_workspace_bytes``) may be passed to avoid the per-call allocation.
     """
     f16, u8 = torch.float16, torch.uint8
-    if not (q.dtype == f16 and k_new.dtype == f16 and v_new.dtype == f16 and k_cache.dtype == u8
-            and v_cache.dtype == u8 and k_cache.is_contiguous() and v_cache.is_contiguous()):
+    act = q.dtype            # float16 as in the reference, or bfloat16 (extension; see the docstring)
+    if not (act in (f16, torch.bfloat16) and k_new.dtype == act and v_new.dtype == act
+            and k_cache.dtype == u8 and v_cache.dtype == u8 and k_cache.is_contiguous()
+            and v_cache.is_contiguous()):
         for t, n in ((q, "q"), (k_new, "k_new"), (v_new, "v_new")):
-            _chk(t.dtype == f16, f"{n} must be float16")
+            _chk(t.dtype == (act if act == torch.bfloat16 else f16),
+                 f"{n} must be float16" + (" (or bfloat16 like q)" if act == torch.bfloat16 else ""))
         for t, n in ((k_cache, "k_cache"), (v_cache, "v_cache")):
             _chk(t.dtype == u8, f"{n} must be uint8")
             _chk(t.is_contiguous(), f"{n} must be contiguous (appended in place)")
@@ -545,7 +551,7 @@ def decode_fused(
     qf = q.contiguous()
     knf = k_new.reshape(B * nh, DIM).contiguous()
     vnf = v_new.reshape(B * nh, DIM).contiguous()
-    out = torch.empty((B, nq, DIM), dtype=torch.float16, device=dev)
+    out = torch.empty((B, nq, DIM), dtype=act, device=dev)
     wld = _row_pitch(n)
     weights = torch.empty((B, nq, wld), dtype=torch.float16, device=dev)
     arr = _lib.C.c_void_p * 5
@@ -554,7 +560,8 @@ def decode_fused(
             qf.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), knf.data_ptr(), vnf.data_ptr(),
             arr(*[t.data_ptr() for t in kp]), arr(*[t.data_ptr() for t in vp]),
             mptr, rpm, float(scaling), out.data_ptr(), weights.data_ptr(), wld,
-            B, nq, nh, T, DIM, n_super_cap, bits, kcp, vcp, ccap, civ,
+            B, nq, nh, T, DIM, n_super_cap, bits, _DT_BF16 if act == torch.bfloat16 else _DT_F16,
+            kcp, vcp, ccap, civ,
             workspace.data_ptr(), workspace.numel(), _lib.current_stream_ptr(dev))
     _lib.check(rc, "decode_fused")
     return out, weights[:, :, :n]

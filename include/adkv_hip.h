@@ -222,6 +222,10 @@ int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void
  * fp16 [H, D].  mask: optional fp32 additive mask as in adkv_softmax.  out: fp16 [B, Hq, D].
  * weights_out: optional fp16 [B, Hq, weights_ld] with weights_ld == adkv_row_pitch(T + 1), columns
  * 0..T valid (the attention weights the reference returns); when NULL they live in the workspace.  Checkpoint tensors as in the _ex entry points (NULL = none).
+ * act_dtype: ADKV_DT_F16, or ADKV_DT_BF16 when q, k_new, v_new and out are bfloat16: they are
+ * rounded to fp16 as they are read and the fp16 result to bf16 as it is written, the values of
+ * the reference's .to(torch.float16) / .to(q.dtype) around its kernels (llama_adkv.py:248-250, 274)
+ * without the four conversion launches.  Logits and weights stay fp16.
  * workspace: >= adkv_decode_fused_workspace_bytes(...) bytes, 256-byte aligned.
  */
 int64_t adkv_decode_fused_workspace_bytes(int B, int Hq, int H, int T, int D, int n_ckpt_cap,
@@ -230,7 +234,7 @@ int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k
                       const void *v_new, const void *const *k_params, const void *const *v_params,
                       const void *mask, int rows_per_mask_row, float scaling,
                       void *out, void *weights_out, int64_t weights_ld,
-                      int B, int Hq, int H, int T, int D, int n_super_cap, int bits,
+                      int B, int Hq, int H, int T, int D, int n_super_cap, int bits, int act_dtype,
                       void *k_ckpt, void *v_ckpt, int n_ckpt_cap, int ckpt_interval,
                       void *workspace, int64_t workspace_bytes, void *stream);
 

@@ -484,6 +484,55 @@ def test_decode_step_replays_from_a_captured_graph(gpu, H, Hq, T, S, bits):
             assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), rep
 
 
+@pytest.mark.parametrize("B,H,Hq,T,S,bits", [
+    (2, 4, 4, 257, 0, 4),        # vector kernels, one segment
+    (2, 3, 3, 530, 64, 4),       # vector kernels, a few segments (narrow partial-sum kernel)
+    (1, 2, 2, 2100, 64, 4),      # many segments (wide partial-sum kernel)
+    (40, 32, 32, 300, 64, 4),    # enough units for four channels per lane
+    (2, 2, 8, 530, 64, 4),       # matrix-core kernels, 4 query heads per KV head
+    (1, 2, 16, 200, 32, 2),      # 2-bit codes, 8 query heads per KV head
+])
+def test_decode_fused_takes_bfloat16_activations(gpu, B, H, Hq, T, S, bits):
+    """q, k_new, v_new in bfloat16: the kernels round them to fp16 on the way in and the result to
+    bfloat16 on the way out.  Everything equals the fp16 call on `.to(float16)` inputs followed by
+    `.to(bfloat16)`: output bits, weights, appended codes, checkpoints."""
+    D = 128
+    tps = 32 // bits
+    kp = [t.to(gpu) for t in synth.make_params(H, D, seed=3, bits=bits).astuple()]
+    vp = [t.to(gpu) for t in synth.make_params(H, D, seed=4, bits=bits).astuple()]
+    k = synth.make_k(B, H, T, D, dtype=torch.float16).to(gpu)
+    v = synth.make_v(B, H, T, D, dtype=torch.float16).to(gpu)
+    g = torch.Generator().manual_seed(T)
+    qb, kb, vb = [(1.01 * torch.randn(B, h, 1, D, generator=g)).to(torch.bfloat16).to(gpu)
+                  for h in (Hq, H, H)]
+    ncap = (T + tps) // S + 1 if S else 0
+
+    def fresh():
+        kc = synth.alloc_cache(B, H, T + tps, D, gpu, bits=bits)
+        vc = synth.alloc_cache(B, H, T + tps, D, gpu, bits=bits)
+        kk = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=gpu) if S else None
+        vk = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=gpu) if S else None
+        ks = torch.zeros(B, H, D, 2, dtype=torch.float16, device=gpu)
+        vs = torch.zeros(B, H, D, 2, dtype=torch.float16, device=gpu)
+        gemv.append_kv_pair(kc, vc, k, v, kp, vp, 0, ks, vs, k_ckpt=kk, v_ckpt=vk, ckpt_interval=S, bits=bits)
+        return kc, vc, kk, vk
+
+    a = fresh()
+    out_a, w_a = gemv.decode_fused(qb.half(), a[0], a[1], kb.half(), vb.half(), kp, vp, T, D ** -0.5, None,
+                                   k_ckpt=a[2], v_ckpt=a[3], ckpt_interval=S, bits=bits)
+    b = fresh()
+    out_b, w_b = gemv.decode_fused(qb, b[0], b[1], kb, vb, kp, vp, T, D ** -0.5, None,
+                                   k_ckpt=b[2], v_ckpt=b[3], ckpt_interval=S, bits=bits)
+    torch.cuda.synchronize()
+    assert out_a.dtype == torch.float16 and out_b.dtype == torch.bfloat16
+    assert torch.equal(out_a.to(torch.bfloat16).view(torch.int16), out_b.view(torch.int16))
+    assert torch.equal(w_a.view(torch.int16), w_b.view(torch.int16))
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    if S:
+        assert torch.equal(a[2].view(torch.int16), b[2].view(torch.int16))
+        assert torch.equal(a[3].view(torch.int16), b[3].view(torch.int16))
+
+
 # ------------------------------------------------------------------ grouped-query / matrix-core kernels
 def _gqa_case(gpu, oracle, B, Hkv, G, T, S, seed=0, bits=4):
     """One QK + OV pass with G query heads per KV head against the oracle run once per group member
