@@ -60,6 +60,40 @@ def test_argument_validation_in_c_abi_needs_no_device():
     assert L.adkv_forward_ov_workspace_bytes(128, 32, 4096, 128, 17, 256) == 2 * 128 * 32 * 128 * 4
 
 
+def test_paired_append_and_fused_decode_validation_needs_no_device():
+    """The newer entry points reject bad dtypes, strides and NULL parameter arrays on the host."""
+    L = _lib.lib()
+    one = ctypes.c_void_p(16)
+    arr5 = (ctypes.c_void_p * 5)(*[16] * 5)
+    st3 = lambda b, h, t: (ctypes.c_int64 * 3)(b, h, t)
+    pair = lambda dtype, ks, vs, params=arr5: [one, one, one, one, dtype, ks, vs, params, params,
+                                               1, 1, 0, 8, 128, 1, 4, one, one, None, None, 0, 0, None]
+    assert L.adkv_append_kv_pair(*pair(0, None, None)) == -6               # fp32 rows are not taken
+    assert L.adkv_append_kv_pair(*pair(1, None, None, None)) == -1         # no parameter arrays
+    assert L.adkv_append_kv_pair(*pair(1, st3(1024, 128, 127), None)) == -3   # token stride below D
+    assert L.adkv_append_kv_pair(*pair(2, st3(1025, 128, 128), None)) == -3   # odd stride: rows unaligned
+    fused = [one] * 5 + [arr5, arr5, None, 1, 1.0, one, None, 0, 1, 1, 1, 8, 128, 2, 4, 0,
+             None, None, 0, 0, one, 1 << 20, None]
+    assert L.adkv_decode_fused(*fused) == -6                                # activation dtype must be f16 / bf16
+
+
+def test_row_strides_of_projection_outputs():
+    """A [B, T, H, D] projection output viewed head-first is handed over with its strides; layouts
+    the library cannot read in place (odd strides, channel stride 2) are packed first."""
+    from adkv_amd.kernel.gemv import _row_strides
+    x = torch.zeros(2, 5, 3, 128, dtype=torch.bfloat16)
+    t, s = _row_strides(x.permute(0, 2, 1, 3))
+    assert t.data_ptr() == x.data_ptr() and list(s) == [5 * 3 * 128, 128, 3 * 128]
+    t, s = _row_strides(x.permute(0, 2, 1, 3).contiguous())
+    assert s is None
+    odd = torch.zeros(2, 3, 5, 129, dtype=torch.float16)[..., :128]         # token stride 129
+    t, s = _row_strides(odd)
+    assert s is None and t.is_contiguous()
+    every_other = torch.zeros(2, 3, 5, 256, dtype=torch.float16)[..., ::2]
+    t, s = _row_strides(every_other)
+    assert s is None and t.is_contiguous()
+
+
 def _p(nh, D, dtype=torch.float16):
     return [torch.zeros(nh, D, dtype=dtype) for _ in range(5)]
 
