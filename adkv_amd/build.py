@@ -1,6 +1,7 @@
 """Builds libadkv_hip.so for gfx950 with hipcc (cross-compiles without a GPU)."""
 from __future__ import annotations
 
+import glob
 import os
 import subprocess
 import sys
@@ -9,8 +10,8 @@ _DIR = os.path.dirname(os.path.abspath(__file__))
 SOURCES = [os.path.join(_DIR, "csrc", "adkv_kernels.hip"),
            os.path.join(_DIR, "csrc", "adkv_fp32.hip"),
            os.path.join(_DIR, "csrc", "fp16_baseline.hip")]
-HEADERS = [os.path.join(_DIR, "csrc", "adkv_device.h"),
-           os.path.join(_DIR, "..", "include", "adkv_hip.h")]
+HEADERS = sorted(glob.glob(os.path.join(_DIR, "csrc", "*.h"))) + \
+    [os.path.join(_DIR, "..", "include", "adkv_hip.h")]
 LIB_PATH = os.path.join(_DIR, "libadkv_hip.so")
 
 # -ffp-contract=off: the fp16 recurrence needs "q*sc + zp" as two roundings where the reference

@@ -21,8 +21,9 @@
 
 #include <stdlib.h>
 
+#include <atomic>
 #include <initializer_list>
-
+#include <mutex>
 #include <type_traits>
 
 #pragma clang fp contract(off)
@@ -1415,14 +1416,32 @@ static void launch_units(long threads, int big, F256 f256, FBIG fbig)
 // Whether single-query-head launches (GQ == 1, head dim 128) also take the matrix-core kernels:
 // the built-in choice, overridden by ADKV_MFMA=0/1 in the environment, overridden by
 // adkv_set_mha_kernel().
-static int g_mha_kernel = -1;
+// The environment is read once, when the first launch asks; the override is an atomic so that
+// launches from several host threads never see a torn value.
+static std::atomic<int> g_mha_kernel{-1};
+static int mha_kernel_default()
+{
+    static const int from_env = [] {
+        const char *e = getenv("ADKV_MFMA");
+        return (e ? atoi(e) : ADKV_MFMA_DEFAULT) != 0 ? 1 : 0;
+    }();
+    return from_env;
+}
 static bool mfma_for_mha()
 {
-    if (g_mha_kernel < 0) {
-        const char *e = getenv("ADKV_MFMA");
-        g_mha_kernel = (e ? atoi(e) : ADKV_MFMA_DEFAULT) != 0;
-    }
-    return g_mha_kernel != 0;
+    const int v = g_mha_kernel.load(std::memory_order_relaxed);
+    return (v < 0 ? mha_kernel_default() : v) != 0;
+}
+
+// ADKV_ENCODE_CPL=1/2 pins the encoder's channels per lane (a measurement aid); read once.
+static int encode_cpl_override()
+{
+    static const int from_env = [] {
+        const char *e = getenv("ADKV_ENCODE_CPL");
+        const int v = e ? atoi(e) : 0;
+        return (v == 1 || v == 2) ? v : 0;
+    }();
+    return from_env;
 }
 
 static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval, int bits = 4)
@@ -1441,7 +1460,10 @@ extern "C" {
 
 int adkv_abi_version(void) { return 10; }
 
-void adkv_set_mha_kernel(int use_matrix_cores) { g_mha_kernel = use_matrix_cores; }
+void adkv_set_mha_kernel(int use_matrix_cores)
+{
+    g_mha_kernel.store(use_matrix_cores < 0 ? -1 : (use_matrix_cores != 0), std::memory_order_relaxed);
+}
 
 int adkv_last_hip_error(void) { return g_last_hip_error; }
 
@@ -1524,11 +1546,8 @@ static int encode_common(void *cache, const void *kv_new,
     const long channels = (long)BH * D;
     const long tensors = second ? 2 : 1;
     int cpl = tensors * channels > 2L * 64 * N_SIMD + 32768 ? 2 : 1;
-    if (const char *e = getenv("ADKV_ENCODE_CPL")) {
-        const int v = atoi(e);
-        if (v == 1 || v == 2)
-            cpl = v;
-    }
+    if (const int forced = encode_cpl_override())
+        cpl = forced;
     const long lanes = channels / cpl;
     const dim3 grid((unsigned)((lanes + 255) / 256), (unsigned)tensors), block(256);
     EncTensor first;

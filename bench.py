@@ -10,7 +10,7 @@ buffers so no cache level can serve re-reads.
 
 Prints ONE JSON line.  `roofline` prices the dominant kernel (the QK scan) on its algorithmic
 bytes, B*H*T*d*bits/8 code bytes per launch, against the 8 TB/s HBM peak; `cpu_baseline` times the
-C oracle of the same step on a bounded sample on the host.
+reference's PyTorch CPU path (eager fp32 recurrence + attention, all host cores) on a bounded sample.
 """
 from __future__ import annotations
 
@@ -56,43 +56,67 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fp16-comparator", action="store_true",
                     help="skip timing the fp16-KV decode kernel beside the ADKV step")
-    ap.add_argument("--cpu-sample-heads", type=int, default=0,
-                    help="heads of one sequence timed on the host (0 = auto, about 10-30 s)")
+    ap.add_argument("--cpu-sample-batch", type=int, default=16,
+                    help="sequences of the batch the host baseline runs (full context, all heads; "
+                         "16 take about 10 s)")
     return ap.parse_args()
 
 
 def cpu_baseline(args, T, D):
-    """C oracle (a scalar port of the same fp16 recurrence) timed on one host core over a sample:
-    `hs` heads of one sequence, full context; scaled to a whole sequence of H heads."""
+    """The reference's PyTorch CPU path timed on this host: for a sample of the batch, the eager
+    fp32 per-token recurrence over whole [B, C] tensors for K and for V over the full context
+    (src/adkv/train/train_model.py:61-81), then softmax(q.K^T/sqrt(d)).V for the single query
+    (src/adkv/train/llama_attention.py:41-44), on all host cores.  That is one decode-attention
+    step of one layer, the unit the GPU number is quoted in.  The C oracle of the fp16 recurrence
+    (one core) is timed beside it as a secondary figure."""
     import numpy as np
     import torch
     from adkv_amd import synth
     from oracle import oracle as O
+    from oracle import torch_cpu
 
     H = args.heads
-    hs = args.cpu_sample_heads or min(H, 16)
-    kp, vp = synth.make_params(H, D, seed=3), synth.make_params(H, D, seed=4)
-    np16 = lambda t: t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.float16)
-    kpn = [np16(t)[:hs] for t in kp.astuple()]
-    vpn = [np16(t)[:hs] for t in vp.astuple()]
-    k = np16(synth.make_k(1, hs, T + 1, D, dtype=torch.float16))
-    v = np16(synth.make_v(1, hs, T + 1, D, dtype=torch.float16))
-    q = np16(synth.make_q(1, hs, D))
-    kc, vc = O.alloc_cache(1, hs, T + 8, D), O.alloc_cache(1, hs, T + 8, D)
-    O.encode_kv_f16(kc, k[:, :, :T], *kpn)
-    O.encode_kv_f16(vc, v[:, :, :T], *vpn)
+    C = H * D
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    Bs = max(1, min(args.batch, args.cpu_sample_batch))
+    f32 = lambda p: [t.float().reshape(-1) for t in p.astuple()]
+    kp, vp = f32(synth.make_params(H, D, seed=3)), f32(synth.make_params(H, D, seed=4))
+    rows = lambda x: x.permute(0, 2, 1, 3).reshape(Bs, T, C).contiguous()          # [B, T, H*d]
+    k = rows(synth.make_k(Bs, H, T, D))
+    v = rows(synth.make_v(Bs, H, T, D))
+    q = synth.make_q(Bs, H, D, dtype=torch.float32).reshape(Bs, C)
+    torch_cpu.decode_step(q, k[:, :64], v[:, :64], kp, vp, H, D ** -0.5)            # warm-up
     t0 = time.perf_counter()
-    O.decode_step_f16(q, kc, vc, k[:, :, T:], v[:, :, T:], kpn, vpn, T, D ** -0.5)
+    torch_cpu.decode_step(q, k, v, kp, vp, H, D ** -0.5)
     dt = time.perf_counter() - t0
-    t_seq = dt * (H / hs)                      # one layer-step for one whole sequence
-    return {
-        "value": 1.0 / (N_LAYERS_MODEL * t_seq),
+    res = {
+        "value": Bs / (N_LAYERS_MODEL * dt),
         "unit": "tokens/s",
-        "cores": 1,
+        "cores": cores,
         "kind": "port",
-        "sample": f"C oracle, 1 sequence x {hs} of {H} heads x ctx {T}, one layer-step = {dt:.2f} s; "
-                  f"scaled linearly to {H} heads",
+        "sample": f"PyTorch CPU eager fp32 (torch {torch.__version__}, {cores} threads): {Bs} of {args.batch} "
+                  f"sequences x {H} heads x ctx {T}, one full layer-step (per-token recurrence for K and V, "
+                  f"then single-query attention) = {dt:.2f} s; value = {Bs} / (32 layers x that time), "
+                  f"i.e. the rate at batch {Bs}, not extrapolated",
     }
+    # secondary: the C oracle of the fp16 recurrence (bit-exact checker), one core
+    hs = min(H, 8)
+    np16 = lambda t: t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.float16)
+    kq = synth.make_params(H, D, seed=3)
+    pn = [np16(t)[:hs] for t in kq.astuple()]
+    kk = np16(synth.make_k(1, hs, T + 1, D, dtype=torch.float16))
+    qq = np16(synth.make_q(1, hs, D))
+    kc, vc = O.alloc_cache(1, hs, T + 8, D), O.alloc_cache(1, hs, T + 8, D)
+    O.encode_kv_f16(kc, kk[:, :, :T], *pn)
+    O.encode_kv_f16(vc, kk[:, :, :T], *pn)
+    t0 = time.perf_counter()
+    O.decode_step_f16(qq, kc, vc, kk[:, :, T:], kk[:, :, T:], pn, pn, T, D ** -0.5)
+    dc = time.perf_counter() - t0
+    res["c_oracle_fp16"] = {"value": 1.0 / (N_LAYERS_MODEL * dc * H / hs), "unit": "tokens/s", "cores": 1,
+                            "sample": f"C oracle of the fp16 recurrence, 1 sequence x {hs} of {H} heads x ctx {T} "
+                                      f"in {dc:.2f} s, scaled linearly to {H} heads"}
+    return res
 
 
 def fp16_comparator(args, dev, adkv_ms):

@@ -673,7 +673,7 @@ def test_paired_append_reads_projection_outputs_in_place(gpu, oracle, dtype, str
         assert np.array_equal(_np16(states[i]).view(np.uint16), want[i][1]), i
 
 
-@pytest.mark.parametrize("G,bits", [(4, 4), (8, 4), (2, 2), (8, 2)])
+@pytest.mark.parametrize("G,bits", [(4, 4), (8, 4), (2, 2), (4, 2), (8, 2)])
 def test_grouped_query_kernels_in_16_wave_workgroups(gpu, oracle, G, bits):
     """A launch big enough for the 16-wave workgroups (128 KV heads x 64 segments = 8192 units):
     the instantiations the small cases above never reach, including the eight-head QK kernel
@@ -851,3 +851,116 @@ def test_encode_rounding_boundaries(gpu, oracle, bits):
     gemv.append_kv(cache, x.to(gpu), *[t.to(gpu) for t in params], 0, st, bits=bits)
     torch.cuda.synchronize()
     assert np.array_equal(cache.cpu().numpy(), want)
+
+
+def test_long_context_grouped_query_full_size(gpu, oracle):
+    """B=16, 32 query heads over 8 KV heads, d=128, ctx 131072, 2-bit codes, bfloat16 activations:
+    the whole step through decode_fused at its real size (the 16-wave matrix-core kernels with
+    four query heads per KV head, 64 segments, chunked softmax).  Size-independent properties over
+    the whole tensor, and two sampled (sequence, KV head) pairs against the oracle:
+    (1) encode(T) + the in-kernel append of token T == encode(T+1), byte for byte, K and V;
+    (2) the replayed state after T-1 == the encoder's, and it is recorded as the closing checkpoint;
+    (3) attention weights sum to one; outputs and weights of the samples within tolerance."""
+    B, H, G, D, T, S, bits = 16, 8, 4, 128, 131072, 256, 2
+    Hq, tps = H * G, 16
+    bf = torch.bfloat16
+    kp = synth.make_params(H, D, bits=bits, seed=3).to(gpu)
+    vp = synth.make_params(H, D, bits=bits, seed=4).to(gpu)
+    caches, fulls, states, ckpts, news = [], [], [], [], []
+    samples = [(0, 0), (B - 1, H - 1)]
+    rows = {bh: [] for bh in samples}                       # the sampled heads' input rows, for the oracle
+    for make, p, seed in ((synth.make_k, kp, 0), (synth.make_v, vp, 1)):
+        x = make(B, H, T + 1, D, seed=seed, dtype=torch.float16, device=gpu)
+        x[:, :, T] = x[:, :, T].to(bf).to(torch.float16)        # the new token arrives as bfloat16
+        ncap = (T + tps) // S + 1
+        part = synth.alloc_cache(B, H, T + tps, D, gpu, bits=bits)
+        full = synth.alloc_cache(B, H, T + tps, D, gpu, bits=bits)
+        st = torch.zeros(B, H, D, 2, dtype=torch.float16, device=gpu)
+        st_full = torch.zeros_like(st)
+        ck = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=gpu)
+        gemv.append_kv(part, x[:, :, :T], *p.astuple(), 0, st, ckpt=ck, ckpt_interval=S, bits=bits)
+        gemv.append_kv(full, x, *p.astuple(), 0, st_full, bits=bits)
+        caches.append(part); fulls.append(full); states.append(st); ckpts.append(ck)
+        news.append(x[:, :, T:T + 1].to(bf))
+        for (b, h) in samples:
+            rows[(b, h)].append(_np16(x[b:b + 1, h:h + 1]))
+        del x
+    torch.cuda.empty_cache()
+    q = synth.make_q(B, Hq, D, dtype=bf, device=gpu)
+    kc, vc = caches[0].clone(), caches[1].clone()
+    out, w = gemv.decode_fused(q, kc, vc, news[0], news[1], kp.astuple(), vp.astuple(), T, D ** -0.5,
+                               k_ckpt=ckpts[0], v_ckpt=ckpts[1], ckpt_interval=S, bits=bits)
+    torch.cuda.synchronize()
+    assert out.dtype == bf and out.shape == (B, Hq, D) and w.shape == (B, Hq, T + 1)
+    assert torch.equal(kc, fulls[0]) and torch.equal(vc, fulls[1])                                 # (1)
+    for ck, st in zip(ckpts, states):                                                              # (2)
+        assert torch.equal(ck[:, :, T // S - 1].view(torch.int16), st.view(torch.int16))
+    st_qk = torch.zeros_like(states[0])
+    gemv.forward_qk(q.to(torch.float16), caches[0].clone(), news[0].to(torch.float16), *kp.astuple(), T,
+                    SMIN, SMAX, state_out=st_qk, ckpt=ckpts[0], ckpt_interval=S, bits=bits)
+    assert torch.equal(st_qk.view(torch.int16), states[0].view(torch.int16))
+    assert torch.all(torch.abs(w.float().sum(-1) - 1) < 2e-2)                                      # (3)
+    qn = _np16(q.to(torch.float16)).reshape(B, H, G, D)
+    got = out.float().cpu().numpy().reshape(B, H, G, D)
+    kpn, vpn = [_np16(t) for t in kp.astuple()], [_np16(t) for t in vp.astuple()]
+    with oracle.code_bits(bits):
+        for (b, h) in samples:
+            xk, xv = rows[(b, h)]
+            ko, vo = oracle.alloc_cache(1, 1, T + tps, D), oracle.alloc_cache(1, 1, T + tps, D)
+            oracle.encode_kv_f16(ko, xk[:, :, :T], *[a[h:h + 1] for a in kpn])
+            oracle.encode_kv_f16(vo, xv[:, :, :T], *[a[h:h + 1] for a in vpn])
+            assert np.array_equal(caches[0][b:b + 1, h:h + 1].cpu().numpy(), ko), (b, h)
+            assert np.array_equal(caches[1][b:b + 1, h:h + 1].cpu().numpy(), vo), (b, h)
+            for j in (0, G - 1):
+                want, w_want, _ = oracle.decode_step_f16(
+                    qn[b:b + 1, h:h + 1, j], ko.copy(), vo.copy(), xk[:, :, T:], xv[:, :, T:],
+                    [a[h:h + 1] for a in kpn], [a[h:h + 1] for a in vpn], T, D ** -0.5)
+                # fp16 result rounded to bf16: half a bf16 ulp on top of the 2e-3 of the fp16 path
+                tol = 2e-3 + 2.0 ** -8 * np.abs(want[0, 0])
+                assert np.all(np.abs(got[b, h, j] - want[0, 0]) <= tol), (b, h, j)
+                # the fp16 logit may sit one ulp from the oracle's (fp32 sums in another order):
+                # a factor exp(ulp * scaling) on the weight, below 1 %
+                wg = _np16(w[b, h * G + j]).astype(np.float64)
+                ww = w_want[0, 0].astype(np.float64)
+                assert np.all(np.abs(wg - ww) <= 0.02 * ww + 1e-7), (b, h, j)
+
+
+def test_streaming_quantiser_full_size(gpu, oracle):
+    """B=8, 32 heads, d=128: prefill-quantise 32768 tokens with checkpoints every 256 (one channel
+    per lane, 128 checkpoints), then 256 single-token appends with the carried state.  The stream
+    equals a one-shot encode of all 33024 tokens byte for byte (whole tensor), two sampled heads
+    equal the oracle's codes and final state, and sampled checkpoints equal the oracle's state
+    after that many tokens."""
+    B, H, D, T, n_app, S = 8, 32, 128, 32768, 256, 256
+    p = synth.make_params(H, D).to(gpu)
+    x = synth.make_k(B, H, T + n_app, D, dtype=torch.float16, device=gpu)
+    ncap = (T + n_app) // S + 1
+    cache = synth.alloc_cache(B, H, T + n_app + 8, D, gpu)
+    ck = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=gpu)
+    st = torch.zeros(B, H, D, 2, dtype=torch.float16, device=gpu)
+    gemv.append_kv(cache, x[:, :, :T], *p.astuple(), 0, st, ckpt=ck, ckpt_interval=S)
+    st_prefill = st.clone()
+    for i in range(n_app):
+        gemv.append_kv(cache, x[:, :, T + i:T + i + 1], *p.astuple(), T + i, st, ckpt=ck, ckpt_interval=S)
+    once = synth.alloc_cache(B, H, T + n_app + 8, D, gpu)
+    ck1 = torch.zeros_like(ck)
+    st1 = torch.zeros_like(st)
+    gemv.encode_kv(once, x, *p.astuple(), SMIN, SMAX, state_out=st1, ckpt=ck1, ckpt_interval=S)
+    torch.cuda.synchronize()
+    assert torch.equal(cache, once)
+    assert torch.equal(st.view(torch.int16), st1.view(torch.int16))
+    assert torch.equal(ck.view(torch.int16), ck1.view(torch.int16))
+    assert ck[:, :, (T + n_app) // S - 1].any() and not ck[:, :, (T + n_app) // S:].any()
+    assert torch.equal(ck[:, :, T // S - 1].view(torch.int16), st_prefill.view(torch.int16))
+    pn = [_np16(t) for t in p.astuple()]
+    for (b, h) in [(0, 0), (B - 1, H - 1)]:
+        ph = [a[h:h + 1] for a in pn]
+        xs = _np16(x[b:b + 1, h:h + 1])
+        want = oracle.alloc_cache(1, 1, T + n_app + 8, D)
+        st_want = oracle.encode_kv_f16(want, xs, *ph)
+        assert np.array_equal(cache[b:b + 1, h:h + 1].cpu().numpy(), want), (b, h)
+        assert np.array_equal(_np16(st[b:b + 1, h:h + 1]).view(np.uint16), st_want), (b, h)
+        for j in (0, 1, 63, 127, 128):                       # state before token (j+1)*S
+            scratch = oracle.alloc_cache(1, 1, (j + 1) * S, D)
+            sj = oracle.encode_kv_f16(scratch, xs[:, :, :(j + 1) * S], *ph)
+            assert np.array_equal(_np16(ck[b:b + 1, h:h + 1, j]).view(np.uint16), sj), (b, h, j)

@@ -124,35 +124,191 @@ def test_prefill_then_decode_steps_match_oracle(gpu, oracle, monkeypatch, interv
     assert layer._cap_len == 128
 
 
-@pytest.mark.gpu
-def test_tiny_llama_generate(gpu):
-    """Random-init 2-layer Llama (2 heads of 128) decodes greedily through the ADKV cache; with
-    near-lossless parameters (tiny scale) its tokens match the dense fp32 model's."""
-    transformers = pytest.importorskip("transformers")
-    from transformers import LlamaConfig, LlamaForCausalLM
-    from adkv_amd.hf.llama_adkv import ADKVConfig, LlamaForCausalLM_ADKV
+def _tiny_cfg(heads, kv_heads):
+    from transformers import LlamaConfig
+    return LlamaConfig(vocab_size=128, hidden_size=128 * heads, intermediate_size=512, num_hidden_layers=2,
+                       num_attention_heads=heads, num_key_value_heads=kv_heads, head_dim=128,
+                       max_position_embeddings=256, attn_implementation="eager")
 
-    cfg = LlamaConfig(vocab_size=128, hidden_size=256, intermediate_size=512, num_hidden_layers=2,
-                      num_attention_heads=2, num_key_value_heads=2, max_position_embeddings=256,
-                      attn_implementation="eager")
+
+def _rope(x, cos, sin):
+    """Rotary embedding written out (x [B, H, T, d]; cos, sin [B, T, d]): the textbook form,
+    x*cos + rotate_half(x)*sin with rotate_half(x) = (-x[d/2:], x[:d/2])."""
+    d = x.shape[-1]
+    rot = torch.cat((-x[..., d // 2:], x[..., :d // 2]), dim=-1)
+    return x * cos[:, None] + rot * sin[:, None]
+
+
+class _AttentionTap:
+    """Records, for every call of every attention module, what went in (hidden states, rotary
+    tables, mask) and what reached o_proj, so a test can recompute the step without the module."""
+
+    def __init__(self, model):
+        self.calls = []            # dicts: layer, hidden, cos, sin, mask, ctx (input of o_proj), out
+        self.cache = None          # the cache object the model made for itself
+        self._handles = []
+        for i, layer in enumerate(model.model.layers):
+            att = layer.self_attn
+            self._handles.append(att.register_forward_pre_hook(self._pre(i), with_kwargs=True))
+            self._handles.append(att.o_proj.register_forward_pre_hook(self._ctx))
+            self._handles.append(att.register_forward_hook(self._post))
+
+    def _pre(self, i):
+        def hook(mod, args, kwargs):
+            cos, sin = kwargs["position_embeddings"]
+            m = kwargs.get("attention_mask")
+            self.cache = kwargs.get("past_key_values")
+            self.calls.append(dict(layer=i, hidden=kwargs["hidden_states"].detach().clone(),
+                                   cos=cos.detach().clone(), sin=sin.detach().clone(),
+                                   mask=None if m is None else m.detach().clone()))
+        return hook
+
+    def _ctx(self, mod, args):
+        self.calls[-1]["ctx"] = args[0].detach().clone()
+
+    def _post(self, mod, args, out):
+        self.calls[-1]["out"] = out[0].detach().clone()
+
+    def close(self):
+        for h in self._handles:
+            h.remove()
+
+
+def _check_decode_calls_against_oracle(oracle, model, calls, params16, pad, prompt_len):
+    """Every single-token call of every attention module, recomputed from the hidden states that
+    entered it: projections and rotary embedding here, quantised attention by the oracle (its own
+    caches, filled from the prompt call's K/V), query head j reading KV head j // G, scaling
+    head_dim**-0.5, the additive mask rebuilt from the known left padding.  The context that
+    reached o_proj must agree within 2e-3 and the module's output with o_proj of the oracle's."""
+    cfg = model.config
+    Hq, H, D = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    G = Hq // H
+    scaling = D ** -0.5
+    caches, T = {}, {}
+    worst = 0.0
+    n_decode = 0
+    for c in calls:
+        att = model.model.layers[c["layer"]].self_attn
+        hs = c["hidden"].float()
+        B, Tq, _ = hs.shape
+        w = lambda lin: lin.weight.detach().float()
+        split = lambda x, n: x.view(B, Tq, n, D).transpose(1, 2)
+        q = _rope(split(hs @ w(att.q_proj).T, Hq), c["cos"].float(), c["sin"].float())
+        k = _rope(split(hs @ w(att.k_proj).T, H), c["cos"].float(), c["sin"].float())
+        v = split(hs @ w(att.v_proj).T, H)
+        kpn, vpn = params16[c["layer"]]
+        if c["layer"] not in caches:                       # the prompt: quantise, nothing to compare
+            assert Tq == prompt_len
+            ko = oracle.alloc_cache(B, H, 256, D)
+            vo = oracle.alloc_cache(B, H, 256, D)
+            oracle.encode_kv_f16(ko, _np16(k.half()), *kpn)
+            oracle.encode_kv_f16(vo, _np16(v.half()), *vpn)
+            caches[c["layer"]], T[c["layer"]] = (ko, vo), Tq
+            continue
+        assert Tq == 1
+        ko, vo = caches[c["layer"]]
+        t = T[c["layer"]]
+        mask = np.zeros((B, 1, t + 1), np.float32)
+        for b in range(B):
+            mask[b, 0, :pad[b]] = -np.inf
+        ctx = np.zeros((B, Hq, D))
+        qn = _np16(q.half()).reshape(B, H, G, D)
+        for j in range(G):                                  # query head h*G + j reads KV head h
+            kc, vc = ko.copy(), vo.copy()
+            o, _, _ = oracle.decode_step_f16(qn[:, :, j], kc, vc, _np16(k.half()), _np16(v.half()),
+                                             kpn, vpn, t, scaling, mask=mask)
+            ctx.reshape(B, H, G, D)[:, :, j] = o
+        caches[c["layer"]], T[c["layer"]] = (kc, vc), t + 1
+        got_ctx = c["ctx"].float().cpu().numpy().reshape(B, Hq, D)
+        err = float(np.max(np.abs(got_ctx - ctx)))
+        worst = max(worst, err)
+        assert err <= 2e-3, (c["layer"], t, err)
+        want_out = torch.from_numpy(ctx.reshape(B, 1, Hq * D)).float().to(hs.device) @ w(att.o_proj).T
+        assert torch.allclose(c["out"].float(), want_out, atol=2e-3, rtol=0), (c["layer"], t)
+        n_decode += 1
+    return caches, T, worst, n_decode
+
+
+def _tiny_raw_calibration(layers, n, seed):
+    """Raw (unconstrained) calibration parameters as the reference's trainer stores them."""
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda: {"init_zp": 0.05 * torch.randn(n, generator=g),
+                  "init_log_sc": math.log(0.03) + 0.2 * torch.randn(n, generator=g),
+                  "alpha": 2.5 + 0.5 * torch.randn(n, generator=g),       # sigmoid -> ~0.92
+                  "beta": -0.5 + 0.5 * torch.randn(n, generator=g),       # 0.1*sigmoid -> ~0.04
+                  "target": 3.5 + 0.1 * torch.randn(n, generator=g)}
+    return [(mk(), mk()) for _ in range(layers)]
+
+
+def _deployment_params16(raw, H, D):
+    """exp / sigmoid / 0.1*sigmoid of the raw values (train_model.py:127-134) in numpy, rounded to
+    fp16 as the module's fp16 buffers do: what the oracle is fed."""
+    out = []
+    for pair in raw:
+        both = []
+        for sd in pair:
+            f = {k: v.numpy().astype(np.float32) for k, v in sd.items()}
+            sig = lambda a: (1.0 / (1.0 + np.exp(-a.astype(np.float64)))).astype(np.float32)
+            vals = (f["init_zp"], np.exp(f["init_log_sc"].astype(np.float64)).astype(np.float32),
+                    sig(f["alpha"]), (0.1 * sig(f["beta"]).astype(np.float64)).astype(np.float32), f["target"])
+            both.append([a.astype(np.float16).reshape(H, D) for a in vals])
+        out.append(tuple(both))
+    return out
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("heads,kv_heads", [(2, 2), (4, 2)])
+def test_tiny_llama_decode_path_matches_oracle_and_dense_model(gpu, oracle, tmp_path, heads, kv_heads):
+    """Random-init 2-layer Llama, a left-padded batch of two prompts, 8 greedy steps through the
+    ADKV cache with parameters read from calibration files (ckpt_{k,v}_{L}.pt -> load_calibration
+    -> load_adkv_config, the route of tools/perf_e2e.py:37-60).  Every decode-path call of every
+    attention module is recomputed with the oracle (see _check_decode_calls_against_oracle); the
+    packed caches at the end are the oracle's byte for byte; and the generated tokens are the
+    dense fp32 model's (the parameters quantise finely enough that the greedy choice survives)."""
+    pytest.importorskip("transformers")
+    from transformers import LlamaForCausalLM
+    from adkv_amd import calib
+    from adkv_amd.hf.llama_adkv import LlamaForCausalLM_ADKV
+
+    cfg = _tiny_cfg(heads, kv_heads)
     torch.manual_seed(0)
     dense = LlamaForCausalLM(cfg).to(gpu).eval()
     model = LlamaForCausalLM_ADKV(cfg).to(gpu).eval()
     model.load_state_dict(dense.state_dict())
-    n = 2 * 128
-    # delta coding with alpha = 1 and an adaptive scale tracks smooth-ish activations closely
-    mk = lambda: ADKVConfig(zp_init=torch.zeros(n), scale_init=torch.full((n,), 0.05),
-                            alpha=torch.full((n,), 0.95), beta=torch.full((n,), 0.05),
-                            quant_target=torch.full((n,), 3.5))
-    model.load_adkv_config([(mk(), mk()) for _ in range(2)])
-    ids = torch.randint(0, 128, (2, 12), generator=torch.Generator().manual_seed(3)).to(gpu)
+    H, D = kv_heads, 128
+    raw = _tiny_raw_calibration(2, H * D, seed=11)
+    calib.save_calibration(tmp_path, raw)
+    model.load_adkv_config(calib.load_calibration(tmp_path, 2, hidden_size=H * D))
+    params16 = _deployment_params16(raw, H, D)
+    for L, layer in enumerate(model.model.layers):          # the buffers hold exactly those fp16 values
+        for side, pn in zip(("key", "value"), params16[L]):
+            for name, a in zip(("zp_init", "scale_init", "alpha", "beta", "quant_target"), pn):
+                assert np.array_equal(_np16(getattr(layer.self_attn, f"{side}_{name}")).view(np.uint16),
+                                      a.reshape(-1).view(np.uint16)), (L, side, name)
+
+    P, new = 12, 8
+    pad = [0, 3]                                             # the second prompt is 3 tokens shorter
+    ids = torch.randint(1, 128, (2, P), generator=torch.Generator().manual_seed(3))
+    amask = torch.ones(2, P, dtype=torch.long)
+    for b, n in enumerate(pad):
+        ids[b, :n] = 0
+        amask[b, :n] = 0
+    ids, amask = ids.to(gpu), amask.to(gpu)
+    tap = _AttentionTap(model)
     with torch.no_grad():
-        out = model.generate(ids, max_new_tokens=8, do_sample=False)
-        ref = dense.generate(ids, max_new_tokens=8, do_sample=False)
-    assert out.shape == (2, 20)
-    assert torch.equal(out[:, :12], ids)
-    # the first generated token comes from the dense prefill path: identical by construction
-    assert torch.equal(out[:, 12], ref[:, 12])
+        out = model.generate(ids, attention_mask=amask, max_new_tokens=new, do_sample=False, pad_token_id=0)
+        tap.close()
+        ref = dense.generate(ids, attention_mask=amask, max_new_tokens=new, do_sample=False, pad_token_id=0)
+    assert out.shape == (2, P + new) and torch.equal(out[:, :P], ids)
+    caches, T, worst, n_decode = _check_decode_calls_against_oracle(oracle, model, tap.calls, params16, pad, P)
+    assert n_decode == 2 * (new - 1) and all(t == P + new - 1 for t in T.values())
+    cache = tap.cache                                      # the cache generate() worked on
+    assert cache is not None and cache.get_seq_length() == P + new - 1
+    n = oracle.n_super(P + new - 1)
+    for L in range(2):
+        assert np.array_equal(cache[L].key_states.cpu().numpy()[:, :, :n], caches[L][0][:, :, :n]), L
+        assert np.array_equal(cache[L].value_states.cpu().numpy()[:, :, :n], caches[L][1][:, :, :n]), L
+    assert torch.equal(out, ref), (out[:, P:].tolist(), ref[:, P:].tolist(), worst)
 
 
 @pytest.mark.gpu
