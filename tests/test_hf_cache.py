@@ -229,6 +229,73 @@ def _check_decode_calls_against_oracle(oracle, model, calls, params16, pad, prom
     return caches, T, worst, n_decode
 
 
+def _reference_greedy(oracle, dense, params16, ids, amask, pad, new):
+    """Greedy decoding of the tiny Llama written out layer by layer from the dense model's weights
+    (fp32): the prompt with ordinary causal attention, every later token with the oracle's quantised
+    decode attention over its own caches.  Shares no code with the ADKV modules or the cache object.
+    Returns (tokens [B, new], logits of each step [new][B, V])."""
+    cfg = dense.config
+    Hq, H, D = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    G, scaling = Hq // H, D ** -0.5
+    m = dense.model
+    B, P = ids.shape
+    dev = ids.device
+    pos = (amask.long().cumsum(-1) - 1).masked_fill(amask == 0, 1)        # positions skip the padding
+    caches = [None] * len(m.layers)
+    toks, step_logits = [], []
+    cur, cur_pos, t = ids, pos, P
+    for step in range(new):
+        h = m.embed_tokens(cur)
+        cos, sin = m.rotary_emb(h, cur_pos)
+        Tq = cur.shape[1]
+        for L, layer in enumerate(m.layers):
+            att = layer.self_attn
+            x = layer.input_layernorm(h)
+            split = lambda y, n: y.view(B, Tq, n, D).transpose(1, 2)
+            q = _rope(split(att.q_proj(x), Hq), cos, sin)
+            k = _rope(split(att.k_proj(x), H), cos, sin)
+            v = split(att.v_proj(x), H)
+            kpn, vpn = params16[L]
+            if step == 0:
+                ko, vo = oracle.alloc_cache(B, H, 256, D), oracle.alloc_cache(B, H, 256, D)
+                oracle.encode_kv_f16(ko, _np16(k.half()), *kpn)
+                oracle.encode_kv_f16(vo, _np16(v.half()), *vpn)
+                caches[L] = (ko, vo)
+                kr, vr = k.repeat_interleave(G, dim=1), v.repeat_interleave(G, dim=1)
+                sc = torch.matmul(q, kr.transpose(2, 3)) * scaling
+                allow = torch.tril(torch.ones(P, P, dtype=torch.bool, device=dev))[None, None] \
+                    & (amask[:, None, None, :] != 0)
+                sc = sc.masked_fill(~allow, float("-inf"))
+                # a padded query row sees nothing; its output is never used, keep it finite
+                sc = torch.where(allow.any(-1, keepdim=True), sc, torch.zeros_like(sc))
+                ctx = torch.matmul(torch.softmax(sc, dim=-1), vr)
+            else:
+                mask = np.zeros((B, 1, t + 1), np.float32)
+                for b in range(B):
+                    mask[b, 0, :pad[b]] = -np.inf
+                ko, vo = caches[L]
+                qn = _np16(q.half()).reshape(B, H, G, D)
+                out = np.zeros((B, H, G, D))
+                for j in range(G):
+                    kc, vc = ko.copy(), vo.copy()
+                    o, _, _ = oracle.decode_step_f16(qn[:, :, j], kc, vc, _np16(k.half()), _np16(v.half()),
+                                                     kpn, vpn, t, scaling, mask=mask)
+                    out[:, :, j] = o
+                caches[L] = (kc, vc)
+                ctx = torch.from_numpy(out.reshape(B, Hq, 1, D)).float().to(dev)
+            h = h + att.o_proj(ctx.transpose(1, 2).reshape(B, Tq, Hq * D))
+            h = h + layer.mlp(layer.post_attention_layernorm(h))
+        logits = dense.lm_head(m.norm(h))[:, -1]
+        step_logits.append(logits)
+        nxt = logits.argmax(-1)
+        toks.append(nxt)
+        if step > 0:
+            t += 1
+        cur = nxt[:, None]
+        cur_pos = cur_pos[:, -1:] + 1
+    return torch.stack(toks, dim=1), step_logits
+
+
 def _tiny_raw_calibration(layers, n, seed):
     """Raw (unconstrained) calibration parameters as the reference's trainer stores them."""
     g = torch.Generator().manual_seed(seed)
@@ -263,8 +330,11 @@ def test_tiny_llama_decode_path_matches_oracle_and_dense_model(gpu, oracle, tmp_
     ADKV cache with parameters read from calibration files (ckpt_{k,v}_{L}.pt -> load_calibration
     -> load_adkv_config, the route of tools/perf_e2e.py:37-60).  Every decode-path call of every
     attention module is recomputed with the oracle (see _check_decode_calls_against_oracle); the
-    packed caches at the end are the oracle's byte for byte; and the generated tokens are the
-    dense fp32 model's (the parameters quantise finely enough that the greedy choice survives)."""
+    packed caches at the end are the oracle's byte for byte; and all generated tokens and the
+    logits behind them equal those of a greedy loop written out in the test from the dense
+    model's weights with the oracle as its decode attention (_reference_greedy).  The first
+    token, which comes from the dense prompt pass, is also the dense model's; later ones need not
+    be: 4-bit K/V codes perturb a random-init model's near-flat logits enough to change an argmax."""
     pytest.importorskip("transformers")
     from transformers import LlamaForCausalLM
     from adkv_amd import calib
@@ -296,9 +366,12 @@ def test_tiny_llama_decode_path_matches_oracle_and_dense_model(gpu, oracle, tmp_
     ids, amask = ids.to(gpu), amask.to(gpu)
     tap = _AttentionTap(model)
     with torch.no_grad():
-        out = model.generate(ids, attention_mask=amask, max_new_tokens=new, do_sample=False, pad_token_id=0)
+        gen = model.generate(ids, attention_mask=amask, max_new_tokens=new, do_sample=False, pad_token_id=0,
+                             output_logits=True, return_dict_in_generate=True)
+        out = gen.sequences
         tap.close()
         ref = dense.generate(ids, attention_mask=amask, max_new_tokens=new, do_sample=False, pad_token_id=0)
+        want_toks, want_logits = _reference_greedy(oracle, dense, params16, ids, amask, pad, new)
     assert out.shape == (2, P + new) and torch.equal(out[:, :P], ids)
     caches, T, worst, n_decode = _check_decode_calls_against_oracle(oracle, model, tap.calls, params16, pad, P)
     assert n_decode == 2 * (new - 1) and all(t == P + new - 1 for t in T.values())
@@ -308,7 +381,14 @@ def test_tiny_llama_decode_path_matches_oracle_and_dense_model(gpu, oracle, tmp_
     for L in range(2):
         assert np.array_equal(cache[L].key_states.cpu().numpy()[:, :, :n], caches[L][0][:, :, :n]), L
         assert np.array_equal(cache[L].value_states.cpu().numpy()[:, :, :n], caches[L][1][:, :, :n]), L
-    assert torch.equal(out, ref), (out[:, P:].tolist(), ref[:, P:].tolist(), worst)
+    assert torch.equal(out[:, P], ref[:, P])               # the dense prompt pass decides the first token
+    assert torch.equal(out[:, P:], want_toks), (out[:, P:].tolist(), want_toks.tolist())
+    # Across layers the two runs drift a little apart: a context vector that differs in its last
+    # bits can move a K/V value of the next layer across a rounding boundary of the quantiser, so
+    # whole-model logits get a looser bound than the 2e-3 each layer meets on its own inputs.
+    for i, (got, want) in enumerate(zip(gen.logits, want_logits)):
+        err = float((got.float() - want.float()).abs().max())
+        assert err <= 2e-2, (i, err)
 
 
 @pytest.mark.gpu
