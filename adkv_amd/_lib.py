@@ -13,7 +13,7 @@ import torch  # noqa: F401  (loads libamdhip64 first)
 
 _DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_DIR, "libadkv_hip.so")
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 _vp, _i, _f = C.c_void_p, C.c_int, C.c_float
 
@@ -39,6 +39,9 @@ PROTOTYPES = {
     "adkv_forward_qk_gqa": (_i, [_vp] * 9 + [_i] * 7 + [C.c_int64, _vp, _vp, _i, _i, _vp]),
     "adkv_forward_ov_gqa_workspace_bytes": (C.c_int64, [_i] * 7),
     "adkv_forward_ov_gqa": (_i, [_vp] * 9 + [_i] * 7 + [C.c_int64, _vp, _vp, _i, _i, _vp, C.c_int64, _vp]),
+    "adkv_init": (_i, []),
+    "adkv_static_scratch_bytes": (C.c_int64, []),
+    "adkv_forward_ov_noalloc": (_i, [_vp] * 9 + [_i] * 7 + [C.c_int64, _vp, _vp, _i, _i, _vp]),
     "adkv_decode_fused_workspace_bytes": (C.c_int64, [_i] * 7),
     "adkv_decode_fused": (_i, [_vp] * 8 + [_i, _f, _vp, _vp, C.c_int64] + [_i] * 8 + [_vp, _vp, _i, _i, _vp,
                                                                             C.c_int64, _vp]),

@@ -1458,7 +1458,7 @@ static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval, int b
 
 extern "C" {
 
-int adkv_abi_version(void) { return 10; }
+int adkv_abi_version(void) { return 11; }
 
 void adkv_set_mha_kernel(int use_matrix_cores)
 {
@@ -1478,6 +1478,9 @@ const char *adkv_strerror(int code)
     case ADKV_E_ALIGN: return "pointer not sufficiently aligned";
     case ADKV_E_UNSUPPORTED: return "unsupported configuration";
     case ADKV_E_WORKSPACE: return "workspace too small";
+    case ADKV_E_SCRATCH_LIMIT:
+        return "launch needs more scratch than the library's static buffer holds (adkv_static_scratch_bytes)";
+    case ADKV_E_DEVICE: return "HIP device query failed";
     case ADKV_E_LAUNCH: return "HIP launch failed";
     default: return "unknown error";
     }
@@ -1824,7 +1827,84 @@ static int forward_ov_impl(const void *attn, void *v_cache, const void *v_new, v
     return rc;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Static scratch for callers that cannot allocate (code under HIP graph capture, serving loops,
+// harnesses that forbid hipMalloc): the fp32 partial sums of a segmented forward_ov live in a
+// device array that is part of the code object, one copy per GPU, held until the process ends.
+// In host code the array's name is only a handle for hipGetSymbolAddress; the device address it
+// yields (a different one on every GPU) is what launches are given.
+// ---------------------------------------------------------------------------------------------
+constexpr int64_t STATIC_SCRATCH_FLOATS = (int64_t)8 << 20; // 32 MiB
+static __device__ __align__(256) float scratch[STATIC_SCRATCH_FLOATS];
+
+constexpr int MAX_DEVICES = 64;
+static std::atomic<float *> g_scratch_ptr[MAX_DEVICES];
+static std::mutex g_scratch_mu;
+
+// Device address of `scratch` on the current device, resolved once per device.
+static int static_scratch(float **out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        g_last_hip_error = (int)e;
+        return ADKV_E_DEVICE;
+    }
+    if (dev < 0 || dev >= MAX_DEVICES)
+        return ADKV_E_UNSUPPORTED;
+    float *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        std::lock_guard<std::mutex> lock(g_scratch_mu);
+        p = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+        if (p == nullptr) {
+            void *addr = nullptr;
+            e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || addr == nullptr) {
+                g_last_hip_error = (int)e;
+                return ADKV_E_DEVICE;
+            }
+            p = (float *)addr;
+            g_scratch_ptr[dev].store(p, std::memory_order_release);
+        }
+    }
+    *out = p;
+    return ADKV_OK;
+}
+
 extern "C" {
+
+int64_t adkv_static_scratch_bytes(void) { return STATIC_SCRATCH_FLOATS * 4; }
+
+int adkv_init(void)
+{
+    float *p = nullptr;
+    return static_scratch(&p);
+}
+
+int adkv_forward_ov_noalloc(const void *attn, void *v_cache, const void *v_new, void *out,
+                            const void *zp, const void *sc, const void *alpha, const void *beta,
+                            const void *tgt,
+                            int B, int Hq, int H, int T, int D, int n_super_cap, int bits, int64_t ld,
+                            void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
+                            void *stream)
+{
+    // what the segment plan of this launch needs, priced before anything touches the device
+    int64_t need = 0;
+    if (ckpt != nullptr && B > 0 && H > 0 && Hq > 0 && Hq % H == 0 && T >= 0 && n_ckpt_cap > 0 &&
+        ckpt_interval > 0)
+        need = adkv_forward_ov_gqa_workspace_bytes(B, Hq, H, T, D, n_ckpt_cap, ckpt_interval);
+    if (need > adkv_static_scratch_bytes())
+        return ADKV_E_SCRATCH_LIMIT;
+    float *ws = nullptr;
+    const int rc = static_scratch(&ws);
+    if (rc)
+        return rc;
+    // Every partial a launch reads was written by the same launch (each segment stores its whole
+    // [B*Hq, D] slice before the summing kernel runs), so nothing has to start at zero.
+    return forward_ov_impl(attn, v_cache, v_new, out, zp, sc, alpha, beta, tgt, B, Hq, H, T, D,
+                           n_super_cap, bits, ld, state_out, ckpt, n_ckpt_cap, ckpt_interval, ws,
+                           adkv_static_scratch_bytes(), stream, 0);
+}
 
 int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void *out,
                         const void *zp, const void *sc, const void *alpha, const void *beta,

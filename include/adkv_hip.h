@@ -28,6 +28,8 @@ extern "C" {
 #define ADKV_E_ALIGN (-5)      /* pointer alignment requirement violated */
 #define ADKV_E_UNSUPPORTED (-6)
 #define ADKV_E_WORKSPACE (-7)  /* workspace missing or too small */
+#define ADKV_E_SCRATCH_LIMIT (-8) /* adkv_forward_ov_noalloc: needs more than adkv_static_scratch_bytes() */
+#define ADKV_E_DEVICE (-9)     /* a HIP device query failed; see adkv_last_hip_error() */
 #define ADKV_E_LAUNCH (-100)   /* HIP reported a launch error; see adkv_last_hip_error() */
 
 /* ABI version of this header; bumped on any signature change. */
@@ -212,6 +214,32 @@ int adkv_forward_ov_gqa(const void *attn, void *v_cache, const void *v_new, void
                         int B, int Hq, int H, int T, int D, int n_super_cap, int bits, int64_t ld,
                         void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
                         void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
+ * adkv_forward_ov_gqa for callers that cannot allocate device memory and have no workspace to
+ * hand over: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * No counterpart in the reference (its binding allocates its output with torch::zeros on every
+ * call, src/adkv/kernel/gemv.cu:1272).  Same arguments and results as adkv_forward_ov_gqa without
+ * `workspace`: the fp32 partial sums of a segmented launch go to a 32 MiB device array that is
+ * part of the library (one copy per GPU, held until the process ends).  The call itself never
+ * allocates or frees.  A launch whose segment plan needs more than adkv_static_scratch_bytes()
+ * (= adkv_forward_ov_gqa_workspace_bytes(...) of the same sizes) is rejected with
+ * ADKV_E_SCRATCH_LIMIT before anything is launched.  All calls on one GPU share that GPU's array:
+ * calls that overlap in time on one GPU (different streams, different threads) race on it; calls
+ * on one stream are safe.  The array needs no clearing between calls (every partial read was
+ * written by the same launch).
+ * adkv_init() resolves the array's address on the CURRENT device; call it once per device at
+ * set-up (outside any graph capture).  adkv_forward_ov_noalloc does the same on its first call on
+ * a device if adkv_init() was not called there.
+ */
+int adkv_init(void);
+int64_t adkv_static_scratch_bytes(void);
+int adkv_forward_ov_noalloc(const void *attn, void *v_cache, const void *v_new, void *out,
+                            const void *zp, const void *sc, const void *alpha, const void *beta,
+                            const void *tgt,
+                            int B, int Hq, int H, int T, int D, int n_super_cap, int bits, int64_t ld,
+                            void *state_out, void *ckpt, int n_ckpt_cap, int ckpt_interval,
+                            void *stream);
 
 /*
  * One decode-attention step of one layer in a single call: forward_qk -> scale/mask/softmax ->
