@@ -1,0 +1,444 @@
+// Vector decode kernels with a PER-HEAD lookup table (head dim 128, 4-bit codes, one query head
+// per KV head, big launches).  Included by adkv_kernels.hip after the shared device helpers.
+//
+// The replay is bound by vector-instruction issue, so every instruction per (channel pair, token)
+// counts.  The scale multiplier f = r16(beta*|q| + omt) (gemv.cu:163) depends only on the code and
+// on two per-channel constants, never on the state: it can come out of a table.  The shared table
+// of qk_kernel / ov_kernel returns (q, |q|) for a code byte and leaves the fused multiply-add to
+// the lane; here the table is built per KV head and returns (q, f) for (code byte, channel pair),
+// which removes one of the six packed instructions per pair and token.
+//
+//   * 256 code bytes x 64 channel pairs x 8 bytes = 128 KB of the CU's 160 KB of LDS, as two
+//     64 KB tables (first / second pair of a lane); entry (b, lane) sits at b*256 + lane*8, so the
+//     32 lanes of a head read 32 distinct 8-byte slots of one 256-byte row whatever their codes
+//     are, and the address is still ONE v_perm_b32: [0, table, code byte, lane*8].
+//   * All 32 (sequence, segment) units of a workgroup must belong to the SAME head: units are
+//     ordered head-major (for one head: segment-major, then sequence pairs), and every head's run
+//     of waves is padded to whole 16-wave workgroups.
+//   * No LDS is left for the logit transpose of qk_kernel, and none is needed: the 8 per-lane
+//     partials are reduced and scattered over the head's 32 lanes with bank-masked DPP adds
+//     (8 + 4 instructions), one row swap and two quad permutes.
+#pragma once
+
+namespace adkv {
+
+constexpr int FT_BLK = 1024;
+constexpr int FT_WAVES = FT_BLK / 64;
+constexpr int FT_TABLE_WORDS64 = 2 * LUT_ENTRIES * 32; // uint2 elements: 2 x 64 KB
+
+// host and device: how the (head, segment, sequence) units of a launch are laid out
+__host__ __device__ inline int ft_pairs_per_seg(int B) { return (B + 1) >> 1; }
+__host__ __device__ inline int ft_wgs_per_head(int B, int nseg)
+{
+    return (nseg * ft_pairs_per_seg(B) + FT_WAVES - 1) / FT_WAVES;
+}
+
+struct FtUnit {
+    int h, seg, bx, lh, c0;
+    bool active, wave_active;
+    __device__ __forceinline__ FtUnit(int B, int H, int nseg)
+    {
+        const int pps = ft_pairs_per_seg(B);
+        const int wph = ft_wgs_per_head(B, nseg);
+        h = (int)blockIdx.x / wph;
+        const int w = ((int)blockIdx.x % wph) * FT_WAVES + (int)(threadIdx.x >> 6); // wave within the head
+        const int sg = __builtin_amdgcn_readfirstlane(w / pps);
+        const int lane = threadIdx.x & 63;
+        const int b = (w % pps) * 2 + (lane >> 5);
+        lh = lane & 31;
+        c0 = lh * 4;
+        wave_active = sg < nseg;
+        active = wave_active && b < B;
+        seg = sg < nseg ? sg : nseg - 1;
+        bx = (b < B ? b : B - 1) * H + h;
+    }
+};
+
+// table[j][code byte][lane] = (q pair, f pair) for channels 4*lane + 2j, 4*lane + 2j + 1 of head h
+__device__ __forceinline__ void ft_fill(uint2 *tab, const h1 *be, const h1 *tg, int h)
+{
+    const int tid = threadIdx.x;
+    const int lh = tid & 31, j = (tid >> 5) & 1, cg = tid >> 6; // cg: 16 code bytes each
+    const int pi = h * 128 + 4 * lh + 2 * j;
+    const h2 b2 = *reinterpret_cast<const h2 *>(be + pi);
+    const h2 t2 = *reinterpret_cast<const h2 *>(tg + pi);
+    const h2 bt = b2 * t2;
+    const h2 omt = splat((h1)1.0f) - bt; // gemv.cu:220-221
+#pragma unroll
+    for (int i = 0; i < LUT_ENTRIES / FT_WAVES; i++) {
+        const int code = cg * (LUT_ENTRIES / FT_WAVES) + i;
+        const h2 q = (h2){(h1)((code & 15) - 8), (h1)((code >> 4) - 8)};
+        const h2 f = pk_fma(b2, pk_abs(q), omt); // gemv.cu:163, first half
+        tab[j * (LUT_ENTRIES * 32) + code * 32 + lh] = make_uint2(as_u32(q), as_u32(f));
+    }
+}
+
+// lane_copy = (1 << 8) | (lane % 32) * 8.  Entry of byte k (0..3) of `bytes` in table j (0 / 1);
+// k and j must be compile-time constants after unrolling (the selector becomes a literal).
+__device__ __forceinline__ uint2 ft_get(const uint2 *tab, uint32_t bytes, uint32_t lane_copy, int k, int j)
+{
+    // [0, j, bytes.byte[k], lane*8]: selector bytes 0-3 pick from lane_copy, 4-7 from bytes, 0x0C is zero
+    const uint32_t sel = (j ? 0x0C010000u : 0x0C0C0000u) | ((4u + (uint32_t)k) << 8);
+    const uint32_t addr = __builtin_amdgcn_perm(bytes, lane_copy, sel);
+    return *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(tab) + addr);
+}
+
+// The main loop needs zp, sc and alpha only (the table holds what beta and the target give); the
+// handful of tokens after it (ragged tail, appended token) use the plain update and load them then.
+__device__ __forceinline__ void ft_init_pairs(Pair *st, const h1 *zp, const h1 *sc, const h1 *al, int h,
+                                              int bx, int c0, int seg, const Seg &sa)
+{
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+        const int pi = h * 128 + c0 + 2 * p;
+        st[p].zp = *reinterpret_cast<const h2 *>(zp + pi);
+        st[p].sc = *reinterpret_cast<const h2 *>(sc + pi);
+        st[p].al = *reinterpret_cast<const h2 *>(al + pi);
+    }
+    if (seg > 0) {
+        const int j = seg * (sa.seg_tokens / sa.ckpt_interval) - 1;
+        load_state<4>(sa.ckpt + (((size_t)bx * sa.n_ckpt_cap + j) * 128 + c0) * 2, st);
+    }
+}
+
+__device__ __forceinline__ void ft_load_beta(Pair *st, const h1 *be, const h1 *tg, int h, int c0)
+{
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+        const int pi = h * 128 + c0 + 2 * p;
+        st[p].be = *reinterpret_cast<const h2 *>(be + pi);
+        const h2 bt = st[p].be * *reinterpret_cast<const h2 *>(tg + pi);
+        st[p].omt = splat((h1)1.0f) - bt;
+    }
+}
+
+// State update with the tabulated multiplier: zp <- r16(alpha*qs + zp), sc <- r16(sc*f).
+__device__ __forceinline__ void update_pair_f(Pair &p, h2 f, h2 qs)
+{
+    p.zp = pk_fma(p.al, qs, p.zp);
+    p.sc = p.sc * f;
+}
+
+// Sum of 8 per-lane partials over the 32 lanes of a head, scattered: afterwards every lane holds
+// the total of ONE token, token_of_lane(lane), the same in the four lanes of a quad.
+//   bit 3 of the lane (banks 0,1 | 2,3): keep tokens 0-3 | 4-7, add the partner's    8 instructions
+//   bit 2 (banks 0,2 | 1,3):             keep tokens +0,+1 | +2,+3                      4
+//   bit 4 (row 0 | 1 of the head):       v_permlane16_swap + add, keep token +0 | +1    2
+//   bits 0,1: all-reduce inside the quad                                                2
+// A masked DPP add writes only the banks of its mask and keeps the other lanes' destination; a
+// DPP operand must not have been written by the two preceding instructions, which the order
+// below guarantees inside the block and the leading s_nop for whatever precedes it.
+__device__ __forceinline__ float reduce8_head32(const float *p)
+{
+    float r0, r1, r2, r3, s0, s1;
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_add_f32_dpp %0, %6, %6 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %1, %7, %7 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %2, %8, %8 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %3, %9, %9 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %0, %10, %10 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %1, %11, %11 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %2, %12, %12 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %3, %13, %13 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        // banks 0,2 take lane+4 (rotate right by 12), banks 1,3 take lane-4 (rotate right by 4)
+        "v_add_f32_dpp %4, %0, %0 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %5, %1, %1 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %4, %2, %2 row_ror:4 row_mask:0xf bank_mask:0xa\n\t"
+        "v_add_f32_dpp %5, %3, %3 row_ror:4 row_mask:0xf bank_mask:0xa\n\t"
+        "s_nop 1\n\t"
+        "v_permlane16_swap_b32 %4, %5\n\t"
+        "s_nop 1"
+        : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3), "=&v"(s0), "=&v"(s1)
+        : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]));
+    float t = s0 + s1;
+    t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0xB1 /*quad_perm:[1,0,3,2]*/,
+                                                               0xF, 0xF, true));
+    t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0x4E /*quad_perm:[2,3,0,1]*/,
+                                                               0xF, 0xF, true));
+    return t;
+}
+
+__device__ __forceinline__ int token_of_lane(int lane)
+{
+    const int bank = (lane >> 2) & 3, row = (lane >> 4) & 1;
+    return 4 * (bank >> 1) + 2 * (bank & 1) + row;
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward_qk  (gemv.cu:435-815), per-head table
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
+    const h1 *__restrict__ q, uint4 *__restrict__ cache, const h1 *__restrict__ k_new,
+    h1 *__restrict__ out,
+    const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
+    const h1 *__restrict__ be, const h1 *__restrict__ tg,
+    int B, int H, int T, int n_super_cap, h1 *__restrict__ state_out, Seg sa)
+{
+    constexpr int D = 128, CPL = 4;
+    using G = Geo<D, CPL>;
+    __shared__ uint2 tab[FT_TABLE_WORDS64]; // the only LDS object: sits at offset 0
+    const FtUnit un(B, H, sa.nseg);
+    ft_fill(tab, be, tg, un.h);
+    __syncthreads();
+    if (!un.wave_active)
+        return; // padding waves of the head's last workgroup
+
+    const int lane = threadIdx.x & 63;
+    const uint32_t lane_copy = 0x100u | ((uint32_t)un.lh * 8u);
+    const int bx = un.bx, lh = un.lh, c0 = un.c0, h = un.h;
+    const bool active = un.active;
+    const bool last = un.seg == sa.nseg - 1;
+
+    Pair st[G::NP];
+    h2 qv[G::NP];
+    ft_init_pairs(st, zp, sc, al, h, bx, c0, un.seg, sa);
+#pragma unroll
+    for (int p = 0; p < G::NP; p++)
+        qv[p] = load_act2(q + (size_t)bx * D + c0 + 2 * p, sa.act_bf16);
+
+    const int t0 = un.seg * sa.seg_tokens;
+    const int t1 = last ? T : t0 + sa.seg_tokens;
+    uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh;
+    const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;
+    h1 *ob = out + (size_t)bx * sa.row_pitch + t0;
+    const int nfull = (t1 - t0) >> 3;
+    const int tk = token_of_lane(lane);
+    const bool storer = active && (lane & 3) == 0;
+
+    auto finish = [&](const float *part, int sg, int ntok) {
+        const float s = reduce8_head32(part);
+        if (storer && tk < ntok)
+            ob[sg * 8 + tk] = (h1)s;
+    };
+
+    // one token of the current supergroup, then the lookups of the same slot of the next one
+    auto token = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2], float &out_t) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int p = 0; p < G::NP; p++) {
+            Pair &s = st[p];
+            const h2 qs = as_h2(e[p][t].x) * s.sc;
+            acc = __builtin_amdgcn_fdot2(qv[p], qs + s.zp, acc, false);
+            update_pair_f(s, as_h2(e[p][t].y), qs);
+        }
+        out_t = acc;
+#pragma unroll
+        for (int p = 0; p < G::NP; p++)
+            e[p][t] = ft_get(tab, nb[p][t & 1], lane_copy, t >> 1, p);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    uint4 buf[PF][1];
+    uint2 lk[G::NP][8];
+    uint32_t nb[G::NP][2];
+    float part[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < PF; i++)
+        buf[i][0] = (i < nfull) ? cb[(size_t)i * G::VPS] : make_uint4(0, 0, 0, 0);
+    if (nfull > 0) {
+        pair_bytes_of<D, CPL>(buf[0], nb);
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+#pragma unroll
+            for (int p = 0; p < G::NP; p++)
+                lk[p][t] = ft_get(tab, nb[p][t & 1], lane_copy, t >> 1, p);
+    }
+    // One supergroup; i = its buffer in the rotation.  Nothing conditional: the trip count is
+    // wave-uniform, the prefetch index is clamped, and the reduction of the previous supergroup
+    // (done here, between the lookups' issue and their first use) stores nothing for sg == 0.
+    auto body = [&](int sg, auto ic) {
+        constexpr int i = decltype(ic)::value;
+        pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
+        buf[i][0] = cb[(size_t)min(sg + PF, nfull - 1) * G::VPS];
+        __builtin_amdgcn_sched_barrier(0);
+        finish(part, sg - 1, sg > 0 ? 8 : 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+            token(t, lk, nb, part[t]);
+    };
+    rotate_over<PF>(nfull, body);
+    if (nfull > 0)
+        finish(part, nfull - 1, 8);
+    if (!last)
+        return;
+
+    // ragged tail: T % 8 tokens of the last supergroup (gemv.cu:648-654); plain arithmetic
+    ft_load_beta(st, be, tg, h, c0);
+    const int ntail = (t1 - t0) & 7;
+    if (ntail) {
+        float tp[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        uint32_t w[4];
+        vec_words(cb[(size_t)nfull * G::VPS], w);
+#pragma unroll
+        for (int pp = 0; pp < 2; pp++) {
+            Pair &s = st[pp];
+            for (int tt = 0; tt < ntail; tt++) {
+                const h2 qc = extract_pair<4>(w[2 * pp], w[2 * pp + 1], tt);
+                const h2 qs = qc * s.sc;
+                const float d = __builtin_amdgcn_fdot2(qv[pp], qs + s.zp, 0.0f, false);
+#pragma unroll
+                for (int k = 0; k < 8; k++)
+                    tp[k] += (k == tt) ? d : 0.0f;
+                update_pair(s, qc, qs);
+            }
+        }
+        finish(tp, nfull, ntail);
+    }
+
+    if (active)
+        publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
+
+    h2 deq[G::NP];
+    append_new_token<D, CPL>(cbh, T, k_new + (size_t)bx * D + c0, st, deq, active, sa.act_bf16);
+    float self = 0.0f;
+#pragma unroll
+    for (int p = 0; p < G::NP; p++)
+        self = __builtin_amdgcn_fdot2(qv[p], deq[p], self, false);
+    self = head_allreduce<G::LPH>(self);
+    if (active && lh == 0)
+        out[(size_t)bx * sa.row_pitch + T] = (h1)self;
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward_ov  (gemv.cu:946-1178), per-head table
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
+    const h1 *__restrict__ attn, uint4 *__restrict__ cache, const h1 *__restrict__ v_new,
+    h1 *__restrict__ out, float *__restrict__ partial,
+    const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
+    const h1 *__restrict__ be, const h1 *__restrict__ tg,
+    int B, int H, int T, int n_super_cap, h1 *__restrict__ state_out, Seg sa)
+{
+    constexpr int D = 128, CPL = 4;
+    using G = Geo<D, CPL>;
+    __shared__ uint2 tab[FT_TABLE_WORDS64];
+    const FtUnit un(B, H, sa.nseg);
+    ft_fill(tab, be, tg, un.h);
+    __syncthreads();
+    if (!un.wave_active)
+        return;
+
+    const uint32_t lane_copy = 0x100u | ((uint32_t)un.lh * 8u);
+    const int bx = un.bx, lh = un.lh, c0 = un.c0, h = un.h;
+    const bool active = un.active;
+    const bool last = un.seg == sa.nseg - 1;
+    const int BH = B * H;
+
+    Pair st[G::NP];
+    float acc[CPL];
+    ft_init_pairs(st, zp, sc, al, h, bx, c0, un.seg, sa);
+#pragma unroll
+    for (int c = 0; c < CPL; c++)
+        acc[c] = 0.0f;
+
+    const int t0 = un.seg * sa.seg_tokens;
+    const int t1 = last ? T : t0 + sa.seg_tokens;
+    uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh;
+    const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;
+    const h1 *wrow = attn + (size_t)bx * sa.row_pitch;
+    const h1 *wb = wrow + t0;
+    const int nfull = (t1 - t0) >> 3;
+
+    auto load_w = [&](int sg) {
+        uint4 r;
+        __builtin_memcpy(&r, wb + (size_t)sg * 8, 16); // row base is only 2-byte aligned
+        return r;
+    };
+    auto token = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2], const uint4 wv) {
+        const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+        const h2 wp = as_h2(ww[t >> 1]);
+        const float wt = (t & 1) ? (float)wp.y : (float)wp.x;
+#pragma unroll
+        for (int p = 0; p < G::NP; p++) {
+            Pair &s = st[p];
+            const h2 qs = as_h2(e[p][t].x) * s.sc;
+            const h2 vd = qs + s.zp;
+            acc[2 * p] = __builtin_fmaf(wt, (float)vd.x, acc[2 * p]);
+            acc[2 * p + 1] = __builtin_fmaf(wt, (float)vd.y, acc[2 * p + 1]);
+            update_pair_f(s, as_h2(e[p][t].y), qs);
+        }
+#pragma unroll
+        for (int p = 0; p < G::NP; p++)
+            e[p][t] = ft_get(tab, nb[p][t & 1], lane_copy, t >> 1, p);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    uint4 buf[PF][1];
+    uint4 wbuf[PF];
+    uint2 lk[G::NP][8];
+    uint32_t nb[G::NP][2];
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+        buf[i][0] = (i < nfull) ? cb[(size_t)i * G::VPS] : make_uint4(0, 0, 0, 0);
+        wbuf[i] = (i < nfull) ? load_w(i) : make_uint4(0, 0, 0, 0);
+    }
+    if (nfull > 0) {
+        pair_bytes_of<D, CPL>(buf[0], nb);
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+#pragma unroll
+            for (int p = 0; p < G::NP; p++)
+                lk[p][t] = ft_get(tab, nb[p][t & 1], lane_copy, t >> 1, p);
+    }
+    auto body = [&](int sg, auto ic) {
+        constexpr int i = decltype(ic)::value;
+        pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
+        const int sgp = min(sg + PF, nfull - 1);
+        buf[i][0] = cb[(size_t)sgp * G::VPS];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+            token(t, lk, nb, wbuf[i]);
+        wbuf[i] = load_w(sgp); // reloaded once its last token is done (see ov_kernel)
+    };
+    rotate_over<PF>(nfull, body);
+
+    if (last) {
+        ft_load_beta(st, be, tg, h, c0);
+        const int ntail = (t1 - t0) & 7;
+        if (ntail) {
+            uint32_t w[4];
+            vec_words(cb[(size_t)nfull * G::VPS], w);
+#pragma unroll
+            for (int pp = 0; pp < 2; pp++) {
+                Pair &s = st[pp];
+                for (int tt = 0; tt < ntail; tt++) {
+                    const h2 qc = extract_pair<4>(w[2 * pp], w[2 * pp + 1], tt);
+                    const h2 qs = qc * s.sc;
+                    const h2 vd = qs + s.zp;
+                    const float wt = (float)wb[nfull * 8 + tt];
+                    acc[2 * pp] = __builtin_fmaf(wt, (float)vd.x, acc[2 * pp]);
+                    acc[2 * pp + 1] = __builtin_fmaf(wt, (float)vd.y, acc[2 * pp + 1]);
+                    update_pair(s, qc, qs);
+                }
+            }
+        }
+        if (active)
+            publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
+        h2 deq[G::NP];
+        append_new_token<D, CPL>(cbh, T, v_new + (size_t)bx * D + c0, st, deq, active, sa.act_bf16);
+        const float wT = (float)wrow[T];
+#pragma unroll
+        for (int p = 0; p < G::NP; p++) {
+            acc[2 * p] = __builtin_fmaf(wT, (float)deq[p].x, acc[2 * p]);
+            acc[2 * p + 1] = __builtin_fmaf(wT, (float)deq[p].y, acc[2 * p + 1]);
+        }
+    }
+    if (!active)
+        return;
+    if (sa.nseg == 1) {
+        h1 *o = out + (size_t)bx * D + c0;
+#pragma unroll
+        for (int p = 0; p < G::NP; p++)
+            store_act2(o + 2 * p, acc[2 * p], acc[2 * p + 1], sa.act_bf16);
+    } else {
+        float2 *o = reinterpret_cast<float2 *>(partial + ((size_t)un.seg * BH + bx) * D + c0);
+#pragma unroll
+        for (int p = 0; p < G::NP; p++)
+            o[p] = make_float2(acc[2 * p], acc[2 * p + 1]);
+    }
+}
+
+} // namespace adkv

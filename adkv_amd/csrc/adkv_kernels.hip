@@ -1277,6 +1277,7 @@ static int check_common(int B, int H, int T, int D, int n_super_cap)
 static inline int lanes_per_head(int D) { return D == 128 ? 32 : 64; }
 
 #include "adkv_gqa_kernels.h"
+#include "adkv_ft_kernels.h"
 
 // Waves a SIMD should hold for packed-f16 issue to run near full rate, and SIMDs on the device.
 constexpr int WAVES_PER_SIMD_TARGET = 4;
@@ -1430,7 +1431,30 @@ static int mha_kernel_default()
 static bool mfma_for_mha()
 {
     const int v = g_mha_kernel.load(std::memory_order_relaxed);
-    return (v < 0 ? mha_kernel_default() : v) != 0;
+    return (v < 0 ? mha_kernel_default() : v) == 1;
+}
+
+// Whether a launch with one query head per KV head takes the kernels with a per-head table
+// (adkv_ft_kernels.h).  They need head dim 128 and 4-bit codes; by default they are taken where
+// the shared-table kernels would run 16-wave workgroups of four-channel lanes anyway and the
+// padding of every head's waves to whole workgroups wastes little.  adkv_set_mha_kernel(2) takes
+// them whenever they can run, (0) never.
+static bool use_head_table(int B, int H, int GQ, int bits, int D, const Seg &seg)
+{
+    if (D != 128 || bits != 4 || GQ != 1)
+        return false;
+    const int v = g_mha_kernel.load(std::memory_order_relaxed);
+    if (v == 2)
+        return true;
+    if (v >= 0 || mha_kernel_default() == 1)
+        return false;
+    const long BH = (long)B * H;
+    const long padded = padded_units<32>((int)BH, seg.nseg);
+    if (padded / 2 <= N_SIMD || padded * 32 < (long)FT_BLK * 256)
+        return false;                                 // small launches: two-channel lanes / 4-wave workgroups
+    const long waves = (long)seg.nseg * ft_pairs_per_seg(B);
+    const long padded_waves = (long)ft_wgs_per_head(B, seg.nseg) * FT_WAVES;
+    return padded_waves * 100 <= waves * 106;
 }
 
 // ADKV_ENCODE_CPL=1/2 pins the encoder's channels per lane (a measurement aid); read once.
@@ -1462,7 +1486,8 @@ int adkv_abi_version(void) { return 11; }
 
 void adkv_set_mha_kernel(int use_matrix_cores)
 {
-    g_mha_kernel.store(use_matrix_cores < 0 ? -1 : (use_matrix_cores != 0), std::memory_order_relaxed);
+    g_mha_kernel.store(use_matrix_cores < 0 ? -1 : (use_matrix_cores > 2 ? 1 : use_matrix_cores),
+                       std::memory_order_relaxed);
 }
 
 int adkv_last_hip_error(void) { return g_last_hip_error; }
@@ -1711,6 +1736,13 @@ static int forward_qk_impl(const void *q, void *k_cache, const void *k_new, void
                          seg);
         return check_launch();
     }
+    if (use_head_table(B, H, GQ, bits, D, seg)) {
+        hipLaunchKernelGGL(qk_ft_kernel, dim3((unsigned)(H * ft_wgs_per_head(B, seg.nseg))), dim3(FT_BLK), 0, st,
+                           (const h1 *)q, (uint4 *)k_cache, (const h1 *)k_new, (h1 *)logits,
+                           (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha, (const h1 *)beta,
+                           (const h1 *)tgt, B, H, T, n_super_cap, (h1 *)state_out, seg);
+        return check_launch();
+    }
     ADKV_DISPATCH_D(qk_kernel, (const h1 *)q, (uint4 *)k_cache, (const h1 *)k_new, (h1 *)logits,
                     (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha, (const h1 *)beta,
                     (const h1 *)tgt, BH, H, T, n_super_cap, (h1 *)state_out, seg);
@@ -1806,6 +1838,11 @@ static int forward_ov_impl(const void *attn, void *v_cache, const void *v_new, v
                          (h1 *)out, (float *)workspace, (const h1 *)zp, (const h1 *)sc,
                          (const h1 *)alpha, (const h1 *)beta, (const h1 *)tgt, BH, H, T, n_super_cap,
                          (h1 *)state_out, seg);
+    } else if (use_head_table(B, H, GQ, bits, D, seg)) {
+        hipLaunchKernelGGL(ov_ft_kernel, dim3((unsigned)(H * ft_wgs_per_head(B, seg.nseg))), dim3(FT_BLK), 0, st,
+                           (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new, (h1 *)out,
+                           (float *)workspace, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,
+                           (const h1 *)beta, (const h1 *)tgt, B, H, T, n_super_cap, (h1 *)state_out, seg);
     } else {
         ADKV_DISPATCH_D(ov_kernel, (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new, (h1 *)out,
                         (float *)workspace, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,
