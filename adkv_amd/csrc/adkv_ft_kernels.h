@@ -119,6 +119,18 @@ __device__ __forceinline__ void update_pair_f(Pair &p, h2 f, h2 qs)
     p.sc = p.sc * f;
 }
 
+// a.x*b.x + a.y*b.y in fp32, as the three-operand form with a literal zero accumulator: the
+// accumulating two-operand form the compiler picks needs its destination cleared first, one more
+// vector instruction per token.  The leading wait state covers an operand that the instruction
+// just before wrote as a packed 16-bit result (on this chip such a result cannot be forwarded to
+// the very next instruction; the compiler pads its own code the same way).
+__device__ __forceinline__ float dot2_from_zero(h2 a, h2 b)
+{
+    float d;
+    asm("s_nop 0\n\tv_dot2_f32_f16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b));
+    return d;
+}
+
 // Sum of 8 per-lane partials over the 32 lanes of a head, scattered: afterwards every lane holds
 // the total of ONE token, token_of_lane(lane), the same in the four lanes of a quad.
 //   bit 3 of the lane (banks 0,1 | 2,3): keep tokens 0-3 | 4-7, add the partner's    8 instructions
@@ -148,15 +160,16 @@ __device__ __forceinline__ float reduce8_head32(const float *p)
         "v_add_f32_dpp %5, %3, %3 row_ror:4 row_mask:0xf bank_mask:0xa\n\t"
         "s_nop 1\n\t"
         "v_permlane16_swap_b32 %4, %5\n\t"
-        "s_nop 1"
+        "s_nop 1\n\t"
+        "v_add_f32 %4, %4, %5\n\t"
+        "s_nop 1\n\t"
+        "v_add_f32_dpp %4, %4, %4 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_add_f32_dpp %4, %4, %4 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0"
         : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3), "=&v"(s0), "=&v"(s1)
         : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]));
-    float t = s0 + s1;
-    t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0xB1 /*quad_perm:[1,0,3,2]*/,
-                                                               0xF, 0xF, true));
-    t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0x4E /*quad_perm:[2,3,0,1]*/,
-                                                               0xF, 0xF, true));
-    return t;
+    return s0;
 }
 
 __device__ __forceinline__ int token_of_lane(int lane)
@@ -214,12 +227,16 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
 
     // one token of the current supergroup, then the lookups of the same slot of the next one
     auto token = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2], float &out_t) {
-        float acc = 0.0f;
+        float acc;
 #pragma unroll
         for (int p = 0; p < G::NP; p++) {
             Pair &s = st[p];
             const h2 qs = as_h2(e[p][t].x) * s.sc;
-            acc = __builtin_amdgcn_fdot2(qv[p], qs + s.zp, acc, false);
+            const h2 kh = qs + s.zp;
+            if (p == 0)
+                acc = dot2_from_zero(qv[p], kh);
+            else
+                acc = __builtin_amdgcn_fdot2(qv[p], kh, acc, false);
             update_pair_f(s, as_h2(e[p][t].y), qs);
         }
         out_t = acc;

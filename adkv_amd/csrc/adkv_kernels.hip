@@ -1482,7 +1482,7 @@ static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval, int b
 
 extern "C" {
 
-int adkv_abi_version(void) { return 11; }
+int adkv_abi_version(void) { return 12; }
 
 void adkv_set_mha_kernel(int use_matrix_cores)
 {
@@ -1695,6 +1695,35 @@ int adkv_encode_kv(void *cache, const void *kv_new,
 
 } // extern "C"
 
+// Which decode kernel family and shape a launch of these sizes takes (the dispatch below, as text).
+static const char *decode_kernel_name(int B, int Hq, int H, int T, int D, int bits, int n_ckpt_cap,
+                                      int ckpt_interval)
+{
+    if (B <= 0 || H <= 0 || Hq <= 0 || Hq % H || T < 0 || (D != 128 && D != 256 && D != 512) ||
+        (bits != 2 && bits != 4))
+        return "invalid";
+    const int GQ = Hq / H;
+    if ((GQ > 1 || bits != 4) && D != 128)
+        return "invalid";
+    int dummy = 0;
+    const Seg seg = plan_segments(n_ckpt_cap > 0 && ckpt_interval > 0 ? &dummy : nullptr, n_ckpt_cap,
+                                  ckpt_interval, B * H, T, D);
+    if (D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha())) {
+        const long threads = padded_units<32>(B * H, seg.nseg) * 32;
+        return threads >= 1024L * 256 ? "gqa_kernel, 16-wave workgroups (matrix cores)"
+                                      : "gqa_kernel, 8-wave workgroups (matrix cores)";
+    }
+    if (use_head_table(B, H, GQ, bits, D, seg))
+        return "ft_kernel (per-head table, 16-wave workgroups)";
+    if (D == 128) {
+        const long units = padded_units<32>(B * H, seg.nseg);
+        if (units / 2 <= N_SIMD)
+            return "kernel<128,2,256> (shared table, two channels per lane)";
+        return units * 32 >= 1024L * 256 ? "kernel<128,4,1024> (shared table)" : "kernel<128,4,256> (shared table)";
+    }
+    return D == 256 ? "kernel<256,4,*> (shared table)" : "kernel<512,8,256> (shared table)";
+}
+
 // act_bf16: q, k_new / v_new and the output are bfloat16 (only adkv_decode_fused asks for it)
 static int forward_qk_impl(const void *q, void *k_cache, const void *k_new, void *logits,
                            const void *zp, const void *sc, const void *alpha, const void *beta,
@@ -1750,6 +1779,12 @@ static int forward_qk_impl(const void *q, void *k_cache, const void *k_new, void
 }
 
 extern "C" {
+
+const char *adkv_decode_kernel_name(int B, int Hq, int H, int T, int D, int bits, int n_ckpt_cap,
+                                    int ckpt_interval)
+{
+    return decode_kernel_name(B, Hq, H, T, D, bits, n_ckpt_cap, ckpt_interval);
+}
 
 int adkv_forward_qk_gqa(const void *q, void *k_cache, const void *k_new, void *logits,
                         const void *zp, const void *sc, const void *alpha, const void *beta,
@@ -2005,7 +2040,8 @@ int adkv_softmax_ex(const void *logits, void *weights, const void *mask,
     if (ld == 0)
         ld = n;
     if (n <= 64 * SM_VEC * 4) {
-        // short rows: a wave per row, the row in 8, 16 or 32 registers per lane
+        // short rows: a wave per row, the row in 8, 16 or 32 registers per lane (longer rows were
+        // measured slower this way: 27 us against 22 us for 4096 rows of 4097 elements)
         const dim3 grid((unsigned)((rows + SM_BLOCK / 64 - 1) / (SM_BLOCK / 64)));
 #define ADKV_SM_WAVE(NVW)                                                                           \
     hipLaunchKernelGGL(softmax_wave_kernel<NVW>, grid, dim3(SM_BLOCK), 0, (hipStream_t)stream,      \
@@ -2052,6 +2088,27 @@ int adkv_softmax(const void *logits, void *weights, const void *mask,
 }
 
 static int64_t pad256(int64_t n) { return (n + 255) & ~(int64_t)255; }
+
+// Events adkv_decode_fused records around its stages in this thread (a measurement hook).
+static thread_local hipEvent_t g_stage_events[4] = {nullptr, nullptr, nullptr, nullptr};
+
+void adkv_set_stage_events(void *const *events)
+{
+    for (int i = 0; i < 4; i++)
+        g_stage_events[i] = events ? (hipEvent_t)events[i] : nullptr;
+}
+
+static int stage_mark(int i, void *stream)
+{
+    if (g_stage_events[i] == nullptr)
+        return ADKV_OK;
+    const hipError_t e = hipEventRecord(g_stage_events[i], (hipStream_t)stream);
+    if (e != hipSuccess) {
+        g_last_hip_error = (int)e;
+        return ADKV_E_LAUNCH;
+    }
+    return ADKV_OK;
+}
 
 int64_t adkv_forward_ov_gqa_workspace_bytes(int B, int Hq, int H, int T, int D, int n_ckpt_cap,
                                             int ckpt_interval)
@@ -2100,20 +2157,26 @@ int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k
     char *ws = (char *)workspace;
     void *logits = ws;
     void *weights = weights_out ? weights_out : (void *)(ws + mat);
-    int rc = forward_qk_impl(q, k_cache, k_new, logits, k_params[0], k_params[1], k_params[2],
-                             k_params[3], k_params[4], B, Hq, H, T, D, n_super_cap, bits, ld,
-                             nullptr, k_ckpt, n_ckpt_cap, ckpt_interval, stream, act_bf16);
+    int rc = stage_mark(0, stream);
     if (rc)
+        return rc;
+    rc = forward_qk_impl(q, k_cache, k_new, logits, k_params[0], k_params[1], k_params[2],
+                         k_params[3], k_params[4], B, Hq, H, T, D, n_super_cap, bits, ld,
+                         nullptr, k_ckpt, n_ckpt_cap, ckpt_interval, stream, act_bf16);
+    if (rc || (rc = stage_mark(1, stream)))
         return rc;
     const int64_t smb = pad256(adkv_softmax_workspace_bytes(B * Hq, T + 1));
     rc = adkv_softmax_ex(logits, weights, mask, B * Hq, T + 1, ld, rows_per_mask_row, scaling,
                          smb ? ws + 2 * mat : nullptr, smb, stream);
+    if (rc || (rc = stage_mark(2, stream)))
+        return rc;
+    rc = forward_ov_impl(weights, v_cache, v_new, out, v_params[0], v_params[1], v_params[2],
+                         v_params[3], v_params[4], B, Hq, H, T, D, n_super_cap, bits, ld,
+                         nullptr, v_ckpt, n_ckpt_cap, ckpt_interval, ws + 2 * mat + smb,
+                         workspace_bytes - 2 * mat - smb, stream, act_bf16);
     if (rc)
         return rc;
-    return forward_ov_impl(weights, v_cache, v_new, out, v_params[0], v_params[1], v_params[2],
-                           v_params[3], v_params[4], B, Hq, H, T, D, n_super_cap, bits, ld,
-                           nullptr, v_ckpt, n_ckpt_cap, ckpt_interval, ws + 2 * mat + smb,
-                           workspace_bytes - 2 * mat - smb, stream, act_bf16);
+    return stage_mark(3, stream);
 }
 
 } // extern "C"

@@ -3,7 +3,7 @@
 
 One "step" is one layer's decode-attention for a batch: forward_qk (+append) -> softmax ->
 forward_ov (+append) over a resident 4-bit K/V cache, the protocol of the reference's
-tools/perf_kernel.py:28-76.  Throughput follows its convention (perf_kernel.py:91-104):
+tools/perf_kernel.py:28-76, issued the way the cache object issues it: one adkv_decode_fused call.  Throughput follows its convention (perf_kernel.py:91-104):
 tokens/s = B / (32 layers * seconds per layer-step).  Caches are produced by running the encoder
 on seeded synthetic K/V (closed loop), and the timed steps rotate over several distinct layer
 buffers so no cache level can serve re-reads.
@@ -53,6 +53,8 @@ def parse():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 1 GiB device-to-device copies (a known-size kernel to scale "
                          "rocprofv3 FETCH_SIZE/WRITE_SIZE readings by)")
+    ap.add_argument("--graph", action="store_true",
+                    help="also replay the step from HIP graphs and report that time beside the headline")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fp16-comparator", action="store_true",
                     help="skip timing the fp16-KV decode kernel beside the ADKV step")
@@ -388,36 +390,36 @@ def main():
         torch.cuda.synchronize()
         del a, b
 
-    ev = lambda: torch.cuda.Event(enable_timing=True)
-    marks = []
+    from adkv_amd import _lib
+    L = _lib.lib()
+    ncap_arg = ncap if S else 0
+    kernel = L.adkv_decode_kernel_name(B, Hq, H, T, D, bits, ncap_arg, S).decode()
+    ws = torch.empty(gemv.decode_fused_workspace_bytes(B, Hq, H, T, D, ncap_arg, S), dtype=torch.uint8, device=dev)
 
-    def step(i, timed):
-        l = i % NL
-        if timed:
-            e = [ev() for _ in range(4)]
-            e[0].record()
-        logits = gemv.forward_qk(q, kcs[l], k_new, *kps[l], T, smin, smax, ckpt=kks[l], ckpt_interval=S,
-                                 bits=bits)
-        if timed:
-            e[1].record()
-        w = gemv.softmax_scale_mask(logits, scaling)
-        if timed:
-            e[2].record()
-        out = gemv.forward_ov(w, vcs[l], v_new, *vps[l], smin, smax, ckpt=vks[l], ckpt_interval=S,
-                              bits=bits)
-        if timed:
-            e[3].record()
-            marks.append(e)
-        return out
+    def fused(l):
+        # the product path: what KVCacheLayer_ADKV.decode calls, one library call per layer-step
+        return gemv.decode_fused(q, kcs[l], vcs[l], k_new, v_new, kps[l], vps[l], T, scaling,
+                                 k_ckpt=kks[l], v_ckpt=vks[l], ckpt_interval=S, bits=bits, workspace=ws)
+
+    # four events per timed step, recorded by the library around the stages of the fused call
+    marks = []
+    for _ in range(args.steps):
+        e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+        for x in e:
+            x.record()                     # creates the underlying hipEvent_t
+        marks.append(e)
+    arr4 = _lib.C.c_void_p * 4
 
     for i in range(args.warmup):
-        step(i, False)
+        fused(i % NL)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(i, True)
+        L.adkv_set_stage_events(arr4(*[x.cuda_event for x in marks[i]]))
+        fused(i % NL)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    L.adkv_set_stage_events(None)
 
     ms_step = wall * 1e3 / args.steps
     qk_ms = sum(e[0].elapsed_time(e[1]) for e in marks) / len(marks)
@@ -425,9 +427,41 @@ def main():
     ov_ms = sum(e[2].elapsed_time(e[3]) for e in marks) / len(marks)
     dev_ms = sorted(e[0].elapsed_time(e[3]) for e in marks)[len(marks) // 2]
 
+    # the same step replayed from HIP graphs (one per layer cache): no host work between launches
+    graph_ms = None
+    if args.graph:
+        graphs = []
+        side = torch.cuda.Stream()
+        for l in range(NL):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                fused(l)
+                torch.cuda.synchronize()
+                with torch.cuda.graph(g, stream=side):
+                    fused(l)
+            graphs.append(g)
+        torch.cuda.synchronize()
+        for i in range(args.warmup):
+            graphs[i % NL].replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            graphs[i % NL].replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
     code_bytes = B * H * T * D * bits / 8.0             # one tensor's codes: bytes per QK launch
     achieved = code_bytes / (qk_ms * 1e-3) / 1e9
     tokens_s = B / (N_LAYERS_MODEL * ms_step * 1e-3)
+    workload_key = f"decode B={B} Hq={Hq} H={H} d={D} ctx={T} bits={bits} ckpt={S}"
+    traffic = None
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            rec = json.load(f).get(workload_key)
+        if rec and rec.get("kernel") == "qk_" + kernel.split(" ")[0]:
+            traffic = rec["bytes_per_launch"]
+    except (OSError, ValueError):
+        pass
 
     res = {
         "metric": "decode-attention tokens/sec (B / (32 layers * layer-step time))",
@@ -445,8 +479,8 @@ def main():
         "config": {
             "workload": f"{'cfg2 Llama-2-7B-shaped' if H == Hq else 'grouped-query'} ADKV decode attention: "
                         f"B={B} H={Hq}{'' if H == Hq else f' (KV heads {H})'} d={D} ctx={T} "
-                        f"{bits}-bit K+V codes, step = forward_qk+softmax+forward_ov, {NL} rotating layer caches, "
-                        f"state checkpoints every {S} tokens",
+                        f"{bits}-bit K+V codes, step = one decode_fused call (forward_qk+softmax+forward_ov, "
+                        f"appending the new token), {NL} rotating layer caches, state checkpoints every {S} tokens",
             "batch": B, "heads": Hq, "kv_heads": H, "head_dim": D, "ctx": T, "bits": bits, "ckpt_interval": S,
             "parallelism": "1 GPU",
         },
@@ -454,19 +488,36 @@ def main():
                       "step_device_median": dev_ms},
         "step_code_GBps": 2 * code_bytes / (ms_step * 1e-3) / 1e9,
         "roofline": {
-            "kernel": "qk_kernel" if (H == Hq and bits == 4) else "qk_gqa_kernel",
+            "kernel": "qk_" + kernel,
             "bound": "hbm",
             "achieved": achieved,
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            # HBM bytes per QK launch from rocprofv3 FETCH_SIZE/WRITE_SIZE scaled by a 1 GiB copy
-            # (profiles/decode_cfg2_pmc_traffic.md); measured for the default workload only
-            # (profiles/encode_cfg3_and_decode_cfg5_pmc_traffic.md for the grouped-query 2-bit shape)
-            "traffic": {(128, 32, 32, 128, 4096, 256, 4): 1.1227e9,
-                        (16, 32, 8, 128, 131072, 256, 2): 0.6911e9}.get((B, Hq, H, D, T, S, bits)),
+            # HBM bytes per QK launch from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a copy of
+            # known size; kept beside the profile it came from (profiles/hbm_traffic.json)
+            "traffic": traffic,
         },
     }
+    if graph_ms is not None:
+        res["graph_replay"] = {"ms_per_step": graph_ms, "tokens_per_s": B / (N_LAYERS_MODEL * graph_ms * 1e-3),
+                               "note": "the same decode_fused step captured once per layer cache and replayed"}
+    # The binding roof of this kernel is vector-instruction issue, not HBM: vector instructions
+    # per launch (profiles/valu_issue.json, from rocprofv3 SQ_INSTS_VALU) x 4 cycles per wave64
+    # instruction / (1024 SIMDs x the kernel's duration) at the shader clock seen under load.
+    try:
+        with open(os.path.join(ROOT, "profiles", "valu_issue.json")) as f:
+            vrec = json.load(f).get(workload_key)
+        if vrec and vrec.get("kernel") == "qk_" + kernel.split(" ")[0]:
+            cycles = qk_ms * 1e-3 * vrec["shader_clock_hz"]
+            busy = vrec["valu_insts_per_launch"] * 4.0 / 1024.0
+            res["roofline_valu"] = {"kernel": "qk_" + kernel, "bound": "valu",
+                                    "achieved": vrec["valu_insts_per_launch"] / (qk_ms * 1e-3) / 1e12,
+                                    "peak": 1024 * vrec["shader_clock_hz"] / 4.0 / 1e12,
+                                    "unit": "T wave64 instructions/s", "frac": busy / cycles,
+                                    "note": "SQ_INSTS_VALU per launch from profiles/valu_issue.json; duration live"}
+    except (OSError, ValueError):
+        pass
     if not args.no_fp16_comparator and D == 128 and H == Hq and bits == 4:
         res["fp16_kv_comparator"] = fp16_comparator(args, dev, ms_step)
     if not args.no_cpu_baseline and H == Hq and bits == 4:

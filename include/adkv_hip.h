@@ -36,9 +36,12 @@ extern "C" {
 int adkv_abi_version(void);
 
 /* Tuning knob, no counterpart in the reference: which decode kernels a launch with as many query
- * heads as KV heads and head dim 128 uses: 1 = the matrix-core kernels (the ones grouped-query
- * launches always use), 0 = the vector kernels, -1 = the library's default (ADKV_MFMA in the
- * environment overrides it).  Results agree to the tolerance of the fp32 accumulation order. */
+ * heads as KV heads and head dim 128 uses: 0 = the vector kernels with the shared code table,
+ * 1 = the matrix-core kernels (the ones grouped-query launches always use), 2 = the vector
+ * kernels with a per-head table wherever they can run (4-bit codes), -1 = the library's choice
+ * (the per-head table for big launches, else the shared one; ADKV_MFMA=1 in the environment,
+ * read once, makes it the matrix-core kernels).  Results agree to the tolerance of the fp32
+ * accumulation order; appended codes, state and checkpoints are identical. */
 void adkv_set_mha_kernel(int use_matrix_cores);
 const char *adkv_strerror(int code);
 /* hipError_t (as int) of the last failed launch in this thread, 0 if none. */
@@ -265,6 +268,22 @@ int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k
                       int B, int Hq, int H, int T, int D, int n_super_cap, int bits, int act_dtype,
                       void *k_ckpt, void *v_ckpt, int n_ckpt_cap, int ckpt_interval,
                       void *workspace, int64_t workspace_bytes, void *stream);
+
+/* Which of the library's decode kernels adkv_forward_qk_gqa / adkv_forward_ov_gqa /
+ * adkv_decode_fused launch for these sizes ("qk_" / "ov_" + the returned text): a static string,
+ * for benchmark records and tests; "invalid" for sizes the entry points reject. */
+const char *adkv_decode_kernel_name(int B, int Hq, int H, int T, int D, int bits, int n_ckpt_cap,
+                                    int ckpt_interval);
+
+/*
+ * Measurement hook, no counterpart in the reference (its benchmark times whole steps with CUDA
+ * events, tools/perf_kernel.py:65-74): `events` is a host array of four hipEvent_t created with
+ * timing enabled, or NULL to switch the hook off.  While set, every adkv_decode_fused call of
+ * THIS host thread records them on its stream: [0] before the QK launch, [1] after it, [2] after
+ * the softmax, [3] after the OV launch and the sum of its segments, so the stages of the product
+ * path can be timed without taking it apart.
+ */
+void adkv_set_stage_events(void *const *events);
 
 /*
  * fp32 ("train / eval") form of the recurrence: fake-quantise a token stream with the state kept
