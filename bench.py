@@ -458,7 +458,7 @@ def main():
     try:
         with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
             rec = json.load(f).get(workload_key)
-        if rec and rec.get("kernel") == "qk_" + kernel.split(" ")[0]:
+        if rec and rec.get("kernel") == "qk_" + kernel.split(" ")[0].rstrip(","):
             traffic = rec["bytes_per_launch"]
     except (OSError, ValueError):
         pass
@@ -508,7 +508,7 @@ def main():
     try:
         with open(os.path.join(ROOT, "profiles", "valu_issue.json")) as f:
             vrec = json.load(f).get(workload_key)
-        if vrec and vrec.get("kernel") == "qk_" + kernel.split(" ")[0]:
+        if vrec and vrec.get("kernel") == "qk_" + kernel.split(" ")[0].rstrip(","):
             cycles = qk_ms * 1e-3 * vrec["shader_clock_hz"]
             busy = vrec["valu_insts_per_launch"] * 4.0 / 1024.0
             res["roofline_valu"] = {"kernel": "qk_" + kernel, "bound": "valu",
