@@ -71,6 +71,7 @@ class KVCacheLayer_ADKV:
         self._device = None
         self._ckpt_interval = CKPT_INTERVAL
         self._views: dict = {}    # id(parameter) -> (parameter, its [H, C] view)
+        self._shares_storage = False   # a batch_view(): its buffers belong to another layer object
 
     # ------------------------------------------------------------------ HF cache protocol
     def get_seq_length(self) -> int:
@@ -125,6 +126,8 @@ class KVCacheLayer_ADKV:
         """Make room for ``T`` tokens.  New slots are zero, as the append kernels expect."""
         if T <= self._cap_len:
             return
+        if self._shares_storage:
+            raise RuntimeError("a batch view cannot grow: reserve() the parent cache for the whole context")
         want = max(T, int(self._cap_len * GROWTH))
         want = -(-want // CAP_LEN) * CAP_LEN
         cap, key, value, kck, vck = self._new_buffers(want)
@@ -137,6 +140,37 @@ class KVCacheLayer_ADKV:
             vck[:, :, :n].copy_(self._value_ckpt)
         self._key_buf, self._value_buf, self._key_ckpt, self._value_ckpt = key, value, kck, vck
         self._cap_len = cap
+
+    # ------------------------------------------------------------------ big batches, prompt in slices
+    def reserve(self, B: int, H: int, C: int, tokens: int, device) -> None:
+        """Allocate for a known batch and context up front: no growth copies later, and the
+        prompt of a batch too big for one dense prefill can be quantised slice by slice
+        through ``batch_view`` (the dense attention of a long prompt, not the cache, is what
+        limits the batch of a single prefill call)."""
+        self._init_buffers(B, H, C, torch.device(device))
+        self._cap_buffers(tokens)
+
+    def batch_view(self, b0: int, b1: int) -> "KVCacheLayer_ADKV":
+        """A layer object over sequences ``b0 .. b1-1`` of this one, sharing its storage (the batch
+        axis is the outermost, so the slices are contiguous).  Quantise a slice of the prompt
+        through it, then ``commit`` the parent."""
+        if self._key_buf is None or not 0 <= b0 < b1 <= self._B:
+            raise ValueError("batch_view needs a reserved cache and a slice inside its batch")
+        v = KVCacheLayer_ADKV(self._bits)
+        v._B, v._H, v._C, v._device = b1 - b0, self._H, self._C, self._device
+        v._ckpt_interval, v._cap_len, v._quant_len = self._ckpt_interval, self._cap_len, self._quant_len
+        v._key_buf, v._value_buf = self._key_buf[b0:b1], self._value_buf[b0:b1]
+        if self._key_ckpt is not None:
+            v._key_ckpt, v._value_ckpt = self._key_ckpt[b0:b1], self._value_ckpt[b0:b1]
+        v._key_state, v._value_state = self._key_state[b0:b1], self._value_state[b0:b1]
+        v._state_valid, v._shares_storage = self._state_valid, True
+        return v
+
+    def commit(self, tokens: int) -> None:
+        """Declare that every sequence now holds ``tokens`` quantised tokens (all slices prefilled)."""
+        if tokens > self._cap_len:
+            raise ValueError("more tokens than the cache holds")
+        self._quant_len, self._state_valid = tokens, True
 
     def _check_geometry(self, B: int, H: int, C: int, device: torch.device):
         if self._key_buf is None:
@@ -306,6 +340,19 @@ class KVCache_ADKV(list):
 
     def get_seq_length(self, layer_idx: int = 0) -> int:
         return self[layer_idx].get_seq_length()
+
+    def reserve(self, B: int, H: int, C: int, tokens: int, device) -> None:
+        for layer in self:
+            layer.reserve(B, H, C, tokens, device)
+
+    def batch_view(self, b0: int, b1: int) -> "KVCache_ADKV":
+        view = KVCache_ADKV(0)
+        view.extend(layer.batch_view(b0, b1) for layer in self)
+        return view
+
+    def commit(self, tokens: int) -> None:
+        for layer in self:
+            layer.commit(tokens)
 
     def get_mask_sizes(self, cache_position, layer_idx: int) -> tuple[int, int]:
         return self[layer_idx].get_mask_sizes(cache_position)

@@ -10,6 +10,9 @@ else from the synthetic benchmark parameters.
     python -m adkv_amd.tools.perf_e2e --batch_size 64 --kv adkv
     python -m adkv_amd.tools.perf_e2e --batch_size 64 --kv fp16
     python -m adkv_amd.tools.perf_e2e --search        # largest batch of each kind that fits
+    python -m adkv_amd.tools.perf_e2e --kv adkv --batch_size 448 --prompt_lenth 3840 --output_length 256 --prefill_slice 8
+                                                      # a batch near the memory limit at ctx 4096: the prompt
+                                                      # is prefilled slice by slice, then the whole batch decodes
 """
 from __future__ import annotations
 
@@ -43,6 +46,10 @@ def parse_args(argv=None):
     ap.add_argument("--search", action="store_true",
                     help="print the largest batch the memory model admits for each cache kind")
     ap.add_argument("--hbm_gib", type=float, default=288.0)
+    ap.add_argument("--prefill_slice", type=int, default=0,
+                    help="prefill the prompt this many sequences at a time into one cache for the whole "
+                         "batch, then decode the whole batch greedily (the dense attention and MLP "
+                         "activations of a long prompt, not the cache, limit the batch of one prefill call)")
     return ap.parse_args(argv)
 
 
@@ -102,6 +109,86 @@ def _heartbeat(stop: threading.Event, every: float = 30.0) -> None:
         print(f"[perf_e2e] running, {time.time() - t0:.0f} s", file=sys.stderr, flush=True)
 
 
+def sliced_run(args, model, cfg, source, device):
+    """Decode phase of a batch near the memory limit (the second number of the reference's
+    protocol, tools/perf_e2e.py:75-78 with --batch_size at the largest value that runs).  The
+    prompt goes in ``--prefill_slice`` sequences at a time: into views of one ADKV cache reserved
+    for the whole batch, or, for the fp16 cache, into per-slice caches concatenated layer by layer
+    afterwards.  Then every step feeds one token per sequence to the whole batch."""
+    from ..hf.cache import KVCache_ADKV
+
+    B, P, N, bs = args.batch_size, args.prompt_lenth, args.output_length, args.prefill_slice
+    g = torch.Generator().manual_seed(1)
+    ids = torch.randint(1, cfg.vocab_size, (B, P), generator=g).to(device)
+    d = cfg.hidden_size // cfg.num_attention_heads
+    first = torch.empty(B, dtype=torch.long, device=device)
+    stop = threading.Event()
+    threading.Thread(target=_heartbeat, args=(stop,), daemon=True).start()
+    torch.cuda.reset_peak_memory_stats()
+    with torch.no_grad():
+        t0 = time.time()
+        if args.kv == "adkv":
+            cache = KVCache_ADKV(cfg.num_hidden_layers)
+            cache.reserve(B, cfg.num_key_value_heads, d, P + N, device)
+            for b0 in range(0, B, bs):
+                b1 = min(B, b0 + bs)
+                r = model(ids[b0:b1], past_key_values=cache.batch_view(b0, b1), use_cache=True, logits_to_keep=1)
+                first[b0:b1] = r.logits[:, -1].argmax(-1)
+            cache.commit(P)
+        else:
+            from transformers import DynamicCache
+            # K and V of the whole batch are allocated before any activation exists and filled
+            # slice by slice: long-lived cache tensors carved out of freed activation blocks
+            # would fragment the allocator's pool by tens of GiB at this size
+            shape = (B, cfg.num_key_value_heads, P, d)
+            full = [(torch.empty(shape, dtype=torch.float16, device=device),
+                     torch.empty(shape, dtype=torch.float16, device=device))
+                    for _ in range(cfg.num_hidden_layers)]
+            for b0 in range(0, B, bs):
+                b1 = min(B, b0 + bs)
+                r = model(ids[b0:b1], use_cache=True, logits_to_keep=1)
+                first[b0:b1] = r.logits[:, -1].argmax(-1)
+                for i, layer in enumerate(r.past_key_values.layers):
+                    full[i][0][b0:b1].copy_(layer.keys)
+                    full[i][1][b0:b1].copy_(layer.values)
+                del r, layer
+                torch.cuda.empty_cache()
+            cache = DynamicCache()
+            for i in range(cfg.num_hidden_layers):
+                k, v = full[i]
+                full[i] = None
+                cache.update(k, v, i)                       # the cache makes its own copy
+                del k, v
+                torch.cuda.empty_cache()
+            del full
+        torch.cuda.synchronize()
+        prefill_s = time.time() - t0
+        print(f"[perf_e2e] prompt done in {prefill_s:.1f} s, "
+              f"{torch.cuda.memory_allocated() / 2 ** 30:.1f} GiB allocated", file=sys.stderr, flush=True)
+        tok = first
+        step_ms = []
+        for i in range(N - 1):
+            torch.cuda.synchronize()
+            t1 = time.time()
+            r = model(tok[:, None], past_key_values=cache, use_cache=True)
+            tok = r.logits[:, -1].argmax(-1)
+            torch.cuda.synchronize()
+            step_ms.append((time.time() - t1) * 1e3)
+            if i < 3 or i % 32 == 0:
+                print(f"[perf_e2e] decode step {i}: {step_ms[-1]:.1f} ms", file=sys.stderr, flush=True)
+    stop.set()
+    assert cache.get_seq_length() == P + N - 1
+    steps = sorted(step_ms)
+    decode_s = sum(step_ms) / 1e3
+    print(json.dumps({
+        "model": args.model, "layers": cfg.num_hidden_layers, "kv": args.kv, "weights": "random init fp16",
+        "adkv_params": source, "batch_size": B, "prompt_length": P, "output_length": N,
+        "prefill_slice": bs, "prefill_s": prefill_s, "decode_s": decode_s,
+        "decode_ms_per_step_median": steps[len(steps) // 2], "decode_ms_per_step_last": step_ms[-1],
+        "decode_tokens_per_s": B * (N - 1) / decode_s,
+        "peak_mem_GiB": torch.cuda.max_memory_allocated() / 2 ** 30}))
+
+
 def main(argv=None):
     args = parse_args(argv)
     if args.search:
@@ -109,6 +196,8 @@ def main(argv=None):
         return
     device = torch.device("cuda:0")
     model, cfg, source = build_model(args, device)
+    if args.prefill_slice > 0:
+        return sliced_run(args, model, cfg, source, device)
     g = torch.Generator().manual_seed(1)
     ids = torch.randint(1, cfg.vocab_size, (args.batch_size, args.prompt_lenth), generator=g).to(device)
     mask = torch.ones_like(ids)

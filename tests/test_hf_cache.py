@@ -479,6 +479,54 @@ def test_cache_save_and_restore_continues_identically(gpu, tmp_path, monkeypatch
     assert torch.equal(chunked[0].value_states[:, :, :n], whole.value_states[:, :, :n])
 
 
+def test_batch_views_share_storage_cpu():
+    c = KVCache_ADKV(2)
+    c.reserve(6, 2, 128, 300, "cpu")
+    assert c[0]._cap_len == 320 and c[1].key_states.shape == (6, 2, 40, 32, 4, 4)
+    v = c.batch_view(2, 5)
+    assert len(v) == 2 and v[0].key_states.shape[0] == 3 and v[0].key_states.is_contiguous()
+    v[1]._key_buf[0, 0, 0, 0, 0, 0] = 9
+    v[1]._key_state[1, 1, 7, 0] = 2.5
+    assert c[1]._key_buf[2, 0, 0, 0, 0, 0] == 9 and c[1]._key_state[3, 1, 7, 0] == 2.5
+    with pytest.raises(RuntimeError, match="cannot grow"):
+        v[0]._cap_buffers(1000)
+    with pytest.raises(ValueError, match="inside its batch"):
+        c[0].batch_view(4, 7)
+    c.commit(10)
+    assert c.get_seq_length() == 10
+    with pytest.raises(ValueError, match="more tokens"):
+        c[0].commit(1000)
+
+
+@pytest.mark.gpu
+def test_prompt_in_batch_slices_equals_one_prefill(gpu):
+    """A cache reserved for the whole batch and filled through batch views, slice by slice, holds
+    the same codes, checkpoints and carried state as one prefill of the whole batch, and decodes
+    to the same outputs."""
+    B, H, D, T0 = 5, 2, 128, 300
+    kp, vp = synth.make_params(H, D, seed=3), synth.make_params(H, D, seed=4)
+    kg, vg = _flat(kp.to(gpu)), _flat(vp.to(gpu))
+    k = synth.make_k(B, H, T0 + 1, D, dtype=torch.float16).to(gpu)
+    v = synth.make_v(B, H, T0 + 1, D, dtype=torch.float16).to(gpu)
+    whole = KVCacheLayer_ADKV()
+    whole.prefill(k[:, :, :T0], v[:, :, :T0], *kg, *vg)
+    sliced = KVCacheLayer_ADKV()
+    sliced.reserve(B, H, D, T0 + 8, gpu)
+    for b0, b1 in ((0, 2), (2, 5)):
+        sliced.batch_view(b0, b1).prefill(k[b0:b1, :, :T0], v[b0:b1, :, :T0], *kg, *vg)
+    sliced.commit(T0)
+    n = whole._n_super(T0)
+    assert torch.equal(sliced.key_states[:, :, :n], whole.key_states[:, :, :n])
+    assert torch.equal(sliced.value_states[:, :, :n], whole.value_states[:, :, :n])
+    nck = T0 // C.CKPT_INTERVAL
+    assert torch.equal(sliced._key_ckpt[:, :, :nck].view(torch.int16), whole._key_ckpt[:, :, :nck].view(torch.int16))
+    assert torch.equal(sliced._key_state.view(torch.int16), whole._key_state.view(torch.int16))
+    q = torch.randn(B, H, 1, D, generator=torch.Generator().manual_seed(5)).half().to(gpu)
+    o1, _ = whole.decode(q, k[:, :, T0:], v[:, :, T0:], *kg, *vg, scaling=D ** -0.5)
+    o2, _ = sliced.decode(q, k[:, :, T0:], v[:, :, T0:], *kg, *vg, scaling=D ** -0.5)
+    assert torch.equal(o1.view(torch.int16), o2.view(torch.int16))
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("bits,G,dtype", [(2, 1, torch.float16), (4, 4, torch.bfloat16), (2, 4, torch.bfloat16)])
 def test_cache_layer_grouped_queries_two_bit_and_bf16(gpu, oracle, bits, G, dtype):
