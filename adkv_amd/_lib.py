@@ -13,7 +13,7 @@ import torch  # noqa: F401  (loads libamdhip64 first)
 
 _DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_DIR, "libadkv_hip.so")
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 _vp, _i, _f = C.c_void_p, C.c_int, C.c_float
 
@@ -42,8 +42,8 @@ PROTOTYPES = {
     "adkv_init": (_i, []),
     "adkv_static_scratch_bytes": (C.c_int64, []),
     "adkv_forward_ov_noalloc": (_i, [_vp] * 9 + [_i] * 7 + [C.c_int64, _vp, _vp, _i, _i, _vp]),
-    "adkv_decode_fused_workspace_bytes": (C.c_int64, [_i] * 7),
-    "adkv_decode_fused": (_i, [_vp] * 8 + [_i, _f, _vp, _vp, C.c_int64] + [_i] * 8 + [_vp, _vp, _i, _i, _vp,
+    "adkv_decode_step_workspace_bytes": (C.c_int64, [_i] * 7),
+    "adkv_decode_step": (_i, [_vp] * 8 + [_i, _f, _vp, _vp, C.c_int64] + [_i] * 8 + [_vp, _vp, _i, _i, _vp,
                                                                             C.c_int64, _vp]),
     "adkv_set_stage_events": (None, [_vp]),
     "adkv_decode_kernel_name": (C.c_char_p, [_i] * 8),

@@ -1196,52 +1196,81 @@ __global__ __launch_bounds__(SM_BLOCK) void softmax_kernel(
 // one workgroup each: the first pass leaves (max, sum of exp(x - max)) per chunk, the second
 // combines a row's chunks and normalises.  Each logit is read twice and nothing depends on the
 // order in which workgroups run.
+
+// (m, s) with s = sum of exp(x - m) over a set of elements; the pair of the union of two sets.
+__device__ __forceinline__ float2 softmax_merge(float2 a, float2 b)
+{
+    const float m = fmaxf(a.x, b.x);
+    if (m == -INFINITY)
+        return make_float2(-INFINITY, 0.0f); // both sets empty or fully masked
+    return make_float2(m, a.y * __expf(a.x - m) + b.y * __expf(b.x - m));
+}
+
+__device__ __forceinline__ float2 softmax_wave_merge(float2 v)
+{
+#pragma unroll
+    for (int k = 1; k < 64; k <<= 1)
+        v = softmax_merge(v, make_float2(__shfl_xor(v.x, k, 64), __shfl_xor(v.y, k, 64)));
+    return v;
+}
+
 __global__ __launch_bounds__(SM_BLOCK) void softmax_part_kernel(
     const h1 *__restrict__ logits, const float *__restrict__ mask, float2 *__restrict__ part,
     int n, long ld, int nchunk, int rows_per_mask_row, float scaling)
 {
-    __shared__ float sm[SM_BLOCK / 64];
+    __shared__ float2 sm[SM_BLOCK / 64];
     const int row = blockIdx.y, ck = blockIdx.x;
     const h1 *l = logits + (size_t)row * ld;
     const float *mk = mask ? mask + (size_t)(row / rows_per_mask_row) * n : nullptr;
     float x[SM_KEEP], mx;
     softmax_load_chunk(l, mk, n, ck * SM_CHUNK, scaling, x, mx);
-    mx = block_reduce(mx, sm, true);
+    // the thread's own (max, sum), then ONE reduction of pairs over the workgroup
     float sum = 0.0f;
     if (mx > -INFINITY) {
 #pragma unroll
         for (int k = 0; k < SM_KEEP; k++)
             sum += __expf(x[k] - mx);
     }
-    sum = block_reduce(sum, sm, false);
-    if (threadIdx.x == 0)
-        part[(size_t)row * nchunk + ck] = make_float2(mx, sum);
+    const float2 w = softmax_wave_merge(make_float2(mx, sum));
+    if ((threadIdx.x & 63) == 0)
+        sm[threadIdx.x >> 6] = w;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float2 r = sm[0];
+#pragma unroll
+        for (int i = 1; i < SM_BLOCK / 64; i++)
+            r = softmax_merge(r, sm[i]);
+        part[(size_t)row * nchunk + ck] = r;
+    }
 }
 
 __global__ __launch_bounds__(SM_BLOCK) void softmax_norm_kernel(
     const h1 *__restrict__ logits, h1 *__restrict__ weights, const float *__restrict__ mask,
     const float2 *__restrict__ part, int n, long ld, int nchunk, int rows_per_mask_row, float scaling)
 {
+    __shared__ float2 row_stats;
     const int row = blockIdx.y, ck = blockIdx.x;
     const h1 *l = logits + (size_t)row * ld;
     h1 *w = weights + (size_t)row * ld;
     const float *mk = mask ? mask + (size_t)(row / rows_per_mask_row) * n : nullptr;
-    const float2 *pr = part + (size_t)row * nchunk;
-    float M = -INFINITY;
-    for (int k = 0; k < nchunk; k++)
-        M = fmaxf(M, pr[k].x);
-    float Z = 0.0f;
-    for (int k = 0; k < nchunk; k++) {
-        const float2 p = pr[k];
-        if (p.x > -INFINITY)
-            Z += p.y * __expf(p.x - M);
-    }
     float x[SM_KEEP], mx;
-    softmax_load_chunk(l, mk, n, ck * SM_CHUNK, scaling, x, mx);
+    softmax_load_chunk(l, mk, n, ck * SM_CHUNK, scaling, x, mx);   // issued first: in flight meanwhile
+    if (threadIdx.x < 64) {
+        // the row's (max, sum) from its chunks: one wave, a chunk per lane and round
+        const float2 *pr = part + (size_t)row * nchunk;
+        float2 v = make_float2(-INFINITY, 0.0f);
+        for (int k = threadIdx.x; k < nchunk; k += 64)
+            v = softmax_merge(v, pr[k]);
+        v = softmax_wave_merge(v);
+        if (threadIdx.x == 0)
+            row_stats = v;
+    }
+    __syncthreads();
+    const float M = row_stats.x, inv = 1.0f / row_stats.y;
 #pragma unroll
     for (int k = 0; k < SM_KEEP; k++)
         x[k] = __expf(x[k] - M);
-    softmax_store_chunk(w, n, ck * SM_CHUNK, x, 1.0f / Z);
+    softmax_store_chunk(w, n, ck * SM_CHUNK, x, inv);
 }
 
 } // namespace adkv
@@ -1482,7 +1511,7 @@ static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval, int b
 
 extern "C" {
 
-int adkv_abi_version(void) { return 12; }
+int adkv_abi_version(void) { return 13; }
 
 void adkv_set_mha_kernel(int use_matrix_cores)
 {
@@ -1724,7 +1753,7 @@ static const char *decode_kernel_name(int B, int Hq, int H, int T, int D, int bi
     return D == 256 ? "kernel<256,4,*> (shared table)" : "kernel<512,8,256> (shared table)";
 }
 
-// act_bf16: q, k_new / v_new and the output are bfloat16 (only adkv_decode_fused asks for it)
+// act_bf16: q, k_new / v_new and the output are bfloat16 (only adkv_decode_step asks for it)
 static int forward_qk_impl(const void *q, void *k_cache, const void *k_new, void *logits,
                            const void *zp, const void *sc, const void *alpha, const void *beta,
                            const void *tgt,
@@ -2089,7 +2118,7 @@ int adkv_softmax(const void *logits, void *weights, const void *mask,
 
 static int64_t pad256(int64_t n) { return (n + 255) & ~(int64_t)255; }
 
-// Events adkv_decode_fused records around its stages in this thread (a measurement hook).
+// Events adkv_decode_step records around its stages in this thread (a measurement hook).
 static thread_local hipEvent_t g_stage_events[4] = {nullptr, nullptr, nullptr, nullptr};
 
 void adkv_set_stage_events(void *const *events)
@@ -2118,7 +2147,7 @@ int64_t adkv_forward_ov_gqa_workspace_bytes(int B, int Hq, int H, int T, int D, 
     return adkv_forward_ov_workspace_bytes(B, H, T, D, n_ckpt_cap, ckpt_interval) * (Hq / H);
 }
 
-int64_t adkv_decode_fused_workspace_bytes(int B, int Hq, int H, int T, int D, int n_ckpt_cap,
+int64_t adkv_decode_step_workspace_bytes(int B, int Hq, int H, int T, int D, int n_ckpt_cap,
                                           int ckpt_interval)
 {
     if (B <= 0 || H <= 0 || Hq <= 0 || T < 0)
@@ -2128,7 +2157,7 @@ int64_t adkv_decode_fused_workspace_bytes(int B, int Hq, int H, int T, int D, in
            adkv_forward_ov_gqa_workspace_bytes(B, Hq, H, T, D, n_ckpt_cap, ckpt_interval);
 }
 
-int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k_new, const void *v_new,
+int adkv_decode_step(const void *q, void *k_cache, void *v_cache, const void *k_new, const void *v_new,
                       const void *const *k_params, const void *const *v_params,
                       const void *mask, int rows_per_mask_row, float scaling,
                       void *out, void *weights_out, int64_t weights_ld,
@@ -2143,7 +2172,7 @@ int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k
     const int act_bf16 = act_dtype == ADKV_DT_BF16;
     if (B <= 0 || H <= 0 || Hq <= 0 || Hq % H || T < 0)
         return ADKV_E_SHAPE;
-    if (workspace_bytes < adkv_decode_fused_workspace_bytes(B, Hq, H, T, D, n_ckpt_cap, ckpt_interval))
+    if (workspace_bytes < adkv_decode_step_workspace_bytes(B, Hq, H, T, D, n_ckpt_cap, ckpt_interval))
         return ADKV_E_WORKSPACE;
     if ((uintptr_t)workspace & 255)
         return ADKV_E_ALIGN;

@@ -21,7 +21,7 @@ import math
 
 import torch
 
-from ..kernel.gemv import append_kv_pair, decode_fused, decode_fused_workspace_bytes
+from ..kernel.gemv import append_kv_pair, decode_step, decode_step_workspace_bytes
 
 SCALE_MIN = math.exp(-4.0)  # kept for API parity; the fp16 recurrence never clamps
 SCALE_MAX = math.exp(4.0)
@@ -254,7 +254,7 @@ class KVCacheLayer_ADKV:
         ctx = self._quant_len
         self._cap_buffers(ctx + 1)
 
-        # fp16 and bf16 activations go in as they are; the kernels convert (see decode_fused)
+        # fp16 and bf16 activations go in as they are; the kernels convert (see decode_step)
         same = query_states.dtype in (torch.float16, torch.bfloat16) \
             and key_states.dtype == query_states.dtype == value_states.dtype
         f16 = (lambda t: t.contiguous()) if same else (lambda t: t.to(torch.float16).contiguous())
@@ -262,8 +262,8 @@ class KVCacheLayer_ADKV:
         S = self._ckpt_interval
         dev = query_states.device
         ncap = self._key_ckpt.shape[2] if S else 0
-        ws = _workspace(dev, decode_fused_workspace_bytes(B, Hq, H, ctx, C, ncap, S))
-        out, weights = decode_fused(
+        ws = _workspace(dev, decode_step_workspace_bytes(B, Hq, H, ctx, C, ncap, S))
+        out, weights = decode_step(
             f16(query_states), self._key_buf, self._value_buf, f16(key_states), f16(value_states),
             (v(key_zp_init), v(key_scale_init), v(key_alpha), v(key_beta), v(key_quant_target)),
             (v(value_zp_init), v(value_scale_init), v(value_alpha), v(value_beta),

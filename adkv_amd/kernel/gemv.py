@@ -473,7 +473,7 @@ def softmax_scale_mask(logits: torch.Tensor, scaling: float,
     return out
 
 
-def decode_fused(
+def decode_step(
     q: torch.Tensor,
     k_cache: torch.Tensor,
     v_cache: torch.Tensor,
@@ -501,7 +501,7 @@ def decode_fused(
     round them to fp16 as they read them and return ``out`` in bfloat16, with the values of the
     reference's ``.to(torch.float16)`` / ``.to(q.dtype)`` around its kernels
     (llama_adkv.py:248-250, 274) but without those launches.  ``workspace`` (uint8, 256-byte aligned, sized by
-    ``decode_fused_workspace_bytes``) may be passed to avoid the per-call allocation.
+    ``decode_step_workspace_bytes``) may be passed to avoid the per-call allocation.
     """
     f16, u8 = torch.float16, torch.uint8
     act = q.dtype            # float16 as in the reference, or bfloat16 (extension; see the docstring)
@@ -544,7 +544,7 @@ def decode_fused(
          "k_ckpt and v_ckpt must both be given, with the same capacity, or both omitted")
     L = _lib.lib()
     if workspace is None:
-        need = L.adkv_decode_fused_workspace_bytes(B, nq, nh, T, DIM, ccap, civ)
+        need = L.adkv_decode_step_workspace_bytes(B, nq, nh, T, DIM, ccap, civ)
         workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     # a caller's workspace is sized against the launch by the library itself ("workspace too small")
     _chk(workspace.dtype == torch.uint8 and workspace.is_cuda, "workspace must be a uint8 device tensor")
@@ -556,19 +556,19 @@ def decode_fused(
     weights = torch.empty((B, nq, wld), dtype=torch.float16, device=dev)
     arr = _lib.C.c_void_p * 5
     with _lib.device_guard(dev):
-        rc = L.adkv_decode_fused(
+        rc = L.adkv_decode_step(
             qf.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), knf.data_ptr(), vnf.data_ptr(),
             arr(*[t.data_ptr() for t in kp]), arr(*[t.data_ptr() for t in vp]),
             mptr, rpm, float(scaling), out.data_ptr(), weights.data_ptr(), wld,
             B, nq, nh, T, DIM, n_super_cap, bits, _DT_BF16 if act == torch.bfloat16 else _DT_F16,
             kcp, vcp, ccap, civ,
             workspace.data_ptr(), workspace.numel(), _lib.current_stream_ptr(dev))
-    _lib.check(rc, "decode_fused")
+    _lib.check(rc, "decode_step")
     return out, weights[:, :, :n]
 
 
-def decode_fused_workspace_bytes(B: int, nq: int, nh: int, T: int, DIM: int, n_ckpt_cap: int = 0,
+def decode_step_workspace_bytes(B: int, nq: int, nh: int, T: int, DIM: int, n_ckpt_cap: int = 0,
                                  ckpt_interval: int = 0) -> int:
-    """Bytes ``decode_fused`` needs for ``nq`` query heads over ``nh`` KV heads."""
-    return int(_lib.lib().adkv_decode_fused_workspace_bytes(B, nq, nh, T, DIM, n_ckpt_cap,
+    """Bytes ``decode_step`` needs for ``nq`` query heads over ``nh`` KV heads."""
+    return int(_lib.lib().adkv_decode_step_workspace_bytes(B, nq, nh, T, DIM, n_ckpt_cap,
                                                             ckpt_interval))

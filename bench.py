@@ -3,7 +3,7 @@
 
 One "step" is one layer's decode-attention for a batch: forward_qk (+append) -> softmax ->
 forward_ov (+append) over a resident 4-bit K/V cache, the protocol of the reference's
-tools/perf_kernel.py:28-76, issued the way the cache object issues it: one adkv_decode_fused call.  Throughput follows its convention (perf_kernel.py:91-104):
+tools/perf_kernel.py:28-76, issued the way the cache object issues it: one adkv_decode_step call.  Throughput follows its convention (perf_kernel.py:91-104):
 tokens/s = B / (32 layers * seconds per layer-step).  Caches are produced by running the encoder
 on seeded synthetic K/V (closed loop), and the timed steps rotate over several distinct layer
 buffers so no cache level can serve re-reads.
@@ -394,11 +394,11 @@ def main():
     L = _lib.lib()
     ncap_arg = ncap if S else 0
     kernel = L.adkv_decode_kernel_name(B, Hq, H, T, D, bits, ncap_arg, S).decode()
-    ws = torch.empty(gemv.decode_fused_workspace_bytes(B, Hq, H, T, D, ncap_arg, S), dtype=torch.uint8, device=dev)
+    ws = torch.empty(gemv.decode_step_workspace_bytes(B, Hq, H, T, D, ncap_arg, S), dtype=torch.uint8, device=dev)
 
     def fused(l):
         # the product path: what KVCacheLayer_ADKV.decode calls, one library call per layer-step
-        return gemv.decode_fused(q, kcs[l], vcs[l], k_new, v_new, kps[l], vps[l], T, scaling,
+        return gemv.decode_step(q, kcs[l], vcs[l], k_new, v_new, kps[l], vps[l], T, scaling,
                                  k_ckpt=kks[l], v_ckpt=vks[l], ckpt_interval=S, bits=bits, workspace=ws)
 
     # four events per timed step, recorded by the library around the stages of the fused call
@@ -479,7 +479,7 @@ def main():
         "config": {
             "workload": f"{'cfg2 Llama-2-7B-shaped' if H == Hq else 'grouped-query'} ADKV decode attention: "
                         f"B={B} H={Hq}{'' if H == Hq else f' (KV heads {H})'} d={D} ctx={T} "
-                        f"{bits}-bit K+V codes, step = one decode_fused call (forward_qk+softmax+forward_ov, "
+                        f"{bits}-bit K+V codes, step = one decode_step call (forward_qk+softmax+forward_ov, "
                         f"appending the new token), {NL} rotating layer caches, state checkpoints every {S} tokens",
             "batch": B, "heads": Hq, "kv_heads": H, "head_dim": D, "ctx": T, "bits": bits, "ckpt_interval": S,
             "parallelism": "1 GPU",
@@ -501,7 +501,7 @@ def main():
     }
     if graph_ms is not None:
         res["graph_replay"] = {"ms_per_step": graph_ms, "tokens_per_s": B / (N_LAYERS_MODEL * graph_ms * 1e-3),
-                               "note": "the same decode_fused step captured once per layer cache and replayed"}
+                               "note": "the same decode_step step captured once per layer cache and replayed"}
     # The binding roof of this kernel is vector-instruction issue, not HBM: vector instructions
     # per launch (profiles/valu_issue.json, from rocprofv3 SQ_INSTS_VALU) x 4 cycles per wave64
     # instruction / (1024 SIMDs x the kernel's duration) at the shader clock seen under load.

@@ -245,9 +245,14 @@ int adkv_forward_ov_noalloc(const void *attn, void *v_cache, const void *v_new, 
                             void *stream);
 
 /*
- * One decode-attention step of one layer in a single call: forward_qk -> scale/mask/softmax ->
- * forward_ov, appending k_new / v_new at slot T of both caches.  Replaces the body of
- * KVCacheLayer_ADKV.decode (src/adkv/hf/llama_adkv.py:245-276).
+ * One decode-attention step of one layer in a single library call: the launches of forward_qk,
+ * scale/mask/softmax and forward_ov (plus the sum of forward_ov's segments) issued back to back
+ * on `stream`, appending k_new / v_new at slot T of both caches.  It is one CALL, not one kernel:
+ * logits and weights pass through the workspace between the launches.  (A single kernel was
+ * evaluated and not built: the softmax arithmetic costs the same vector instructions wherever it
+ * runs, these kernels are bound by vector-instruction issue and not by the logits' round trip, and
+ * the per-head table that the QK and OV kernels each build needs the whole LDS of a CU for itself.)
+ * Replaces the body of KVCacheLayer_ADKV.decode (src/adkv/hf/llama_adkv.py:245-276).
  * q: fp16 [B, Hq, D] with Hq a multiple of the H KV heads (Hq == H is the reference's case).
  * k_params / v_params: host arrays of five device pointers {zp, sc, alpha, beta, tgt}, each
  * fp16 [H, D].  mask: optional fp32 additive mask as in adkv_softmax.  out: fp16 [B, Hq, D].
@@ -257,11 +262,11 @@ int adkv_forward_ov_noalloc(const void *attn, void *v_cache, const void *v_new, 
  * rounded to fp16 as they are read and the fp16 result to bf16 as it is written, the values of
  * the reference's .to(torch.float16) / .to(q.dtype) around its kernels (llama_adkv.py:248-250, 274)
  * without the four conversion launches.  Logits and weights stay fp16.
- * workspace: >= adkv_decode_fused_workspace_bytes(...) bytes, 256-byte aligned.
+ * workspace: >= adkv_decode_step_workspace_bytes(...) bytes, 256-byte aligned.
  */
-int64_t adkv_decode_fused_workspace_bytes(int B, int Hq, int H, int T, int D, int n_ckpt_cap,
+int64_t adkv_decode_step_workspace_bytes(int B, int Hq, int H, int T, int D, int n_ckpt_cap,
                                           int ckpt_interval);
-int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k_new,
+int adkv_decode_step(const void *q, void *k_cache, void *v_cache, const void *k_new,
                       const void *v_new, const void *const *k_params, const void *const *v_params,
                       const void *mask, int rows_per_mask_row, float scaling,
                       void *out, void *weights_out, int64_t weights_ld,
@@ -270,7 +275,7 @@ int adkv_decode_fused(const void *q, void *k_cache, void *v_cache, const void *k
                       void *workspace, int64_t workspace_bytes, void *stream);
 
 /* Which of the library's decode kernels adkv_forward_qk_gqa / adkv_forward_ov_gqa /
- * adkv_decode_fused launch for these sizes ("qk_" / "ov_" + the returned text): a static string,
+ * adkv_decode_step launch for these sizes ("qk_" / "ov_" + the returned text): a static string,
  * for benchmark records and tests; "invalid" for sizes the entry points reject. */
 const char *adkv_decode_kernel_name(int B, int Hq, int H, int T, int D, int bits, int n_ckpt_cap,
                                     int ckpt_interval);
@@ -278,7 +283,7 @@ const char *adkv_decode_kernel_name(int B, int Hq, int H, int T, int D, int bits
 /*
  * Measurement hook, no counterpart in the reference (its benchmark times whole steps with CUDA
  * events, tools/perf_kernel.py:65-74): `events` is a host array of four hipEvent_t created with
- * timing enabled, or NULL to switch the hook off.  While set, every adkv_decode_fused call of
+ * timing enabled, or NULL to switch the hook off.  While set, every adkv_decode_step call of
  * THIS host thread records them on its stream: [0] before the QK launch, [1] after it, [2] after
  * the softmax, [3] after the OV launch and the sum of its segments, so the stages of the product
  * path can be timed without taking it apart.

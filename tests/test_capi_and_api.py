@@ -74,7 +74,7 @@ def test_paired_append_and_fused_decode_validation_needs_no_device():
     assert L.adkv_append_kv_pair(*pair(2, st3(1025, 128, 128), None)) == -3   # odd stride: rows unaligned
     fused = [one] * 5 + [arr5, arr5, None, 1, 1.0, one, None, 0, 1, 1, 1, 8, 128, 2, 4, 0,
              None, None, 0, 0, one, 1 << 20, None]
-    assert L.adkv_decode_fused(*fused) == -6                                # activation dtype must be f16 / bf16
+    assert L.adkv_decode_step(*fused) == -6                                # activation dtype must be f16 / bf16
 
 
 def test_row_strides_of_projection_outputs():

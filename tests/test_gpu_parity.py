@@ -383,8 +383,8 @@ def test_fp16_comparator_rejects_other_head_dims(gpu):
 @pytest.mark.parametrize("B,H,T,D,S,masked", [
     (2, 4, 257, 128, 0, False), (2, 3, 530, 128, 64, True), (1, 2, 100, 256, 16, False),
     (1, 2, 0, 128, 0, False)])
-def test_decode_fused_equals_three_calls(gpu, B, H, T, D, S, masked):
-    """adkv_decode_fused is the three entry points chained inside the library: outputs, weights,
+def test_decode_step_equals_three_calls(gpu, B, H, T, D, S, masked):
+    """adkv_decode_step is the three entry points chained inside the library: outputs, weights,
     appended codes and checkpoints must equal the separate calls bit for bit."""
     kp = [t.to(gpu) for t in synth.make_params(H, D, seed=3).astuple()]
     vp = [t.to(gpu) for t in synth.make_params(H, D, seed=4).astuple()]
@@ -414,7 +414,7 @@ def test_decode_fused_equals_three_calls(gpu, B, H, T, D, S, masked):
     out = gemv.forward_ov(w, vc, v[:, :, T:], *vp, SMIN, SMAX, ckpt=vk, ckpt_interval=S)
 
     kc2, vc2, kk2, vk2 = fresh()
-    out2, w2 = gemv.decode_fused(q, kc2, vc2, k[:, :, T:], v[:, :, T:], kp, vp, T, scaling, mask,
+    out2, w2 = gemv.decode_step(q, kc2, vc2, k[:, :, T:], v[:, :, T:], kp, vp, T, scaling, mask,
                                  k_ckpt=kk2, v_ckpt=vk2, ckpt_interval=S)
     torch.cuda.synchronize()
     assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
@@ -451,12 +451,12 @@ def test_decode_step_replays_from_a_captured_graph(gpu, H, Hq, T, S, bits):
                             k_ckpt=kk, v_ckpt=vk, ckpt_interval=S, bits=bits)
         return kc, vc, kk, vk
 
-    ws_bytes = gemv.decode_fused_workspace_bytes(B, Hq, H, T, D, ncap, S)
+    ws_bytes = gemv.decode_step_workspace_bytes(B, Hq, H, T, D, ncap, S)
     ws = torch.empty(ws_bytes + 256, dtype=torch.uint8, device=gpu)
     ws = ws[(-ws.data_ptr()) % 256:][:ws_bytes]
 
     def step(kc, vc, kk, vk):
-        return gemv.decode_fused(q, kc, vc, k[:, :, T:], v[:, :, T:], kp, vp, T, scaling, None,
+        return gemv.decode_step(q, kc, vc, k[:, :, T:], v[:, :, T:], kp, vp, T, scaling, None,
                                  k_ckpt=kk, v_ckpt=vk, ckpt_interval=S, bits=bits, workspace=ws)
 
     e = fresh()
@@ -495,7 +495,7 @@ def test_decode_step_replays_from_a_captured_graph(gpu, H, Hq, T, S, bits):
     (2, 2, 8, 530, 64, 4),       # matrix-core kernels, 4 query heads per KV head
     (1, 2, 16, 200, 32, 2),      # 2-bit codes, 8 query heads per KV head
 ])
-def test_decode_fused_takes_bfloat16_activations(gpu, B, H, Hq, T, S, bits):
+def test_decode_step_takes_bfloat16_activations(gpu, B, H, Hq, T, S, bits):
     """q, k_new, v_new in bfloat16: the kernels round them to fp16 on the way in and the result to
     bfloat16 on the way out.  Everything equals the fp16 call on `.to(float16)` inputs followed by
     `.to(bfloat16)`: output bits, weights, appended codes, checkpoints."""
@@ -521,10 +521,10 @@ def test_decode_fused_takes_bfloat16_activations(gpu, B, H, Hq, T, S, bits):
         return kc, vc, kk, vk
 
     a = fresh()
-    out_a, w_a = gemv.decode_fused(qb.half(), a[0], a[1], kb.half(), vb.half(), kp, vp, T, D ** -0.5, None,
+    out_a, w_a = gemv.decode_step(qb.half(), a[0], a[1], kb.half(), vb.half(), kp, vp, T, D ** -0.5, None,
                                    k_ckpt=a[2], v_ckpt=a[3], ckpt_interval=S, bits=bits)
     b = fresh()
-    out_b, w_b = gemv.decode_fused(qb, b[0], b[1], kb, vb, kp, vp, T, D ** -0.5, None,
+    out_b, w_b = gemv.decode_step(qb, b[0], b[1], kb, vb, kp, vp, T, D ** -0.5, None,
                                    k_ckpt=b[2], v_ckpt=b[3], ckpt_interval=S, bits=bits)
     torch.cuda.synchronize()
     assert out_a.dtype == torch.float16 and out_b.dtype == torch.bfloat16
@@ -877,7 +877,7 @@ def test_encode_rounding_boundaries(gpu, oracle, bits):
 
 def test_long_context_grouped_query_full_size(gpu, oracle):
     """B=16, 32 query heads over 8 KV heads, d=128, ctx 131072, 2-bit codes, bfloat16 activations:
-    the whole step through decode_fused at its real size (the 16-wave matrix-core kernels with
+    the whole step through decode_step at its real size (the 16-wave matrix-core kernels with
     four query heads per KV head, 64 segments, chunked softmax).  Size-independent properties over
     the whole tensor, and two sampled (sequence, KV head) pairs against the oracle:
     (1) encode(T) + the in-kernel append of token T == encode(T+1), byte for byte, K and V;
@@ -910,7 +910,7 @@ def test_long_context_grouped_query_full_size(gpu, oracle):
     torch.cuda.empty_cache()
     q = synth.make_q(B, Hq, D, dtype=bf, device=gpu)
     kc, vc = caches[0].clone(), caches[1].clone()
-    out, w = gemv.decode_fused(q, kc, vc, news[0], news[1], kp.astuple(), vp.astuple(), T, D ** -0.5,
+    out, w = gemv.decode_step(q, kc, vc, news[0], news[1], kp.astuple(), vp.astuple(), T, D ** -0.5,
                                k_ckpt=ckpts[0], v_ckpt=ckpts[1], ckpt_interval=S, bits=bits)
     torch.cuda.synchronize()
     assert out.dtype == bf and out.shape == (B, Hq, D) and w.shape == (B, Hq, T + 1)
