@@ -494,11 +494,25 @@ def test_decode_step_replays_from_a_captured_graph(gpu, H, Hq, T, S, bits):
     (40, 32, 32, 300, 64, 4),    # enough units for four channels per lane
     (2, 2, 8, 530, 64, 4),       # matrix-core kernels, 4 query heads per KV head
     (1, 2, 16, 200, 32, 2),      # 2-bit codes, 8 query heads per KV head
+    (3, 2, -2, 530, 64, 4),      # the per-head-table kernels (forced), a few segments
+    (5, 3, -3, 257, 0, 4),       # the per-head-table kernels (forced), one segment
 ])
 def test_decode_step_takes_bfloat16_activations(gpu, B, H, Hq, T, S, bits):
     """q, k_new, v_new in bfloat16: the kernels round them to fp16 on the way in and the result to
     bfloat16 on the way out.  Everything equals the fp16 call on `.to(float16)` inputs followed by
-    `.to(bfloat16)`: output bits, weights, appended codes, checkpoints."""
+    `.to(bfloat16)`: output bits, weights, appended codes, checkpoints.  (A negative Hq means
+    -Hq query heads with the per-head-table kernels forced.)"""
+    from adkv_amd import _lib
+    if Hq < 0:
+        Hq = -Hq
+        _lib.lib().adkv_set_mha_kernel(2)
+    try:
+        _bf16_case(gpu, B, H, Hq, T, S, bits)
+    finally:
+        _lib.lib().adkv_set_mha_kernel(-1)
+
+
+def _bf16_case(gpu, B, H, Hq, T, S, bits):
     D = 128
     tps = 32 // bits
     kp = [t.to(gpu) for t in synth.make_params(H, D, seed=3, bits=bits).astuple()]
