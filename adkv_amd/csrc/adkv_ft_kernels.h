@@ -119,65 +119,6 @@ __device__ __forceinline__ void update_pair_f(Pair &p, h2 f, h2 qs)
     p.sc = p.sc * f;
 }
 
-// a.x*b.x + a.y*b.y in fp32, as the three-operand form with a literal zero accumulator: the
-// accumulating two-operand form the compiler picks needs its destination cleared first, one more
-// vector instruction per token.  The leading wait state covers an operand that the instruction
-// just before wrote as a packed 16-bit result (on this chip such a result cannot be forwarded to
-// the very next instruction; the compiler pads its own code the same way).
-__device__ __forceinline__ float dot2_from_zero(h2 a, h2 b)
-{
-    float d;
-    asm("s_nop 0\n\tv_dot2_f32_f16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b));
-    return d;
-}
-
-// Sum of 8 per-lane partials over the 32 lanes of a head, scattered: afterwards every lane holds
-// the total of ONE token, token_of_lane(lane), the same in the four lanes of a quad.
-//   bit 3 of the lane (banks 0,1 | 2,3): keep tokens 0-3 | 4-7, add the partner's    8 instructions
-//   bit 2 (banks 0,2 | 1,3):             keep tokens +0,+1 | +2,+3                      4
-//   bit 4 (row 0 | 1 of the head):       v_permlane16_swap + add, keep token +0 | +1    2
-//   bits 0,1: all-reduce inside the quad                                                2
-// A masked DPP add writes only the banks of its mask and keeps the other lanes' destination; a
-// DPP operand must not have been written by the two preceding instructions, which the order
-// below guarantees inside the block and the leading s_nop for whatever precedes it.
-__device__ __forceinline__ float reduce8_head32(const float *p)
-{
-    float r0, r1, r2, r3, s0, s1;
-    asm volatile(
-        "s_nop 1\n\t"
-        "v_add_f32_dpp %0, %6, %6 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
-        "v_add_f32_dpp %1, %7, %7 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
-        "v_add_f32_dpp %2, %8, %8 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
-        "v_add_f32_dpp %3, %9, %9 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
-        "v_add_f32_dpp %0, %10, %10 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-        "v_add_f32_dpp %1, %11, %11 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-        "v_add_f32_dpp %2, %12, %12 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-        "v_add_f32_dpp %3, %13, %13 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
-        // banks 0,2 take lane+4 (rotate right by 12), banks 1,3 take lane-4 (rotate right by 4)
-        "v_add_f32_dpp %4, %0, %0 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
-        "v_add_f32_dpp %5, %1, %1 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
-        "v_add_f32_dpp %4, %2, %2 row_ror:4 row_mask:0xf bank_mask:0xa\n\t"
-        "v_add_f32_dpp %5, %3, %3 row_ror:4 row_mask:0xf bank_mask:0xa\n\t"
-        "s_nop 1\n\t"
-        "v_permlane16_swap_b32 %4, %5\n\t"
-        "s_nop 1\n\t"
-        "v_add_f32 %4, %4, %5\n\t"
-        "s_nop 1\n\t"
-        "v_add_f32_dpp %4, %4, %4 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
-        "s_nop 1\n\t"
-        "v_add_f32_dpp %4, %4, %4 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
-        "s_nop 0"
-        : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3), "=&v"(s0), "=&v"(s1)
-        : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]));
-    return s0;
-}
-
-__device__ __forceinline__ int token_of_lane(int lane)
-{
-    const int bank = (lane >> 2) & 3, row = (lane >> 4) & 1;
-    return 4 * (bank >> 1) + 2 * (bank & 1) + row;
-}
-
 // ---------------------------------------------------------------------------------------------
 // forward_qk  (gemv.cu:435-815), per-head table
 // ---------------------------------------------------------------------------------------------

@@ -127,6 +127,74 @@ __device__ __forceinline__ float head_allreduce(float v)
     return v;
 }
 
+// a.x*b.x + a.y*b.y in fp32, as the three-operand form with a literal zero accumulator: the
+// accumulating two-operand form the compiler picks needs its destination cleared first, one more
+// vector instruction per token.  The leading wait state covers an operand that the instruction
+// just before wrote as a packed 16-bit result (on this chip such a result cannot be forwarded to
+// the very next instruction; the compiler pads its own code the same way).
+__device__ __forceinline__ float dot2_from_zero(h2 a, h2 b)
+{
+    float d;
+    asm("s_nop 0\n\tv_dot2_f32_f16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b));
+    return d;
+}
+
+// Sum of 8 per-lane partials over the 32 lanes of a head, scattered: afterwards every lane holds
+// the total of ONE token, token_of_lane(lane), the same in the four lanes of a quad.
+//   bit 3 of the lane (banks 0,1 | 2,3): keep tokens 0-3 | 4-7, add the partner's    8 instructions
+//   bit 2 (banks 0,2 | 1,3):             keep tokens +0,+1 | +2,+3                      4
+//   bit 4 (row 0 | 1 of the head):       v_permlane16_swap + add, keep token +0 | +1    2
+//   bits 0,1: all-reduce inside the quad                                                2
+// A masked DPP add writes only the banks of its mask and keeps the other lanes' destination; a
+// DPP operand must not have been written by the two preceding instructions, which the order
+// below guarantees inside the block and the leading s_nop for whatever precedes it.
+__device__ __forceinline__ float reduce8_head32(const float *p)
+{
+    float r0, r1, r2, r3, s0, s1;
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_add_f32_dpp %0, %6, %6 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %1, %7, %7 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %2, %8, %8 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %3, %9, %9 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %0, %10, %10 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %1, %11, %11 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %2, %12, %12 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %3, %13, %13 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        // banks 0,2 take lane+4 (rotate right by 12), banks 1,3 take lane-4 (rotate right by 4)
+        "v_add_f32_dpp %4, %0, %0 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %5, %1, %1 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %4, %2, %2 row_ror:4 row_mask:0xf bank_mask:0xa\n\t"
+        "v_add_f32_dpp %5, %3, %3 row_ror:4 row_mask:0xf bank_mask:0xa\n\t"
+        "s_nop 1\n\t"
+        "v_permlane16_swap_b32 %4, %5\n\t"
+        "s_nop 1\n\t"
+        "v_add_f32 %4, %4, %5\n\t"
+        "s_nop 1\n\t"
+        "v_add_f32_dpp %4, %4, %4 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_add_f32_dpp %4, %4, %4 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0"
+        : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3), "=&v"(s0), "=&v"(s1)
+        : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]));
+    return s0;
+}
+
+__device__ __forceinline__ int token_of_lane(int lane)
+{
+    const int bank = (lane >> 2) & 3, row = (lane >> 4) & 1;
+    return 4 * (bank >> 1) + 2 * (bank & 1) + row;
+}
+
+// The same sum over a head of LPH lanes: a 64-lane head adds its two halves at the end (both then
+// hold every token's total).
+template <int LPH>
+__device__ __forceinline__ float reduce8_head(const float *p)
+{
+    const float s = reduce8_head32(p);
+    return LPH == 64 ? xor32_add(s) : s;
+}
+
 // (zp, sc) of CPL consecutive channels <-> the interleaved [channel][2] fp16 layout used for
 // state_out and checkpoints.
 template <int CPL>
@@ -613,9 +681,8 @@ __device__ __forceinline__ void pair_bytes_of(const typename Geo<D, CPL>::Vec *u
 // forward_qk  (gemv.cu:435-815)
 // ---------------------------------------------------------------------------------------------
 // Per lane and supergroup: 8 fp32 partial logits (v_dot2_f32_f16 over the lane's channel pairs).
-// They are summed across the head's lanes through a wave-private, conflict-free (stride 9) LDS
-// transpose: lane (g, tk) adds the partials of token tk from lanes 8g..8g+7, then row/half swaps
-// fold the remaining LPH/8 groups.
+// They are summed across the head's lanes and scattered by reduce8_head (masked DPP adds and row
+// swaps, no LDS): afterwards every quad of lanes holds the total of one token.
 template <int D, int CPL, int BLK>
 __global__ __launch_bounds__(BLK) void qk_kernel(
     const h1 *__restrict__ q, uint4 *__restrict__ cache, const h1 *__restrict__ k_new,
@@ -625,15 +692,14 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
     int BH, int H, int T, int n_super_cap, h1 *__restrict__ state_out, Seg sa)
 {
     using G = Geo<D, CPL>;
-    // one allocation so the table sits at LDS offset 0 (its byte address is used as is)
-    __shared__ uint2 smem[LUT_WORDS64 + (BLK / 64) * 64 * 9 / 2];
+    // the only LDS object: the table sits at LDS offset 0 (its byte address is used as is)
+    __shared__ uint2 smem[LUT_WORDS64];
     const uint2 *lut = smem;
     lut_fill(smem, threadIdx.x, BLK);
     __syncthreads();
 
     const int lane = threadIdx.x & 63;
     const uint32_t lane_copy = (uint32_t)(lane & (LUT_COPIES - 1)) * 8u;
-    float *myred = reinterpret_cast<float *>(smem + LUT_WORDS64) + (threadIdx.x >> 6) * 64 * 9;
 
     const Unit<D, CPL, BLK> un(BH, sa.nseg);
     const int bx = un.bx, lh = un.lh, c0 = un.c0;
@@ -655,44 +721,34 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
     const Vec *cb = cbh + (size_t)(t0 >> 3) * G::VPS;                                           // this segment
     h1 *ob = out + (size_t)bx * sa.row_pitch + t0;
     const int nfull = (t1 - t0) >> 3;
-    const int tk = lane & 7, g8 = lane >> 3;
-
-    // ---- cross-lane sum of the 8 per-token partials, split in three phases so that the LDS round
-    // trip of supergroup sg-1 hides under the arithmetic of supergroup sg
-    auto red_write = [&](const float *part) {
-#pragma unroll
-        for (int k = 0; k < 8; k++)
-            myred[lane * 9 + k] = part[k];
-    };
-    auto red_read = [&](float *tmp) {
-#pragma unroll
-        for (int r = 0; r < 8; r++)
-            tmp[r] = myred[(g8 * 8 + r) * 9 + tk];
-    };
-    auto red_finish = [&](const float *tmp, int sg, int ntok) {
-        float s = ((tmp[0] + tmp[1]) + (tmp[2] + tmp[3])) + ((tmp[4] + tmp[5]) + (tmp[6] + tmp[7]));
-        s = xor8_add(s);
-        s = xor16_add(s);
-        if (G::LPH == 64)
-            s = xor32_add(s);
-        if (active && lh < 8 && tk < ntok)
+    // the token whose total this lane's quad ends up with, and the one lane per token that stores
+    // it (a 64-lane head holds every total twice, once per half)
+    const int tk = token_of_lane(lane);
+    const bool storer = active && (lane & 3) == 0 && (G::LPH == 32 || lane < 32);
+    auto finish = [&](const float *part, int sg, int ntok) {
+        const float s = reduce8_head<G::LPH>(part);
+        if (storer && tk < ntok)
             ob[sg * 8 + tk] = (h1)s;
     };
 
     // ---- software pipeline over the full supergroups.  Global loads run PF supergroups ahead.
     // Table lookups run one supergroup ahead and are issued token by token between the arithmetic
     // of the current supergroup (the LDS counter holds only 15 outstanding operations, so issuing a
-    // whole supergroup's lookups at once would stall on them).  The logit reduction of supergroup
-    // sg-1 is read at the start of iteration sg and finished a few tokens into it.
+    // whole supergroup's lookups at once would stall on them).  The logits of supergroup sg-1 are
+    // reduced and stored at the start of iteration sg, while the first lookups are in flight.
     // The lookup for the next supergroup goes into the slot the current token has just vacated, so
     // one supergroup's worth of registers holds both.
     auto token = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2], float &out_t) {
-        float acc = 0.0f;
+        float acc;
 #pragma unroll
         for (int p = 0; p < G::NP; p++) {
             Pair &s = st[p];
             const h2 qs = as_h2(e[p][t].x) * s.sc;
-            acc = __builtin_amdgcn_fdot2(qv[p], qs + s.zp, acc, false);
+            const h2 kh = qs + s.zp;
+            if (p == 0)
+                acc = dot2_from_zero(qv[p], kh);
+            else
+                acc = __builtin_amdgcn_fdot2(qv[p], kh, acc, false);
             update_pair_abs(s, as_h2(e[p][t].y), qs);
         }
         out_t = acc;
@@ -705,6 +761,7 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
     Vec buf[PF][G::NV];
     uint2 lk[G::NP][8];
     uint32_t nb[G::NP][2];
+    float part[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < PF; i++) {
 #pragma unroll
@@ -724,10 +781,8 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
     // reduction of the previous supergroup stores nothing when there is none (sg == 0).
     auto body = [&](int sg, auto ic) {
         constexpr int i = decltype(ic)::value;
-        float tmp[8], part[8];
         // bytes of supergroup sg+1 (stale data past the end: looked up, never used)
         pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
-        red_read(tmp);
         {
             // unconditional, clamped to the segment's last supergroup: a load inside a branch
             // makes the next wait cover every load in flight, this one included
@@ -737,21 +792,15 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
                 buf[i][v] = cb[(size_t)sgp * G::VPS + v];
         }
         __builtin_amdgcn_sched_barrier(0);
+        finish(part, sg - 1, sg > 0 ? 8 : 0);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int t = 0; t < 3; t++)
+        for (int t = 0; t < 8; t++)
             token(t, lk, nb, part[t]);
-        red_finish(tmp, sg - 1, sg > 0 ? 8 : 0); // early, so tmp[] is dead while part[] fills up
-#pragma unroll
-        for (int t = 3; t < 8; t++)
-            token(t, lk, nb, part[t]);
-        red_write(part);
     };
     rotate_over<PF>(nfull, body);
-    if (nfull > 0) {
-        float tmp[8];
-        red_read(tmp);
-        red_finish(tmp, nfull - 1, 8);
-    }
+    if (nfull > 0)
+        finish(part, nfull - 1, 8);
     if (!last)
         return;
 
@@ -780,10 +829,7 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
                 }
             }
         }
-        float tmp[8];
-        red_write(part);
-        red_read(tmp);
-        red_finish(tmp, nfull, ntail);
+        finish(part, nfull, ntail);
     }
 
     if (active)
