@@ -262,6 +262,24 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
 // ---------------------------------------------------------------------------------------------
 // forward_ov  (gemv.cu:946-1178), per-head table
 // ---------------------------------------------------------------------------------------------
+//
+// MM: the contraction runs on the matrix cores.  v_mfma_f32_4x4x4_16B_f16 multiplies, in each group
+// of four lanes, the 4x4 matrix whose row i is lane i's A operand with the matrix whose column r is
+// lane r's B operand, and lane r receives column r of the product.  With
+//   B of lane r = (x_A[t], x_B[t], x_A[t+1], x_B[t+1])   the lane's channel pair at two tokens, which
+//                                                        is two consecutive registers as they are,
+//   A of lane 0 = (w[t], 0, w[t+1], 0),  A of lane 1 = (0, w[t], 0, w[t+1]),  A of lanes 2, 3 = 0,
+// element 0 of the lane's result is sum w*x_A and element 1 is sum w*x_B: the lane's own two
+// outputs, nothing crosses lanes.  Because the product is linear, the dequantised value q*sc + zp
+// is never formed: one instruction takes the (q*sc) registers of the two tokens, a second one the
+// two zero-points, both accumulate into the same four registers.  That removes the packed add and
+// the two mixed-precision multiply-adds per (pair, token) from the vector pipe (7 -> 4
+// instructions); the 16 matrix instructions per supergroup ride beside the vector ones (measured:
+// up to 4 per 16 packed instructions cost nothing with four waves per SIMD).  The weights reach the
+// A layout with two v_perm_b32 per token pair and per-lane selectors.  A non-finite cached value
+// makes both outputs of its channel PAIR non-finite (0 * inf inside the product); the vector form
+// confines it to its own channel.
+template <bool MM>
 __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
     const h1 *__restrict__ attn, uint4 *__restrict__ cache, const h1 *__restrict__ v_new,
     h1 *__restrict__ out, float *__restrict__ partial,
@@ -286,10 +304,18 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
 
     Pair st[G::NP];
     float acc[CPL];
+    f4v acc4[G::NP];
     ft_init_pairs(st, zp, sc, al, h, bx, c0, un.seg, sa);
 #pragma unroll
     for (int c = 0; c < CPL; c++)
         acc[c] = 0.0f;
+#pragma unroll
+    for (int p = 0; p < G::NP; p++)
+        acc4[p] = (f4v){0.0f, 0.0f, 0.0f, 0.0f};
+    // selectors that turn the word (w[t], w[t+1]) into this lane's two A registers
+    const int role = threadIdx.x & 3;
+    const uint32_t sel_a0 = role == 0 ? 0x0C0C0100u : role == 1 ? 0x01000C0Cu : 0x0C0C0C0Cu;
+    const uint32_t sel_a1 = role == 0 ? 0x0C0C0302u : role == 1 ? 0x03020C0Cu : 0x0C0C0C0Cu;
 
     const int t0 = un.seg * sa.seg_tokens;
     const int t1 = last ? T : t0 + sa.seg_tokens;
@@ -323,6 +349,37 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
         __builtin_amdgcn_sched_barrier(0);
     };
 
+    // two tokens of the current supergroup on the matrix cores, then the lookups of the same two
+    // slots of the next one
+    auto token2 = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2], const uint4 wv) {
+        const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+        const uint32_t w2 = ww[t >> 1];
+        const h4v a = as_h4(__builtin_amdgcn_perm(w2, w2, sel_a0), __builtin_amdgcn_perm(w2, w2, sel_a1));
+        uint32_t qs[G::NP][2], z[G::NP][2];
+#pragma unroll
+        for (int k = 0; k < 2; k++)
+#pragma unroll
+            for (int p = 0; p < G::NP; p++) {
+                Pair &s = st[p];
+                const h2 x = as_h2(e[p][t + k].x) * s.sc;
+                qs[p][k] = as_u32(x);
+                z[p][k] = as_u32(s.zp);
+                update_pair_f(s, as_h2(e[p][t + k].y), x);
+            }
+#pragma unroll
+        for (int p = 0; p < G::NP; p++)
+            acc4[p] = __builtin_amdgcn_mfma_f32_4x4x4f16(a, as_h4(qs[p][0], qs[p][1]), acc4[p], 0, 0, 0);
+#pragma unroll
+        for (int p = 0; p < G::NP; p++)
+            acc4[p] = __builtin_amdgcn_mfma_f32_4x4x4f16(a, as_h4(z[p][0], z[p][1]), acc4[p], 0, 0, 0);
+#pragma unroll
+        for (int k = 0; k < 2; k++)
+#pragma unroll
+            for (int p = 0; p < G::NP; p++)
+                e[p][t + k] = ft_get(tab, nb[p][(t + k) & 1], lane_copy, (t + k) >> 1, p);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
     uint4 buf[PF][1];
     uint4 wbuf[PF];
     uint2 lk[G::NP][8];
@@ -346,12 +403,25 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
         const int sgp = min(sg + PF, nfull - 1);
         buf[i][0] = cb[(size_t)sgp * G::VPS];
         __builtin_amdgcn_sched_barrier(0);
+        if (MM) {
 #pragma unroll
-        for (int t = 0; t < 8; t++)
-            token(t, lk, nb, wbuf[i]);
+            for (int t = 0; t < 8; t += 2)
+                token2(t, lk, nb, wbuf[i]);
+        } else {
+#pragma unroll
+            for (int t = 0; t < 8; t++)
+                token(t, lk, nb, wbuf[i]);
+        }
         wbuf[i] = load_w(sgp); // reloaded once its last token is done (see ov_kernel)
     };
     rotate_over<PF>(nfull, body);
+    if (MM) {
+#pragma unroll
+        for (int p = 0; p < G::NP; p++) {
+            acc[2 * p] = acc4[p].x;
+            acc[2 * p + 1] = acc4[p].y;
+        }
+    }
 
     if (last) {
         ft_load_beta(st, be, tg, h, c0);

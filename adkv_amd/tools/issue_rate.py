@@ -1,6 +1,8 @@
 """Builds and runs the vector-instruction issue-rate microbenchmark (issue_rate.hip) on cuda:0.
 
     python -m adkv_amd.tools.issue_rate            # build if needed, run, print the table
+    python -m adkv_amd.tools.issue_rate --all      # plus a survey of 32-bit and scalar-f16 forms at 4 and 8 waves
+    python -m adkv_amd.tools.issue_rate --mfma     # matrix-core instructions interleaved with packed vector arithmetic
     python -m adkv_amd.tools.issue_rate --build    # build only (hipcc cross-compiles without a GPU)
 """
 from __future__ import annotations
@@ -28,7 +30,7 @@ def main(argv=None):
     if "--build" in argv:
         print(exe)
         return 0
-    return subprocess.call([exe])
+    return subprocess.call([exe] + [a for a in argv if a in ("--all", "--mfma")])
 
 
 if __name__ == "__main__":
