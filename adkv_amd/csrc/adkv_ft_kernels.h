@@ -80,7 +80,23 @@ __device__ __forceinline__ uint2 ft_get(const uint2 *tab, uint32_t bytes, uint32
     // [0, j, bytes.byte[k], lane*8]: selector bytes 0-3 pick from lane_copy, 4-7 from bytes, 0x0C is zero
     const uint32_t sel = (j ? 0x0C010000u : 0x0C0C0000u) | ((4u + (uint32_t)k) << 8);
     const uint32_t addr = __builtin_amdgcn_perm(bytes, lane_copy, sel);
+#ifdef ADKV_ABLATE_NO_LOOKUP
+    return make_uint2(addr | 0x3c003c00u, 0x3c003c00u); // timing only: no LDS read, results are wrong
+#else
     return *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(tab) + addr);
+#endif
+}
+
+// Which supergroup the main loops prefetch.  ADKV_ABLATE_CODE_WINDOW=m (a measurement aid, see
+// tools/ablate.py; results are wrong) keeps every unit inside its first m+1 supergroups, so the
+// same instruction stream runs with its code bytes coming from a cache instead of from HBM.
+__device__ __forceinline__ int ft_prefetch_index(int sg, int nfull)
+{
+#ifdef ADKV_ABLATE_CODE_WINDOW
+    return min(sg & (ADKV_ABLATE_CODE_WINDOW), nfull - 1);
+#else
+    return min(sg + PF, nfull - 1);
+#endif
 }
 
 // The main loop needs zp, sc and alpha only (the table holds what beta and the target give); the
@@ -208,7 +224,7 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
     auto body = [&](int sg, auto ic) {
         constexpr int i = decltype(ic)::value;
         pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
-        buf[i][0] = cb[(size_t)min(sg + PF, nfull - 1) * G::VPS];
+        buf[i][0] = cb[(size_t)ft_prefetch_index(sg, nfull) * G::VPS];
         __builtin_amdgcn_sched_barrier(0);
         finish(part, sg - 1, sg > 0 ? 8 : 0);
         __builtin_amdgcn_sched_barrier(0);
@@ -400,7 +416,7 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
     auto body = [&](int sg, auto ic) {
         constexpr int i = decltype(ic)::value;
         pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
-        const int sgp = min(sg + PF, nfull - 1);
+        const int sgp = ft_prefetch_index(sg, nfull);
         buf[i][0] = cb[(size_t)sgp * G::VPS];
         __builtin_amdgcn_sched_barrier(0);
         if (MM) {

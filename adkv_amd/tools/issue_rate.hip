@@ -1,5 +1,5 @@
 // Vector-instruction issue rates on gfx950, the numbers the decode kernels' instruction budget is
-// priced with.  Each kernel runs ITER iterations of 16 independent instances of ONE instruction per
+// priced with.  Each kernel runs ITER rounds of 16 independent instances of ONE instruction per
 // wave (256-thread workgroups, 256 * waves-per-SIMD of them so that every SIMD of the 256 CUs holds
 // that many waves); the table gives nanoseconds per instruction per SIMD and, from wave 0's
 // cycle counter, shader-clock ticks per instruction.
@@ -9,6 +9,12 @@
 #include <stdint.h>
 #include <stdio.h>
 #define ITER 4096
+// The timed loops are unrolled UNR times: a taken branch costs the wave that takes it some 20 cycles
+// of issue, which with 16 instructions per trip and four waves per SIMD reads as 2.28 ns per packed
+// instruction where the pipe itself takes 1.77 ns (4 cycles at 2.26 GHz).  -DUNR=1 shows that.
+#ifndef UNR
+#define UNR 8
+#endif
 #define REP16(X) X(0) X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(9) X(10) X(11) X(12) X(13) X(14) X(15)
 
 #define KERNEL(NAME, ASM) \
@@ -16,8 +22,10 @@ __global__ __launch_bounds__(1024) void NAME(uint32_t* out, uint32_t seed) { \
     uint32_t r[16]; uint32_t a = seed + threadIdx.x, b = seed * 3 + 1, c = seed ^ 0x3c003c00; \
     for (int i = 0; i < 16; i++) r[i] = seed + i; \
     unsigned long long t0 = clock64(); \
-    for (int it = 0; it < ITER; it++) { \
-        _Pragma("unroll") for (int i = 0; i < 16; i++) asm volatile(ASM : "+v"(r[i]) : "v"(a), "v"(b), "v"(c)); \
+    for (int it = 0; it < ITER / UNR; it++) { \
+        _Pragma("unroll") for (int u = 0; u < UNR; u++) { \
+            _Pragma("unroll") for (int i = 0; i < 16; i++) asm volatile(ASM : "+v"(r[i]) : "v"(a), "v"(b), "v"(c)); \
+        } \
     } \
     unsigned long long t1 = clock64(); \
     uint32_t s = 0; for (int i = 0; i < 16; i++) s ^= r[i]; \
@@ -76,9 +84,11 @@ __global__ __launch_bounds__(1024) void k_lds64(uint32_t* out, uint32_t seed) {
     __syncthreads();
     uint32_t addr = ((threadIdx.x * 2654435761u + seed) & 0xFF00u) | ((threadIdx.x & 31) << 3);
     uint2 r[16];
-    for (int it = 0; it < ITER; it++) {
-        _Pragma("unroll") for (int i = 0; i < 16; i++) asm volatile("ds_read_b64 %0, %1" : "=v"(r[i]) : "v"(addr));
-        asm volatile("s_waitcnt lgkmcnt(0)");
+    for (int it = 0; it < ITER / UNR; it++) {
+        _Pragma("unroll") for (int u = 0; u < UNR; u++) {
+            _Pragma("unroll") for (int i = 0; i < 16; i++) asm volatile("ds_read_b64 %0, %1" : "=v"(r[i]) : "v"(addr));
+            asm volatile("s_waitcnt lgkmcnt(0)");
+        }
     }
     uint32_t s = 0; for (int i = 0; i < 16; i++) s ^= r[i].x ^ r[i].y;
     if (s == 0x12345) out[threadIdx.x] = s;
@@ -98,7 +108,8 @@ __global__ __launch_bounds__(1024) void k_mix(uint32_t* out, uint32_t seed) {
     f16x4 ma = {(_Float16)1, (_Float16)2, (_Float16)(int)(seed & 3), (_Float16)0.5f}, mb = ma;
     constexpr int N = NV > NM ? NV : NM;
     unsigned long long t0 = clock64();
-    for (int it = 0; it < ITER; it++) {
+    for (int it = 0; it < ITER / UNR; it++) {
+        _Pragma("unroll") for (int u = 0; u < UNR; u++)
         _Pragma("unroll") for (int i = 0; i < N; i++) {
             if (i * NV / N != (i + 1) * NV / N)
                 asm volatile("v_pk_fma_f16 %0, %1, %2, %3" : "+v"(r[i & 15]) : "v"(a), "v"(b), "v"(c));
