@@ -34,6 +34,11 @@ namespace adkv {
 #define ADKV_PF 4
 #endif
 constexpr int PF = ADKV_PF; // supergroups in flight per lane
+// 1: the per-head-table OV kernel contracts on the matrix cores; 0 builds its vector form instead
+// (a measurement aid for tools/ablate.py, not compiled into the shipped library).
+#ifndef ADKV_FT_OV_MM
+#define ADKV_FT_OV_MM 1
+#endif
 #ifndef ADKV_MFMA_DEFAULT
 #define ADKV_MFMA_DEFAULT 0
 #endif
@@ -1532,17 +1537,6 @@ static bool use_head_table(int B, int H, int GQ, int bits, int D, const Seg &seg
     return padded_waves * 100 <= waves * 106;
 }
 
-// Whether the per-head-table kernels contract on the matrix cores (ADKV_FT_MM=0 keeps the vector
-// form, a measurement aid); read once.
-static bool ft_matrix_cores()
-{
-    static const bool on = [] {
-        const char *e = getenv("ADKV_FT_MM");
-        return e ? atoi(e) != 0 : true;
-    }();
-    return on;
-}
-
 // ADKV_ENCODE_CPL=1/2 pins the encoder's channels per lane (a measurement aid); read once.
 static int encode_cpl_override()
 {
@@ -1960,16 +1954,10 @@ static int forward_ov_impl(const void *attn, void *v_cache, const void *v_new, v
                          (const h1 *)alpha, (const h1 *)beta, (const h1 *)tgt, BH, H, T, n_super_cap,
                          (h1 *)state_out, seg);
     } else if (use_head_table(B, H, GQ, bits, D, seg)) {
-        if (ft_matrix_cores())
-            hipLaunchKernelGGL(ov_ft_kernel<true>, dim3((unsigned)(H * ft_wgs_per_head(B, seg.nseg))), dim3(FT_BLK), 0, st,
-                               (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new, (h1 *)out,
-                               (float *)workspace, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,
-                               (const h1 *)beta, (const h1 *)tgt, B, H, T, n_super_cap, (h1 *)state_out, seg);
-        else
-            hipLaunchKernelGGL(ov_ft_kernel<false>, dim3((unsigned)(H * ft_wgs_per_head(B, seg.nseg))), dim3(FT_BLK), 0, st,
-                               (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new, (h1 *)out,
-                               (float *)workspace, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,
-                               (const h1 *)beta, (const h1 *)tgt, B, H, T, n_super_cap, (h1 *)state_out, seg);
+        hipLaunchKernelGGL(ov_ft_kernel<ADKV_FT_OV_MM != 0>, dim3((unsigned)(H * ft_wgs_per_head(B, seg.nseg))),
+                           dim3(FT_BLK), 0, st, (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new, (h1 *)out,
+                           (float *)workspace, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,
+                           (const h1 *)beta, (const h1 *)tgt, B, H, T, n_super_cap, (h1 *)state_out, seg);
     } else {
         ADKV_DISPATCH_D(ov_kernel, (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new, (h1 *)out,
                         (float *)workspace, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,

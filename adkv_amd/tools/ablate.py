@@ -1,7 +1,8 @@
 """What the per-head-table decode kernels wait for, measured by taking things away.
 
 Builds the library several times from the committed sources with measurement-only macros
-(adkv_ft_kernels.h: ADKV_ABLATE_NO_LOOKUP skips the LDS table reads, ADKV_ABLATE_CODE_WINDOW=m
+(ADKV_FT_OV_MM=0 gives the OV kernel's vector contraction back; adkv_ft_kernels.h:
+ADKV_ABLATE_NO_LOOKUP skips the LDS table reads, ADKV_ABLATE_CODE_WINDOW=m
 keeps every unit's code prefetch inside its first m+1 supergroups, so the bytes come from L1 / L2 /
 the memory-side cache instead of HBM), then runs the cfg2 decode step (B=128, 32 heads x 128,
 ctx 4096, 4-bit, checkpoints every 256 tokens) with each build in a process of its own and prints
@@ -23,7 +24,7 @@ _DIR = os.path.dirname(os.path.abspath(__file__))
 OUT = os.path.join(_DIR, "_ablate")
 VARIANTS = [
     ("as shipped", []),
-    ("vector contraction in OV", None),                       # same library, ADKV_FT_MM=0
+    ("vector contraction in OV", ["-DADKV_FT_OV_MM=0"]),
     ("no table lookups", ["-DADKV_ABLATE_NO_LOOKUP"]),
     ("codes from L1 (2 supergroups per unit)", ["-DADKV_ABLATE_CODE_WINDOW=1"]),
     ("codes from L2 (4 per unit)", ["-DADKV_ABLATE_CODE_WINDOW=3"]),
@@ -43,8 +44,6 @@ def build_variants() -> None:
 
     def one(i):
         flags = VARIANTS[i][1]
-        if flags is None:
-            return
         subprocess.run([hipcc, *_build.HIPCC_FLAGS, *flags, "-o", _path(i), *_build.SOURCES],
                        check=True, capture_output=True)
 
@@ -121,8 +120,6 @@ def main(argv=None) -> int:
     for i, (name, flags) in enumerate(VARIANTS + [VARIANTS[0]]):
         env = dict(os.environ)
         env["ADKV_ABLATE_LIB"] = _build.LIB_PATH if not flags else _path(i)
-        if flags is None:
-            env["ADKV_FT_MM"] = "0"
         r = subprocess.run([sys.executable, "-m", "adkv_amd.tools.ablate", "--child"], env=env,
                            capture_output=True, text=True, timeout=300)
         if r.returncode != 0:
