@@ -498,7 +498,21 @@ def main():
             # known size; kept beside the profile it came from (profiles/hbm_traffic.json)
             "traffic": traffic,
         },
+        # the second big launch of the step, same algorithmic bytes (the V codes)
+        "roofline_ov": {"kernel": "ov_" + kernel, "bound": "hbm", "achieved": code_bytes / (ov_ms * 1e-3) / 1e9,
+                        "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": code_bytes / (ov_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                        "note": "forward_ov stage incl. the partial-sum kernel"},
     }
+    # what the memory system itself delivers for these kernels' access pattern with nothing else
+    # running (tools/hbm_streams, recorded in profiles/hbm_pattern_ceiling.json)
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_pattern_ceiling.json")) as f:
+            ceil = next(iter(json.load(f).values()))
+        res["roofline"]["pattern_ceiling"] = {"GBps": ceil["best_GBps"], "frac_of_peak": ceil["best_GBps"] / HBM_PEAK_GBPS,
+                                              "achieved_over_ceiling": achieved / ceil["best_GBps"],
+                                              "note": "loads only, same access pattern: python -m adkv_amd.tools.hbm_streams"}
+    except (OSError, ValueError, StopIteration, KeyError):
+        pass
     if graph_ms is not None:
         res["graph_replay"] = {"ms_per_step": graph_ms, "tokens_per_s": B / (N_LAYERS_MODEL * graph_ms * 1e-3),
                                "note": "the same decode_step step captured once per layer cache and replayed"}
