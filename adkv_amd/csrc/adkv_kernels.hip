@@ -1265,23 +1265,66 @@ __device__ __forceinline__ float2 softmax_wave_merge(float2 v)
     return v;
 }
 
+// SUB chunks per workgroup.  With SUB > 1 and every chunk inside the row, all of the workgroup's
+// loads are issued before anything waits for one (a 256-thread workgroup that fetches 12 KB and
+// leaves is mostly launch and latency: 3.0 TB/s over the 512 rows of 131 073 logits of the
+// long-context shape; 48 KB per workgroup: see the kernel trace of that shape); the merged pair
+// goes to the first chunk's slot and the other slots get the neutral element.
+template <int SUB>
 __global__ __launch_bounds__(SM_BLOCK) void softmax_part_kernel(
     const h1 *__restrict__ logits, const float *__restrict__ mask, float2 *__restrict__ part,
     int n, long ld, int nchunk, int rows_per_mask_row, float scaling)
 {
     __shared__ float2 sm[SM_BLOCK / 64];
-    const int row = blockIdx.y, ck = blockIdx.x;
+    const int row = blockIdx.y, ck0 = blockIdx.x * SUB;
     const h1 *l = logits + (size_t)row * ld;
     const float *mk = mask ? mask + (size_t)(row / rows_per_mask_row) * n : nullptr;
-    float x[SM_KEEP], mx;
-    softmax_load_chunk(l, mk, n, ck * SM_CHUNK, scaling, x, mx);
-    // the thread's own (max, sum), then ONE reduction of pairs over the workgroup
-    float sum = 0.0f;
-    if (mx > -INFINITY) {
+    float mx = -INFINITY, sum = 0.0f;
+    if (SUB > 1 && !mk && (ck0 + SUB) * SM_CHUNK <= n) {
+        uint4 raw[SUB][SM_NV];
 #pragma unroll
-        for (int k = 0; k < SM_KEEP; k++)
-            sum += __expf(x[k] - mx);
+        for (int s = 0; s < SUB; s++)
+#pragma unroll
+            for (int v = 0; v < SM_NV; v++)
+                __builtin_memcpy(&raw[s][v], l + (size_t)(ck0 + s) * SM_CHUNK + (v * SM_BLOCK + threadIdx.x) * SM_VEC, 16);
+        float x[SUB][SM_KEEP];
+#pragma unroll
+        for (int s = 0; s < SUB; s++)
+#pragma unroll
+            for (int v = 0; v < SM_NV; v++) {
+                const uint32_t w[4] = {raw[s][v].x, raw[s][v].y, raw[s][v].z, raw[s][v].w};
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const h2 p = as_h2(w[k]);
+                    x[s][v * SM_VEC + 2 * k] = (float)p.x * scaling;
+                    x[s][v * SM_VEC + 2 * k + 1] = (float)p.y * scaling;
+                    mx = fmaxf(mx, fmaxf(x[s][v * SM_VEC + 2 * k], x[s][v * SM_VEC + 2 * k + 1]));
+                }
+            }
+        if (mx > -INFINITY) {
+#pragma unroll
+            for (int s = 0; s < SUB; s++)
+#pragma unroll
+                for (int k = 0; k < SM_KEEP; k++)
+                    sum += __expf(x[s][k] - mx);
+        }
+    } else {
+        // the generic way, a chunk at a time (chunks past the end of the row are all -inf)
+        for (int s = 0; s < SUB; s++) {
+            float x[SM_KEEP], m1;
+            softmax_load_chunk(l, mk, n, (ck0 + s) * SM_CHUNK, scaling, x, m1);
+            float s1 = 0.0f;
+            if (m1 > -INFINITY) {
+#pragma unroll
+                for (int k = 0; k < SM_KEEP; k++)
+                    s1 += __expf(x[k] - m1);
+            }
+            const float2 r = softmax_merge(make_float2(mx, sum), make_float2(m1, s1));
+            mx = r.x;
+            sum = r.y;
+        }
     }
+    // the thread's own (max, sum), then ONE reduction of pairs over the workgroup
     const float2 w = softmax_wave_merge(make_float2(mx, sum));
     if ((threadIdx.x & 63) == 0)
         sm[threadIdx.x >> 6] = w;
@@ -1291,8 +1334,10 @@ __global__ __launch_bounds__(SM_BLOCK) void softmax_part_kernel(
 #pragma unroll
         for (int i = 1; i < SM_BLOCK / 64; i++)
             r = softmax_merge(r, sm[i]);
-        part[(size_t)row * nchunk + ck] = r;
+        part[(size_t)row * nchunk + ck0] = r;
     }
+    if (threadIdx.x > 0 && threadIdx.x < SUB && ck0 + (int)threadIdx.x < nchunk)
+        part[(size_t)row * nchunk + ck0 + threadIdx.x] = make_float2(-INFINITY, 0.0f);
 }
 
 __global__ __launch_bounds__(SM_BLOCK) void softmax_norm_kernel(
@@ -2150,9 +2195,17 @@ int adkv_softmax_ex(const void *logits, void *weights, const void *mask,
         return ADKV_E_ALIGN;
     const int nchunk = (n + SM_CHUNK - 1) / SM_CHUNK;
     const dim3 grid((unsigned)nchunk, (unsigned)rows);
-    hipLaunchKernelGGL(softmax_part_kernel, grid, dim3(SM_BLOCK), 0, (hipStream_t)stream,
-                       (const h1 *)logits, (const float *)mask, (float2 *)workspace, n, (long)ld, nchunk,
-                       mask ? rows_per_mask_row : 1, scaling);
+    if (nchunk >= 8 && !mask) {
+        // long rows: four chunks per workgroup in the first pass
+        const dim3 grid4((unsigned)((nchunk + 3) / 4), (unsigned)rows);
+        hipLaunchKernelGGL(softmax_part_kernel<4>, grid4, dim3(SM_BLOCK), 0, (hipStream_t)stream,
+                           (const h1 *)logits, (const float *)mask, (float2 *)workspace, n, (long)ld, nchunk,
+                           1, scaling);
+    } else {
+        hipLaunchKernelGGL(softmax_part_kernel<1>, grid, dim3(SM_BLOCK), 0, (hipStream_t)stream,
+                           (const h1 *)logits, (const float *)mask, (float2 *)workspace, n, (long)ld, nchunk,
+                           mask ? rows_per_mask_row : 1, scaling);
+    }
     hipLaunchKernelGGL(softmax_norm_kernel, grid, dim3(SM_BLOCK), 0, (hipStream_t)stream,
                        (const h1 *)logits, (h1 *)weights, (const float *)mask,
                        (const float2 *)workspace, n, (long)ld, nchunk, mask ? rows_per_mask_row : 1,

@@ -107,7 +107,11 @@ def test_forward_qk_and_ov(gpu, oracle, B, H, T, D):
 
 
 @pytest.mark.parametrize("rows,n,mask_mode", [(6, 1, None), (6, 130, None), (8, 4097, "b1"), (8, 257, "bh"),
-                                              (4, 5121, None), (6, 20000, "b1"), (2, 131073, "bh")])
+                                              (4, 5121, None), (6, 20000, "b1"), (2, 131073, "bh"),
+                                              # long unmasked rows: four chunks per workgroup in the first
+                                              # pass (all inside the row / last group ragged / one group only)
+                                              (4, 131073, None), (2, 60000, None), (2, 49152, None),
+                                              (2, 49153, None)])
 def test_softmax(gpu, rows, n, mask_mode):
     g = torch.Generator().manual_seed(n)
     B, H = 2, rows // 2
