@@ -13,8 +13,9 @@
 //     32 lanes of a head read 32 distinct 8-byte slots of one 256-byte row whatever their codes
 //     are, and the address is still ONE v_perm_b32: [0, table, code byte, lane*8].
 //   * All 32 (sequence, segment) units of a workgroup must belong to the SAME head: units are
-//     ordered head-major (for one head: segment-major, then sequence pairs), and every head's run
-//     of waves is padded to whole 16-wave workgroups.
+//     ordered head-major (for one head: a wave per pair of sequences and segment, consecutive
+//     quads of waves on different segments, interleave_segment), and every head's run of waves is padded
+//     to whole 16-wave workgroups.
 //   * No LDS is left for the logit transpose of qk_kernel, and none is needed: the 8 per-lane
 //     partials are reduced and scattered over the head's 32 lanes with bank-masked DPP adds
 //     (8 + 4 instructions), one row swap and two quad permutes.
@@ -30,7 +31,7 @@ constexpr int FT_TABLE_WORDS64 = 2 * LUT_ENTRIES * 32; // uint2 elements: 2 x 64
 __host__ __device__ inline int ft_pairs_per_seg(int B) { return (B + 1) >> 1; }
 __host__ __device__ inline int ft_wgs_per_head(int B, int nseg)
 {
-    return (nseg * ft_pairs_per_seg(B) + FT_WAVES - 1) / FT_WAVES;
+    return (nseg * pad4(ft_pairs_per_seg(B)) + FT_WAVES - 1) / FT_WAVES;
 }
 
 struct FtUnit {
@@ -41,15 +42,17 @@ struct FtUnit {
         const int pps = ft_pairs_per_seg(B);
         const int wph = ft_wgs_per_head(B, nseg);
         h = (int)blockIdx.x / wph;
-        const int w = ((int)blockIdx.x % wph) * FT_WAVES + (int)(threadIdx.x >> 6); // wave within the head
-        const int sg = __builtin_amdgcn_readfirstlane(w / pps);
+        const int w = __builtin_amdgcn_readfirstlane(((int)blockIdx.x % wph) * FT_WAVES +
+                                                     (int)(threadIdx.x >> 6)); // wave within the head
+        int sg, pair;
+        interleave_segment(w, nseg, sg, pair);
         const int lane = threadIdx.x & 63;
-        const int b = (w % pps) * 2 + (lane >> 5);
+        const int b = pair * 2 + (lane >> 5);
         lh = lane & 31;
         c0 = lh * 4;
-        wave_active = sg < nseg;
+        wave_active = pair < pps;
         active = wave_active && b < B;
-        seg = sg < nseg ? sg : nseg - 1;
+        seg = sg;
         bx = (b < B ? b : B - 1) * H + h;
     }
 };

@@ -153,6 +153,8 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
     uint2 *tile = smem + LUT_WORDS64 + (threadIdx.x >> 6) * TILE_WORDS64;
 
     const Unit<D, CPL, BLK> un(BH, sa.nseg);
+    if (!un.wave_active)
+        return; // padding waves
     const int bx = un.bx, lh = un.lh, c0 = un.c0;
     const bool active = un.active;
     const bool last = un.seg == sa.nseg - 1;
@@ -338,6 +340,8 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
     const uint32_t lane_copy = table_lane_offset<BITS>(lane);
 
     const Unit<D, CPL, BLK> un(BH, sa.nseg);
+    if (!un.wave_active)
+        return; // padding waves
     const int bx = un.bx, lh = un.lh, c0 = un.c0;
     const bool active = un.active;
     const bool last = un.seg == sa.nseg - 1;

@@ -235,34 +235,58 @@ __device__ __forceinline__ void store_state_n(h1 *dst, const Pair *st)
         *reinterpret_cast<h2 *>(dst) = (h2){st[0].zp.x, st[0].sc.x};
 }
 
-// Which (head, segment) this lane works on.  Units are ordered segment-major and every segment's
-// run of units is padded to whole waves, so all lanes of a wave work on the same segment and
-// everything derived from it (token range, trip counts) is wave-uniform: the decode loops then
-// branch on scalars instead of masking lanes.  Units past the end are clamped to a valid one and
-// flagged inactive: they compute but never store.
+// Which (head, segment) this lane works on.  Every segment's run of units is padded to whole
+// waves, so all lanes of a wave work on the same segment and everything derived from it (token
+// range, trip counts) is wave-uniform: the decode loops then branch on scalars instead of masking
+// lanes.  Units past the end are clamped to a valid one and flagged inactive: they compute but
+// never store.
+//
+// Consecutive waves take DIFFERENT segments of the same sequences (interleave_segment): the last
+// segment of a context is shorter than the others whenever the length is not a multiple of the
+// segment size (a 640-token context cut at 512 is a 512-token and a 128-token segment), and with
+// all short waves in one workgroup and all long ones in another, half the CUs went idle after a
+// quarter of the launch (B=128: 640 tokens took as long as 1024).  Mixed, every SIMD holds long
+// and short waves and the long ones speed up when the short ones leave (two waves issue nearly as
+// fast as four).
+//
+// wave index -> (segment, wave within the segment).  A wave's SIMD is its index modulo 4 (a
+// workgroup's waves go round the SIMDs), so the mapping works on quads of waves: quad q takes
+// segment q mod nseg, and its four waves are four consecutive waves' worth of units of that
+// segment; every SIMD then walks through the segments in turn.  Each segment's waves are padded
+// to a multiple of four (pad4); padding waves leave right after the table is built.
+__host__ __device__ inline int pad4(int n) { return (n + 3) & ~3; }
+__host__ __device__ inline void interleave_segment(int wave, int nseg, int &seg, int &wave_in_seg)
+{
+    const int q = wave >> 2, g = q / nseg;
+    seg = q - g * nseg;
+    wave_in_seg = g * 4 + (wave & 3);
+}
+
 template <int LPH>
 static inline long padded_units(int BH, int nseg)
 {
     constexpr int UPW = 64 / LPH; // units per wave
-    return (long)nseg * (((long)BH + UPW - 1) / UPW * UPW);
+    return (long)nseg * pad4((BH + UPW - 1) / UPW) * UPW;
 }
 
 template <int D, int CPL, int BLK>
 struct Unit {
     int bx, seg, lh, c0;
-    bool active;
+    bool active, wave_active;
     __device__ __forceinline__ Unit(int BH, int nseg)
     {
         using G = Geo<D, CPL>;
         constexpr int UPW = 64 / G::LPH;
-        const int per_seg = (BH + UPW - 1) / UPW * UPW;
+        const int waves_per_seg = (BH + UPW - 1) / UPW;
         const long gl = (long)blockIdx.x * BLK + threadIdx.x;
-        const long slot = gl / G::LPH;
         lh = (int)(gl % G::LPH);
-        const int sg = __builtin_amdgcn_readfirstlane((int)(slot / per_seg));
-        const int b = (int)(slot % per_seg);
-        active = sg < nseg && b < BH;
-        seg = sg < nseg ? sg : nseg - 1;
+        const int wave = __builtin_amdgcn_readfirstlane((int)(gl >> 6));
+        int sg, wis;
+        interleave_segment(wave, nseg, sg, wis);
+        const int b = wis * UPW + (int)((gl & 63) / G::LPH);
+        wave_active = wis < waves_per_seg;
+        active = wave_active && b < BH;
+        seg = sg;
         bx = b < BH ? b : BH - 1;
         c0 = lh * CPL;
     }
@@ -707,6 +731,8 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
     const uint32_t lane_copy = (uint32_t)(lane & (LUT_COPIES - 1)) * 8u;
 
     const Unit<D, CPL, BLK> un(BH, sa.nseg);
+    if (!un.wave_active)
+        return; // padding waves
     const int bx = un.bx, lh = un.lh, c0 = un.c0;
     const bool active = un.active;
     const bool last = un.seg == sa.nseg - 1;
@@ -873,6 +899,8 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
     const uint32_t lane_copy = (uint32_t)(threadIdx.x & (LUT_COPIES - 1)) * 8u;
 
     const Unit<D, CPL, BLK> un(BH, sa.nseg);
+    if (!un.wave_active)
+        return; // padding waves
     const int bx = un.bx, lh = un.lh, c0 = un.c0;
     const bool active = un.active;
     const bool last = un.seg == sa.nseg - 1;
