@@ -312,8 +312,13 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
     const FtUnit un(B, H, sa.nseg);
     ft_fill(tab, be, tg, un.h);
     __syncthreads();
-    if (!un.wave_active)
+    if (!un.wave_active) {
+        if (sa.combine) { // the two barriers of the in-workgroup sum below
+            __syncthreads();
+            __syncthreads();
+        }
         return;
+    }
 
     const uint32_t lane_copy = 0x100u | ((uint32_t)un.lh * 8u);
     const int bx = un.bx, lh = un.lh, c0 = un.c0, h = un.h;
@@ -473,9 +478,29 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
             acc[2 * p + 1] = __builtin_fmaf(wT, (float)deq[p].y, acc[2 * p + 1]);
         }
     }
+    if (sa.combine) {
+        // nseg is 2 or 4: the waves holding the other segments of these sequences are 4, 8, 12
+        // waves away in this workgroup (interleave_segment: quad q takes segment q mod nseg).  The
+        // table is finished with once every wave is here; its first 16 KB take the partial sums,
+        // and the wave of segment 0 adds them in segment order (what ov_finalize_kernel does).
+        __syncthreads();
+        float4 *red = reinterpret_cast<float4 *>(tab);
+        const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        red[wv * 64 + lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+        __syncthreads();
+        if (un.seg != 0 || !active)
+            return;
+        for (int s = 1; s < sa.nseg; s++) {
+            const float4 p = red[(wv + 4 * s) * 64 + lane];
+            acc[0] += p.x;
+            acc[1] += p.y;
+            acc[2] += p.z;
+            acc[3] += p.w;
+        }
+    }
     if (!active)
         return;
-    if (sa.nseg == 1) {
+    if (sa.nseg == 1 || sa.combine) {
         h1 *o = out + (size_t)bx * D + c0;
 #pragma unroll
         for (int p = 0; p < G::NP; p++)

@@ -82,6 +82,7 @@ struct Seg {
     int nseg;
     long row_pitch;     // elements between rows of the logits / attention-weight matrix (>= T + 1)
     int act_bf16;       // q, the new token and the output are bfloat16 (see load_act2 / store_act2)
+    int combine;        // ov_ft_kernel: the segments' partial outputs are added inside the workgroup
 };
 
 __device__ __forceinline__ float wave_xor_add(float v, int mask)
@@ -1451,6 +1452,7 @@ static Seg plan_segments(void *ckpt, int n_ckpt_cap, int ckpt_interval, int BH, 
     s.nseg = 1;
     s.row_pitch = T + 1;
     s.act_bf16 = 0;
+    s.combine = 0;
     if (!ckpt || ckpt_interval <= 0 || T <= ckpt_interval)
         return s;
     const int avail = (T + ckpt_interval - 1) / ckpt_interval;               // finest split
@@ -1718,6 +1720,7 @@ static int encode_common(void *cache, const void *kv_new,
     seg.nseg = 1;
     seg.row_pitch = T + 1;
     seg.act_bf16 = 0;
+    seg.combine = 0;
     // Lane width, measured on an MI355X (4096 tokens, ms for 65 536 / 131 072 / 196 608 / 262 144 /
     // 524 288 channels): one channel per lane 0.29 / 0.44 / 0.60 / 0.74 / 1.38, two 0.43 / 0.44 /
     // 0.55 / 0.60 / 1.17, four 0.78 / 0.78 / 0.78 / 0.79 / 1.18.  Up to two waves per SIMD the
@@ -2027,6 +2030,9 @@ static int forward_ov_impl(const void *attn, void *v_cache, const void *v_new, v
                          (const h1 *)alpha, (const h1 *)beta, (const h1 *)tgt, BH, H, T, n_super_cap,
                          (h1 *)state_out, seg);
     } else if (use_head_table(B, H, GQ, bits, D, seg)) {
+        // two or four segments: the waves of one (sequence pair) sit in the same workgroup
+        // (interleave_segment) and add their partial outputs there, no second launch
+        seg.combine = (seg.nseg == 2 || seg.nseg == 4) ? 1 : 0;
         hipLaunchKernelGGL(ov_ft_kernel<ADKV_FT_OV_MM != 0>, dim3((unsigned)(H * ft_wgs_per_head(B, seg.nseg))),
                            dim3(FT_BLK), 0, st, (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new, (h1 *)out,
                            (float *)workspace, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,
@@ -2039,7 +2045,7 @@ static int forward_ov_impl(const void *attn, void *v_cache, const void *v_new, v
     }
     if ((rc = check_launch()))
         return rc;
-    if (seg.nseg > 1) {
+    if (seg.nseg > 1 && !seg.combine) {
         const long n = (long)BH * GQ * D;
         if (seg.nseg > 8)
             hipLaunchKernelGGL(ov_finalize_wide_kernel, dim3((unsigned)((n + 63) / 64)), dim3(256), 0, st,
