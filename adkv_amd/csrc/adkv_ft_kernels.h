@@ -152,10 +152,6 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
     using G = Geo<D, CPL>;
     __shared__ uint2 tab[FT_TABLE_WORDS64]; // the only LDS object: sits at offset 0
     const FtUnit un(B, H, sa.nseg);
-    ft_fill(tab, be, tg, un.h);
-    __syncthreads();
-    if (!un.wave_active)
-        return; // padding waves of the head's last workgroup
 
     const int lane = threadIdx.x & 63;
     const uint32_t lane_copy = 0x100u | ((uint32_t)un.lh * 8u);
@@ -178,6 +174,18 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
     const int nfull = (t1 - t0) >> 3;
     const int tk = token_of_lane(lane);
     const bool storer = active && (lane & 3) == 0;
+
+    // The first code words, like the parameters and the query above, are requested BEFORE the
+    // table is built, so that their latency runs beside the fill instead of after it (padding
+    // waves have valid, clamped addresses and simply drop what they loaded).
+    uint4 buf[PF][1];
+#pragma unroll
+    for (int i = 0; i < PF; i++)
+        buf[i][0] = (i < nfull) ? cb[(size_t)i * G::VPS] : make_uint4(0, 0, 0, 0);
+    ft_fill(tab, be, tg, un.h);
+    __syncthreads();
+    if (!un.wave_active)
+        return; // padding waves of the head's last workgroup
 
     auto finish = [&](const float *part, int sg, int ntok) {
         const float s = reduce8_head32(part);
@@ -206,13 +214,9 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    uint4 buf[PF][1];
     uint2 lk[G::NP][8];
     uint32_t nb[G::NP][2];
     float part[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-    for (int i = 0; i < PF; i++)
-        buf[i][0] = (i < nfull) ? cb[(size_t)i * G::VPS] : make_uint4(0, 0, 0, 0);
     if (nfull > 0) {
         pair_bytes_of<D, CPL>(buf[0], nb);
 #pragma unroll
@@ -310,15 +314,6 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
     using G = Geo<D, CPL>;
     __shared__ uint2 tab[FT_TABLE_WORDS64];
     const FtUnit un(B, H, sa.nseg);
-    ft_fill(tab, be, tg, un.h);
-    __syncthreads();
-    if (!un.wave_active) {
-        if (sa.combine) { // the two barriers of the in-workgroup sum below
-            __syncthreads();
-            __syncthreads();
-        }
-        return;
-    }
 
     const uint32_t lane_copy = 0x100u | ((uint32_t)un.lh * 8u);
     const int bx = un.bx, lh = un.lh, c0 = un.c0, h = un.h;
@@ -354,6 +349,24 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
         __builtin_memcpy(&r, wb + (size_t)sg * 8, 16); // row base is only 2-byte aligned
         return r;
     };
+    // the first code words and weights, like the parameters above, are requested before the
+    // table is built (see qk_ft_kernel)
+    uint4 buf[PF][1];
+    uint4 wbuf[PF];
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+        buf[i][0] = (i < nfull) ? cb[(size_t)i * G::VPS] : make_uint4(0, 0, 0, 0);
+        wbuf[i] = (i < nfull) ? load_w(i) : make_uint4(0, 0, 0, 0);
+    }
+    ft_fill(tab, be, tg, un.h);
+    __syncthreads();
+    if (!un.wave_active) {
+        if (sa.combine) { // the two barriers of the in-workgroup sum below
+            __syncthreads();
+            __syncthreads();
+        }
+        return;
+    }
     auto token = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2], const uint4 wv) {
         const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
         const h2 wp = as_h2(ww[t >> 1]);
@@ -404,15 +417,8 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    uint4 buf[PF][1];
-    uint4 wbuf[PF];
     uint2 lk[G::NP][8];
     uint32_t nb[G::NP][2];
-#pragma unroll
-    for (int i = 0; i < PF; i++) {
-        buf[i][0] = (i < nfull) ? cb[(size_t)i * G::VPS] : make_uint4(0, 0, 0, 0);
-        wbuf[i] = (i < nfull) ? load_w(i) : make_uint4(0, 0, 0, 0);
-    }
     if (nfull > 0) {
         pair_bytes_of<D, CPL>(buf[0], nb);
 #pragma unroll
