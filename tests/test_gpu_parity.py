@@ -753,6 +753,8 @@ def test_grouped_query_kernels_in_16_wave_workgroups(gpu, oracle, G, bits):
     (3, 2, 100, 16), (1, 2, 63, 8), (5, 2, 257, 64), (2, 3, 530, 64),  # odd batches: half-empty waves
     (2, 2, 1024, 256), (33, 3, 72, 8),                                 # several workgroups per head
     (40, 2, 300, 0),                                                   # no checkpoints, 20 waves per head
+    (4, 2, 40, 32), (2, 2, 64, 32), (5, 3, 100, 32), (9, 2, 127, 32),  # two / four segments (ragged last one):
+                                                                       # partial outputs added in the workgroup
 ])
 def test_per_head_table_kernels(gpu, oracle, B, H, T, S):
     """The decode kernels that keep a per-head (code, channel pair) -> (q, scale multiplier) table
