@@ -286,23 +286,24 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
 // forward_ov  (gemv.cu:946-1178), per-head table
 // ---------------------------------------------------------------------------------------------
 //
-// MM: the contraction runs on the matrix cores.  v_mfma_f32_4x4x4_16B_f16 multiplies, in each group
-// of four lanes, the 4x4 matrix whose row i is lane i's A operand with the matrix whose column r is
-// lane r's B operand, and lane r receives column r of the product.  With
+// MM != 0: the contraction runs on the matrix cores.  v_mfma_f32_4x4x4_16B_f16 multiplies, in each
+// group of four lanes, the 4x4 matrix whose row i is lane i's A operand with the matrix whose
+// column r is lane r's B operand, and lane r receives column r of the product.  With
 //   B of lane r = (x_A[t], x_B[t], x_A[t+1], x_B[t+1])   the lane's channel pair at two tokens, which
 //                                                        is two consecutive registers as they are,
 //   A of lane 0 = (w[t], 0, w[t+1], 0),  A of lane 1 = (0, w[t], 0, w[t+1]),  A of lanes 2, 3 = 0,
 // element 0 of the lane's result is sum w*x_A and element 1 is sum w*x_B: the lane's own two
-// outputs, nothing crosses lanes.  Because the product is linear, the dequantised value q*sc + zp
-// is never formed: one instruction takes the (q*sc) registers of the two tokens, a second one the
-// two zero-points, both accumulate into the same four registers.  That removes the packed add and
-// the two mixed-precision multiply-adds per (pair, token) from the vector pipe (7 -> 4
-// instructions); the 16 matrix instructions per supergroup ride beside the vector ones (measured:
-// up to 4 per 16 packed instructions cost nothing with four waves per SIMD).  The weights reach the
-// A layout with two v_perm_b32 per token pair and per-lane selectors.  A non-finite cached value
-// makes both outputs of its channel PAIR non-finite (0 * inf inside the product); the vector form
-// confines it to its own channel.
-template <bool MM>
+// outputs, nothing crosses lanes, products exact and sums in fp32 as in the vector form.  One
+// instruction per (pair, two tokens) replaces four mixed-precision multiply-adds; a matrix
+// instruction takes one issue slot and then runs beside the vector pipe.  The weights reach the A
+// layout with two v_perm_b32 per token pair and per-lane selectors.
+//   MM == 2 (shipped): x = r16(q*sc + zp), the reference's dequantised value (gemv.cu:1085-1086).
+//   MM == 1: the product is linear, so one instruction takes the two q*sc registers and a second
+//   one the two zero-points and the packed add goes as well; outputs then differ by the skipped
+//   roundings (up to half an fp16 ulp of the largest value), for 1 % of the kernel's time.
+// A non-finite cached value makes both outputs of its channel PAIR non-finite (0 * inf inside the
+// product); the vector form confines it to its own channel.
+template <int MM>
 __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
     const h1 *__restrict__ attn, uint4 *__restrict__ cache, const h1 *__restrict__ v_new,
     h1 *__restrict__ out, float *__restrict__ partial,
@@ -399,16 +400,18 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
             for (int p = 0; p < G::NP; p++) {
                 Pair &s = st[p];
                 const h2 x = as_h2(e[p][t + k].x) * s.sc;
-                qs[p][k] = as_u32(x);
+                qs[p][k] = as_u32(MM == 2 ? x + s.zp : x);
                 z[p][k] = as_u32(s.zp);
                 update_pair_f(s, as_h2(e[p][t + k].y), x);
             }
 #pragma unroll
         for (int p = 0; p < G::NP; p++)
             acc4[p] = __builtin_amdgcn_mfma_f32_4x4x4f16(a, as_h4(qs[p][0], qs[p][1]), acc4[p], 0, 0, 0);
+        if (MM == 1) {
 #pragma unroll
-        for (int p = 0; p < G::NP; p++)
-            acc4[p] = __builtin_amdgcn_mfma_f32_4x4x4f16(a, as_h4(z[p][0], z[p][1]), acc4[p], 0, 0, 0);
+            for (int p = 0; p < G::NP; p++)
+                acc4[p] = __builtin_amdgcn_mfma_f32_4x4x4f16(a, as_h4(z[p][0], z[p][1]), acc4[p], 0, 0, 0);
+        }
 #pragma unroll
         for (int k = 0; k < 2; k++)
 #pragma unroll

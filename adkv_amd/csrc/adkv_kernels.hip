@@ -34,10 +34,11 @@ namespace adkv {
 #define ADKV_PF 4
 #endif
 constexpr int PF = ADKV_PF; // supergroups in flight per lane
-// 1: the per-head-table OV kernel contracts on the matrix cores; 0 builds its vector form instead
-// (a measurement aid for tools/ablate.py, not compiled into the shipped library).
+// How the per-head-table OV kernel contracts: 2 = on the matrix cores over the rounded dequantised
+// values (shipped); 1 = on the matrix cores over q*sc and zp separately, without their fp16 sum;
+// 0 = vector form.  0 and 1 are built by tools/ablate.py only.
 #ifndef ADKV_FT_OV_MM
-#define ADKV_FT_OV_MM 1
+#define ADKV_FT_OV_MM 2
 #endif
 #ifndef ADKV_MFMA_DEFAULT
 #define ADKV_MFMA_DEFAULT 0
@@ -2033,7 +2034,7 @@ static int forward_ov_impl(const void *attn, void *v_cache, const void *v_new, v
         // two or four segments: the waves of one (sequence pair) sit in the same workgroup
         // (interleave_segment) and add their partial outputs there, no second launch
         seg.combine = (seg.nseg == 2 || seg.nseg == 4) ? 1 : 0;
-        hipLaunchKernelGGL(ov_ft_kernel<ADKV_FT_OV_MM != 0>, dim3((unsigned)(H * ft_wgs_per_head(B, seg.nseg))),
+        hipLaunchKernelGGL(ov_ft_kernel<ADKV_FT_OV_MM>, dim3((unsigned)(H * ft_wgs_per_head(B, seg.nseg))),
                            dim3(FT_BLK), 0, st, (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new, (h1 *)out,
                            (float *)workspace, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,
                            (const h1 *)beta, (const h1 *)tgt, B, H, T, n_super_cap, (h1 *)state_out, seg);

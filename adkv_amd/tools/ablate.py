@@ -1,7 +1,8 @@
 """What the per-head-table decode kernels wait for, measured by taking things away.
 
 Builds the library several times from the committed sources with measurement-only macros
-(ADKV_FT_OV_MM=0 gives the OV kernel's vector contraction back; adkv_ft_kernels.h:
+(ADKV_FT_OV_MM=0 / 1: the OV kernel's vector contraction / the matrix one without the add;
+adkv_ft_kernels.h:
 ADKV_ABLATE_NO_LOOKUP skips the LDS table reads, ADKV_ABLATE_CODE_WINDOW=m
 keeps every unit's code prefetch inside its first m+1 supergroups, so the bytes come from L1 / L2 /
 the memory-side cache instead of HBM), then runs the cfg2 decode step (B=128, 32 heads x 128,
@@ -25,6 +26,7 @@ OUT = os.path.join(_DIR, "_ablate")
 VARIANTS = [
     ("as shipped", []),
     ("vector contraction in OV", ["-DADKV_FT_OV_MM=0"]),
+    ("OV: matrix contraction of q*sc and zp apart (no add)", ["-DADKV_FT_OV_MM=1"]),
     ("no table lookups", ["-DADKV_ABLATE_NO_LOOKUP"]),
     ("codes from L1 (2 supergroups per unit)", ["-DADKV_ABLATE_CODE_WINDOW=1"]),
     ("codes from L2 (4 per unit)", ["-DADKV_ABLATE_CODE_WINDOW=3"]),
