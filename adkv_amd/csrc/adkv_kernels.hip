@@ -1591,10 +1591,15 @@ static bool mfma_for_mha()
 }
 
 // Whether a launch with one query head per KV head takes the kernels with a per-head table
-// (adkv_ft_kernels.h).  They need head dim 128 and 4-bit codes; by default they are taken where
-// the shared-table kernels would run 16-wave workgroups of four-channel lanes anyway and the
-// padding of every head's waves to whole workgroups wastes little.  adkv_set_mha_kernel(2) takes
-// them whenever they can run, (0) never.
+// (adkv_ft_kernels.h).  They need head dim 128 and 4-bit codes.  By default the choice follows a
+// model of the two launches, both bound by vector issue: the per-head-table kernels run 16-wave
+// workgroups, one per CU, in ceil(workgroups / 256) rounds of one segment each (every head's
+// waves padded to whole workgroups), at 0.87 of the shared-table kernels' time per wave; the
+// shared-table kernels run the same rounds when the launch is big enough for 16-wave workgroups,
+// and otherwise spread 4-wave workgroups over the SIMDs, where the fullest SIMD sets the time
+// (its waves / 4 rounds).  Measured (B x 32 heads, ctx; per-head table against shared table):
+// 34 x 3000: 155 / 192 us, 40 x 1500: 91 / 108, 24 x 3000: 142 / 145, 20 x 8192 (288 workgroups,
+// two rounds): 370 / 260.  adkv_set_mha_kernel(2) takes them whenever they can run, (0) never.
 static bool use_head_table(int B, int H, int GQ, int bits, int D, const Seg &seg)
 {
     if (D != 128 || bits != 4 || GQ != 1)
@@ -1606,11 +1611,17 @@ static bool use_head_table(int B, int H, int GQ, int bits, int D, const Seg &seg
         return false;
     const long BH = (long)B * H;
     const long padded = padded_units<32>((int)BH, seg.nseg);
-    if (padded / 2 <= N_SIMD || padded * 32 < (long)FT_BLK * 256)
-        return false;                                 // small launches: two-channel lanes / 4-wave workgroups
-    const long waves = (long)seg.nseg * ft_pairs_per_seg(B);
-    const long padded_waves = (long)ft_wgs_per_head(B, seg.nseg) * FT_WAVES;
-    return padded_waves * 100 <= waves * 106;
+    const long waves_shared = padded / 2;
+    if (waves_shared <= N_SIMD)
+        return false;                                 // every wave a SIMD to itself: two-channel lanes
+    const long wgs_ft = (long)H * ft_wgs_per_head(B, seg.nseg);
+    const double t_ft = 0.87 * (double)((wgs_ft + 255) / 256);
+    double t_shared;
+    if (padded * 32 >= (long)FT_BLK * 256)
+        t_shared = (double)(((padded * 32 + FT_BLK - 1) / FT_BLK + 255) / 256);
+    else
+        t_shared = (double)((waves_shared + N_SIMD - 1) / N_SIMD) / WAVES_PER_SIMD_TARGET;
+    return t_ft <= t_shared;
 }
 
 // ADKV_ENCODE_CPL=1/2 pins the encoder's channels per lane (a measurement aid); read once.
