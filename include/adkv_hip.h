@@ -39,7 +39,7 @@ int adkv_abi_version(void);
  * heads as KV heads and head dim 128 uses: 0 = the vector kernels with the shared code table,
  * 1 = the matrix-core kernels (the ones grouped-query launches always use), 2 = the vector
  * kernels with a per-head table wherever they can run (4-bit codes), -1 = the library's choice
- * (the per-head table for big launches, else the shared one; ADKV_MFMA=1 in the environment,
+ * (the per-head table where its launch is the faster one, else the shared one; ADKV_MFMA=1 in the environment,
  * read once, makes it the matrix-core kernels).  Results agree to the tolerance of the fp32
  * accumulation order; appended codes, state and checkpoints are identical. */
 void adkv_set_mha_kernel(int use_matrix_cores);
