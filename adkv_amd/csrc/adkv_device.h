@@ -18,6 +18,13 @@ namespace adkv {
 typedef _Float16 h1;
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 
+// operand types of v_mfma_f32_4x4x4_16B_f16: four fp16 (two registers), four fp32
+typedef float f4v __attribute__((ext_vector_type(4)));
+typedef _Float16 h4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ h4v as_h4(uint32_t lo, uint32_t hi)
+{
+    return __builtin_bit_cast(h4v, make_uint2(lo, hi));
+}
 __device__ __forceinline__ h2 as_h2(uint32_t u) { return __builtin_bit_cast(h2, u); }
 __device__ __forceinline__ uint32_t as_u32(h2 h) { return __builtin_bit_cast(uint32_t, h); }
 __device__ __forceinline__ h2 pk_fma(h2 a, h2 b, h2 c) { return __builtin_elementwise_fma(a, b, c); }

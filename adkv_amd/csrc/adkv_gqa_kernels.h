@@ -25,8 +25,6 @@
 
 namespace adkv {
 
-typedef float f4v __attribute__((ext_vector_type(4)));
-typedef _Float16 h4v __attribute__((ext_vector_type(4)));
 
 constexpr int GQA_D = 128;
 constexpr int GQA_CPL = 4;
@@ -40,10 +38,6 @@ __device__ __forceinline__ float dpp_mov(float v)
                                                                   0xF, false));
 }
 
-__device__ __forceinline__ h4v as_h4(uint32_t lo, uint32_t hi)
-{
-    return __builtin_bit_cast(h4v, make_uint2(lo, hi));
-}
 
 // The code words of one supergroup -> the per-pair byte streams the table is indexed with.
 template <int BITS>

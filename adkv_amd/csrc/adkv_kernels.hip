@@ -914,6 +914,17 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
 #pragma unroll
     for (int c = 0; c < CPL; c++)
         acc[c] = 0.0f;
+    // Four-channel (and wider) lanes contract on the matrix cores, as ov_ft_kernel does and for the
+    // reason given there: B = the lane's dequantised pair at two tokens, A = (w[t], 0, w[t+1], 0)
+    // from lane 0 of each group of four, (0, w[t], 0, w[t+1]) from lane 1, zeros from lanes 2, 3.
+    constexpr bool MM = CPL >= 4;
+    f4v acc4[G::NP];
+#pragma unroll
+    for (int p = 0; p < G::NP; p++)
+        acc4[p] = (f4v){0.0f, 0.0f, 0.0f, 0.0f};
+    const int role = threadIdx.x & 3;
+    const uint32_t sel_a0 = role == 0 ? 0x0C0C0100u : role == 1 ? 0x01000C0Cu : 0x0C0C0C0Cu;
+    const uint32_t sel_a1 = role == 0 ? 0x0C0C0302u : role == 1 ? 0x03020C0Cu : 0x0C0C0C0Cu;
 
     const int t0 = un.seg * sa.seg_tokens;
     const int t1 = last ? T : t0 + sa.seg_tokens;
@@ -950,6 +961,33 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
         __builtin_amdgcn_sched_barrier(0);
     };
 
+    // two tokens of the current supergroup on the matrix cores, then the lookups of the same two
+    // slots of the next one
+    auto token2 = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2], const uint4 wv) {
+        const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+        const uint32_t w2 = ww[t >> 1];
+        const h4v a = as_h4(__builtin_amdgcn_perm(w2, w2, sel_a0), __builtin_amdgcn_perm(w2, w2, sel_a1));
+        uint32_t vd[G::NP][2];
+#pragma unroll
+        for (int k = 0; k < 2; k++)
+#pragma unroll
+            for (int p = 0; p < G::NP; p++) {
+                Pair &s = st[p];
+                const h2 qs = as_h2(e[p][t + k].x) * s.sc;
+                vd[p][k] = as_u32(qs + s.zp);
+                update_pair_abs(s, as_h2(e[p][t + k].y), qs);
+            }
+#pragma unroll
+        for (int p = 0; p < G::NP; p++)
+            acc4[p] = __builtin_amdgcn_mfma_f32_4x4x4f16(a, as_h4(vd[p][0], vd[p][1]), acc4[p], 0, 0, 0);
+#pragma unroll
+        for (int k = 0; k < 2; k++)
+#pragma unroll
+            for (int p = 0; p < G::NP; p++)
+                e[p][t + k] = lut_get(lut, nb[p][(t + k) & 1], lane_copy, (t + k) >> 1);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
     Vec buf[PF][G::NV];
     uint4 wbuf[PF];
     uint2 lk[G::NP][8];
@@ -978,14 +1016,27 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
         for (int v = 0; v < G::NV; v++)
             buf[i][v] = cb[(size_t)sgp * G::VPS + v];
         __builtin_amdgcn_sched_barrier(0);
+        if (MM) {
 #pragma unroll
-        for (int t = 0; t < 8; t++)
-            token(t, lk, nb, wbuf[i]);
+            for (int t = 0; t < 8; t += 2)
+                token2(t, lk, nb, wbuf[i]);
+        } else {
+#pragma unroll
+            for (int t = 0; t < 8; t++)
+                token(t, lk, nb, wbuf[i]);
+        }
         // the weights are reloaded once their last token is done: loading them earlier into a
         // second register set costs copies at the loop edge, which wait for the load they move
         wbuf[i] = load_w(sgp);
     };
     rotate_over<PF>(nfull, body);
+    if (MM) {
+#pragma unroll
+        for (int p = 0; p < G::NP; p++) {
+            acc[2 * p] = acc4[p].x;
+            acc[2 * p + 1] = acc4[p].y;
+        }
+    }
 
     if (last) {
         const int ntail = (t1 - t0) & 7;
@@ -1594,12 +1645,12 @@ static bool mfma_for_mha()
 // (adkv_ft_kernels.h).  They need head dim 128 and 4-bit codes.  By default the choice follows a
 // model of the two launches, both bound by vector issue: the per-head-table kernels run 16-wave
 // workgroups, one per CU, in ceil(workgroups / 256) rounds of one segment each (every head's
-// waves padded to whole workgroups), at 0.87 of the shared-table kernels' time per wave; the
+// waves padded to whole workgroups), at 0.93 of the shared-table kernels' time per wave; the
 // shared-table kernels run the same rounds when the launch is big enough for 16-wave workgroups,
 // and otherwise spread 4-wave workgroups over the SIMDs, where the fullest SIMD sets the time
 // (its waves / 4 rounds).  Measured (B x 32 heads, ctx; per-head table against shared table):
-// 34 x 3000: 155 / 192 us, 40 x 1500: 91 / 108, 24 x 3000: 142 / 145, 20 x 8192 (288 workgroups,
-// two rounds): 370 / 260.  adkv_set_mha_kernel(2) takes them whenever they can run, (0) never.
+// 128 x 4096: 587 / 624 us per layer-step, 34 x 3000: 155 / 181, 40 x 1500: 89 / 107, 24 x 3000:
+// 141 / 141, 20 x 8192 (288 workgroups, two rounds): 369 / 255.  adkv_set_mha_kernel(2) takes them whenever they can run, (0) never.
 static bool use_head_table(int B, int H, int GQ, int bits, int D, const Seg &seg)
 {
     if (D != 128 || bits != 4 || GQ != 1)
@@ -1615,7 +1666,7 @@ static bool use_head_table(int B, int H, int GQ, int bits, int D, const Seg &seg
     if (waves_shared <= N_SIMD)
         return false;                                 // every wave a SIMD to itself: two-channel lanes
     const long wgs_ft = (long)H * ft_wgs_per_head(B, seg.nseg);
-    const double t_ft = 0.87 * (double)((wgs_ft + 255) / 256);
+    const double t_ft = 0.93 * (double)((wgs_ft + 255) / 256);
     double t_shared;
     if (padded * 32 >= (long)FT_BLK * 256)
         t_shared = (double)(((padded * 32 + FT_BLK - 1) / FT_BLK + 255) / 256);
