@@ -1152,8 +1152,10 @@ constexpr int SM_BLOCK = 256;
 constexpr int SM_VEC = 8;                             // fp16 values per 16-byte access
 constexpr int SM_NV = 3;                              // such accesses per thread and chunk
 constexpr int SM_KEEP = SM_VEC * SM_NV;               // row elements a thread keeps in registers
-constexpr int SM_CHUNK = SM_BLOCK * SM_KEEP;          // row elements one workgroup holds
+constexpr int SM_CHUNK = SM_BLOCK * SM_KEEP;          // row elements a 256-thread workgroup holds
+constexpr int SM_ROW_MAX = 24576;                     // longest row a single workgroup keeps in registers
 
+template <int NT = SM_BLOCK>
 __device__ __forceinline__ float block_reduce(float v, float *sm, bool is_max)
 {
 #pragma unroll
@@ -1168,7 +1170,7 @@ __device__ __forceinline__ float block_reduce(float v, float *sm, bool is_max)
     __syncthreads();
     float r = sm[0];
 #pragma unroll
-    for (int i = 1; i < SM_BLOCK / 64; i++)
+    for (int i = 1; i < NT / 64; i++)
         r = is_max ? fmaxf(r, sm[i]) : r + sm[i];
     return r;
 }
@@ -1278,31 +1280,32 @@ __global__ __launch_bounds__(SM_BLOCK) void softmax_wave_kernel(
     softmax_store_chunk<NV, 64>(w, n, 0, x, 1.0f / sum, lane);
 }
 
-// One workgroup per row.  A row of up to SM_CHUNK elements is read once and kept in registers;
-// longer rows are walked three times (the chunked kernels below avoid that when the caller gives
-// a workspace).
-__global__ __launch_bounds__(SM_BLOCK) void softmax_kernel(
+// One workgroup of NT threads per row.  A row of up to NT * NV * 8 elements is read once and kept
+// in registers (the launcher picks NT and NV by the row length, up to 24576 elements); longer rows
+// are walked three times (the chunked kernels below avoid that when the caller gives a workspace).
+template <int NT, int NV>
+__global__ __launch_bounds__(NT) void softmax_kernel(
     const h1 *__restrict__ logits, h1 *__restrict__ weights, const float *__restrict__ mask,
     int n, long ld, int rows_per_mask_row, float scaling)
 {
-    __shared__ float sm[SM_BLOCK / 64];
+    __shared__ float sm[NT / 64];
     const int row = blockIdx.x;
     const h1 *l = logits + (size_t)row * ld;
     h1 *w = weights + (size_t)row * ld;
     const float *mk = mask ? mask + (size_t)(row / rows_per_mask_row) * n : nullptr;
 
-    if (n <= SM_CHUNK) {
-        float x[SM_KEEP], mx;
-        softmax_load_chunk(l, mk, n, 0, scaling, x, mx);
-        mx = block_reduce(mx, sm, true);
+    if (n <= NT * NV * SM_VEC) {
+        float x[NV * SM_VEC], mx;
+        softmax_load_chunk<NV, NT>(l, mk, n, 0, scaling, x, mx);
+        mx = block_reduce<NT>(mx, sm, true);
         float sum = 0.0f;
 #pragma unroll
-        for (int k = 0; k < SM_KEEP; k++) {
+        for (int k = 0; k < NV * SM_VEC; k++) {
             x[k] = __expf(x[k] - mx);
             sum += x[k];
         }
-        sum = block_reduce(sum, sm, false);
-        softmax_store_chunk(w, n, 0, x, 1.0f / sum);
+        sum = block_reduce<NT>(sum, sm, false);
+        softmax_store_chunk<NV, NT>(w, n, 0, x, 1.0f / sum);
         return;
     }
     auto at = [&](int i) {
@@ -1312,15 +1315,15 @@ __global__ __launch_bounds__(SM_BLOCK) void softmax_kernel(
         return v;
     };
     float mx = -INFINITY;
-    for (int i = threadIdx.x; i < n; i += SM_BLOCK)
+    for (int i = threadIdx.x; i < n; i += NT)
         mx = fmaxf(mx, at(i));
-    mx = block_reduce(mx, sm, true);
+    mx = block_reduce<NT>(mx, sm, true);
     float sum = 0.0f;
-    for (int i = threadIdx.x; i < n; i += SM_BLOCK)
+    for (int i = threadIdx.x; i < n; i += NT)
         sum += __expf(at(i) - mx);
-    sum = block_reduce(sum, sm, false);
+    sum = block_reduce<NT>(sum, sm, false);
     const float inv = 1.0f / sum;
-    for (int i = threadIdx.x; i < n; i += SM_BLOCK)
+    for (int i = threadIdx.x; i < n; i += NT)
         w[i] = (h1)(__expf(at(i) - mx) * inv);
 }
 
@@ -2236,7 +2239,7 @@ int adkv_forward_ov(const void *attn, void *v_cache, const void *v_new, void *ou
 
 int64_t adkv_softmax_workspace_bytes(int rows, int n)
 {
-    if (rows <= 0 || n <= SM_CHUNK)
+    if (rows <= 0 || n <= SM_ROW_MAX)
         return 0;
     return (int64_t)rows * ((n + SM_CHUNK - 1) / SM_CHUNK) * 8;
 }
@@ -2280,10 +2283,29 @@ int adkv_softmax_ex(const void *logits, void *weights, const void *mask,
     }
     const int64_t need = adkv_softmax_workspace_bytes(rows, n);
     if (need == 0 || !workspace || rows > 65535) {
-        // one workgroup per row; rows that do not fit in its registers are read three times
-        hipLaunchKernelGGL(softmax_kernel, dim3((unsigned)rows), dim3(SM_BLOCK), 0, (hipStream_t)stream,
-                           (const h1 *)logits, (h1 *)weights, (const float *)mask, n, (long)ld,
-                           mask ? rows_per_mask_row : 1, scaling);
+        // one workgroup per row, sized so that the row stays in its registers (read once, written
+        // once); rows beyond 24576 elements without a workspace are read three times
+#define ADKV_SM_ROW(NT, NV)                                                                         \
+    hipLaunchKernelGGL((softmax_kernel<NT, NV>), dim3((unsigned)rows), dim3(NT), 0,                 \
+                       (hipStream_t)stream, (const h1 *)logits, (h1 *)weights, (const float *)mask, \
+                       n, (long)ld, mask ? rows_per_mask_row : 1, scaling)
+        // (threads, 16-byte vectors per thread) per row length, measured on 4096 rows: 4097 elements
+        // 18.4 us with 256 x 3 and 16.7 with 320 x 2; 8192: 35.5 with 512 x 3, 24.3 with 512 x 2;
+        // 10000: 36.9 with 512 x 3, 33.0 with 256 x 6; 16384: 76.5 with 1024 x 3, 46.9 with 1024 x 2;
+        // 2048 rows of 24576: 42.1 with 1024 x 3, 37.4 with 512 x 6
+        if (n <= 5120)
+            ADKV_SM_ROW(320, 2);
+        else if (n <= SM_CHUNK || n > SM_ROW_MAX)
+            ADKV_SM_ROW(SM_BLOCK, SM_NV);
+        else if (n <= 8192)
+            ADKV_SM_ROW(512, 2);
+        else if (n <= 12288)
+            ADKV_SM_ROW(256, 6);
+        else if (n <= 16384)
+            ADKV_SM_ROW(1024, 2);
+        else
+            ADKV_SM_ROW(512, 6);
+#undef ADKV_SM_ROW
         return check_launch();
     }
     if (workspace_bytes < need)

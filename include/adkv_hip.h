@@ -96,9 +96,9 @@ int adkv_forward_ov(const void *attn, void *v_cache, const void *v_new, void *ou
 int adkv_softmax(const void *logits, void *weights, const void *mask,
                  int rows, int n, int rows_per_mask_row, float scaling, void *stream);
 
-/* The same with a workspace of adkv_softmax_workspace_bytes(rows, n) bytes (0 for short rows):
- * long rows (contexts of tens of thousands of tokens) are then cut into chunks that many
- * workgroups process, instead of one workgroup walking the row three times.  ld: pitch of both
+/* The same with a workspace of adkv_softmax_workspace_bytes(rows, n) bytes (0 for rows of up to
+ * 24576 elements, which one workgroup keeps in its registers): longer rows are then cut into
+ * chunks that many workgroups process, instead of one workgroup walking the row three times.  ld: pitch of both
  * matrices in elements (0 = n); the mask stays packed. */
 int64_t adkv_softmax_workspace_bytes(int rows, int n);
 int adkv_softmax_ex(const void *logits, void *weights, const void *mask,

@@ -111,7 +111,14 @@ def test_forward_qk_and_ov(gpu, oracle, B, H, T, D):
                                               # long unmasked rows: four chunks per workgroup in the first
                                               # pass (all inside the row / last group ragged / one group only)
                                               (4, 131073, None), (2, 60000, None), (2, 49152, None),
-                                              (2, 49153, None)])
+                                              (2, 49153, None),
+                                              # one workgroup per row, its shape chosen by the length:
+                                              # first and last length of each shape, then the
+                                              # shortest chunked row
+                                              (4, 2049, None), (4, 5120, "b1"), (4, 6144, None),
+                                              (4, 6145, "bh"), (4, 8192, None), (4, 8193, "b1"),
+                                              (4, 12288, None), (4, 12289, "b1"), (2, 16384, None),
+                                              (2, 16385, "bh"), (2, 24576, None), (2, 24577, "bh")])
 def test_softmax(gpu, rows, n, mask_mode):
     g = torch.Generator().manual_seed(n)
     B, H = 2, rows // 2
