@@ -1327,6 +1327,110 @@ __global__ __launch_bounds__(NT) void softmax_kernel(
         w[i] = (h1)(__expf(at(i) - mx) * inv);
 }
 
+// Unmasked rows of up to 1024 * NV * 8 elements (139 264 with NV = 17), one 1024-thread workgroup
+// per row: the row stays in registers AS FP16 (NV 16-byte vectors per thread), so it is read once
+// and written once; maximum, sum and weights are three walks over registers.  Two such workgroups
+// fit a CU (128 registers per lane); few and very long rows are better cut into chunks.
+// scaling must be non-zero: elements past the end of the row are held as the infinity that
+// scaling turns into -inf.
+constexpr int SM_REG_NV = 17;
+constexpr int SM_REG_MAX = 1024 * SM_REG_NV * SM_VEC;
+#ifndef ADKV_SM_REG_MIN_ROWS
+#define ADKV_SM_REG_MIN_ROWS 128
+#endif
+constexpr int SM_REG_MIN_ROWS = ADKV_SM_REG_MIN_ROWS;
+
+template <int NV>
+__global__ __launch_bounds__(1024) void softmax_regrow_kernel(
+    const h1 *__restrict__ logits, h1 *__restrict__ weights, int n, long ld, float scaling)
+{
+    constexpr int NT = 1024;
+    __shared__ float sm[NT / 64];
+    const h1 *l = logits + (size_t)blockIdx.x * ld;
+    h1 *w = weights + (size_t)blockIdx.x * ld;
+    const int tid = threadIdx.x;
+    const uint32_t pad = scaling > 0.0f ? 0xFC00FC00u : 0x7C007C00u; // scaling * pad = -inf
+
+    uint4 raw[NV];
+#pragma unroll
+    for (int v = 0; v < NV; v++) {
+        const int i0 = (v * NT + tid) * SM_VEC;
+        if (i0 + SM_VEC <= n) {
+            __builtin_memcpy(&raw[v], l + i0, 16); // rows are only 2-byte aligned
+        } else {
+            uint32_t u[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const uint32_t lo = i0 + 2 * k < n ? __builtin_bit_cast(uint16_t, l[i0 + 2 * k]) : (pad & 0xFFFFu);
+                const uint32_t hi = i0 + 2 * k + 1 < n ? __builtin_bit_cast(uint16_t, l[i0 + 2 * k + 1]) : (pad & 0xFFFFu);
+                u[k] = lo | (hi << 16);
+            }
+            raw[v] = make_uint4(u[0], u[1], u[2], u[3]);
+        }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int v = 0; v < NV; v++) {
+        const uint32_t u[4] = {raw[v].x, raw[v].y, raw[v].z, raw[v].w};
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const h2 p = as_h2(u[k]);
+            mx = fmaxf(mx, fmaxf((float)p.x * scaling, (float)p.y * scaling));
+        }
+    }
+    mx = block_reduce<NT>(mx, sm, true);
+    // each walk converts the row again: values carried over from the walk before (which the
+    // compiler would otherwise keep, 136 more registers per lane) are cut off here
+    auto forget = [&]() {
+#pragma unroll
+        for (int v = 0; v < NV; v++)
+            asm volatile("" : "+v"(raw[v].x), "+v"(raw[v].y), "+v"(raw[v].z), "+v"(raw[v].w));
+    };
+    forget();
+    // exp(x * scaling - mx) = exp2(x * s2 + c2)
+    const float s2 = scaling * 1.44269504088896340736f;
+    const float c2 = mx == -INFINITY ? 0.0f : -mx * 1.44269504088896340736f;
+    float sum = 0.0f;
+#pragma unroll
+    for (int v = 0; v < NV; v++) {
+        const uint32_t u[4] = {raw[v].x, raw[v].y, raw[v].z, raw[v].w};
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const h2 p = as_h2(u[k]);
+            sum += __builtin_amdgcn_exp2f(__builtin_fmaf((float)p.x, s2, c2));
+            sum += __builtin_amdgcn_exp2f(__builtin_fmaf((float)p.y, s2, c2));
+        }
+    }
+    sum = block_reduce<NT>(sum, sm, false);
+    const float inv = 1.0f / sum;
+    forget();
+#pragma unroll
+    for (int v = 0; v < NV; v++) {
+        const int i0 = (v * NT + tid) * SM_VEC;
+        const uint32_t u[4] = {raw[v].x, raw[v].y, raw[v].z, raw[v].w};
+        uint32_t o[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const h2 p = as_h2(u[k]);
+            o[k] = as_u32((h2){(h1)(__builtin_amdgcn_exp2f(__builtin_fmaf((float)p.x, s2, c2)) * inv),
+                               (h1)(__builtin_amdgcn_exp2f(__builtin_fmaf((float)p.y, s2, c2)) * inv)});
+        }
+        if (i0 + SM_VEC <= n) {
+            const uint4 ov = make_uint4(o[0], o[1], o[2], o[3]);
+            __builtin_memcpy(w + i0, &ov, 16);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const h2 p = as_h2(o[k]);
+                if (i0 + 2 * k < n)
+                    w[i0 + 2 * k] = p.x;
+                if (i0 + 2 * k + 1 < n)
+                    w[i0 + 2 * k + 1] = p.y;
+            }
+        }
+    }
+}
+
 // Rows longer than one workgroup can hold in registers are cut into chunks of SM_CHUNK elements,
 // one workgroup each: the first pass leaves (max, sum of exp(x - max)) per chunk, the second
 // combines a row's chunks and normalises.  Each logit is read twice and nothing depends on the
@@ -2279,6 +2383,28 @@ int adkv_softmax_ex(const void *logits, void *weights, const void *mask,
         else
             ADKV_SM_WAVE(4);
 #undef ADKV_SM_WAVE
+        return check_launch();
+    }
+    const int reg_nv = (n + 1024 * SM_VEC - 1) / (1024 * SM_VEC); // 16-byte vectors per thread
+    if (n > SM_ROW_MAX && !mask && n <= SM_REG_MAX && (rows >= SM_REG_MIN_ROWS || reg_nv <= 9) &&
+        scaling != 0.0f && scaling == scaling) {
+        // long unmasked rows stay in registers, unless they are few and very long (32 rows of
+        // 131 073: 14.6 us cut into chunks, 19.8 us this way; 128 rows: 28.1 and 24.8; 512 rows:
+        // 74.8 and 56.7; 64 rows of 32 769: 11.4 and 9.4; 4096 rows of 24 577: 148 and 80)
+#define ADKV_SM_REG(NV)                                                                             \
+    case NV:                                                                                        \
+        hipLaunchKernelGGL(softmax_regrow_kernel<NV>, dim3((unsigned)rows), dim3(1024), 0,          \
+                           (hipStream_t)stream, (const h1 *)logits, (h1 *)weights, n, (long)ld,     \
+                           scaling);                                                                \
+        break
+        switch (reg_nv) {
+            ADKV_SM_REG(4); ADKV_SM_REG(5); ADKV_SM_REG(6); ADKV_SM_REG(7); ADKV_SM_REG(8);
+            ADKV_SM_REG(9); ADKV_SM_REG(10); ADKV_SM_REG(11); ADKV_SM_REG(12); ADKV_SM_REG(13);
+            ADKV_SM_REG(14); ADKV_SM_REG(15); ADKV_SM_REG(16);
+        default:
+            ADKV_SM_REG(17);
+        }
+#undef ADKV_SM_REG
         return check_launch();
     }
     const int64_t need = adkv_softmax_workspace_bytes(rows, n);

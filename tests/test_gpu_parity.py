@@ -118,7 +118,14 @@ def test_forward_qk_and_ov(gpu, oracle, B, H, T, D):
                                               (4, 2049, None), (4, 5120, "b1"), (4, 6144, None),
                                               (4, 6145, "bh"), (4, 8192, None), (4, 8193, "b1"),
                                               (4, 12288, None), (4, 12289, "b1"), (2, 16384, None),
-                                              (2, 16385, "bh"), (2, 24576, None), (2, 24577, "bh")])
+                                              (2, 16385, "bh"), (2, 24576, None), (2, 24577, "bh"),
+                                              # long unmasked rows kept in registers as fp16 (one
+                                              # 1024-thread workgroup per row): shortest, a full
+                                              # 9-vector row, the longest; one element more goes
+                                              # back to the chunked kernels
+                                              (2, 24577, None), (2, 73728, None), (2, 73729, None),
+                                              (128, 131073, None), (130, 139264, None),
+                                              (130, 139265, None)])
 def test_softmax(gpu, rows, n, mask_mode):
     g = torch.Generator().manual_seed(n)
     B, H = 2, rows // 2
@@ -135,6 +142,19 @@ def test_softmax(gpu, rows, n, mask_mode):
         ref = ref + (mask[:, :, 0, :] if mask.dim() == 4 else mask)
     ref = torch.softmax(ref.double(), -1)
     assert torch.max(torch.abs(w.cpu().double() - ref)) < 6e-4  # half an fp16 ulp at 1.0 + eps
+
+
+@pytest.mark.parametrize("n", [4097, 30000, 70000])
+@pytest.mark.parametrize("scaling", [-0.05, 0.0])
+def test_softmax_negative_and_zero_scaling(gpu, n, scaling):
+    """The register-resident long-row kernel pads a row with the infinity that the scaling turns
+    into -inf; a negative scaling flips it and a zero scaling must take another kernel."""
+    g = torch.Generator().manual_seed(n)
+    l = (torch.randn(1, 2, n, generator=g) * 8).half()
+    w = gemv.softmax_scale_mask(l.to(gpu), scaling)
+    ref = torch.softmax(l.double() * scaling, -1)
+    assert torch.max(torch.abs(w.cpu().double() - ref)) < 6e-4
+    assert torch.all(torch.isfinite(w.cpu().float()))
 
 
 @pytest.mark.parametrize("B,H,T,D", [(1, 32, 1024, 128), (2, 4, 257, 128), (1, 2, 100, 256)])
