@@ -87,3 +87,41 @@ def test_random_config(gpu, oracle, seed):
     assert np.all(np.abs(og - wo) <= _ulp16(wo) + 1e-3), what
     if S:
         assert torch.equal(ck.view(torch.int16), ckv.view(torch.int16)), what
+
+
+def _softmax_config(seed):
+    rng = random.Random(1000 + seed)
+    # row lengths spread over every kernel of the softmax: a wave per row, a workgroup per row in
+    # its six shapes, rows held in registers as fp16, the chunked pair
+    n = int(round(2.0 ** rng.uniform(0.0, 17.2)))
+    near = rng.choice([None, None, 2048, 5120, 6144, 8192, 12288, 16384, 24576, 73728, 139264])
+    if near is not None:
+        n = max(1, near + rng.randint(-2, 2))
+    B = rng.randint(1, 3)
+    H = rng.randint(1, max(1, min(48, 6_000_000 // (B * n))))
+    if n > 24576 and rng.random() < 0.5:
+        H = max(H, (128 + B - 1) // B) if B * n * 130 <= 40_000_000 else H   # enough rows for registers
+    mask_mode = rng.choice([None, None, "b1", "bh"])
+    scaling = rng.choice([0.0884, 0.0884, 1.0, 0.125, -0.05])
+    return B, H, n, mask_mode, scaling
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_softmax_random_shapes(gpu, seed):
+    B, H, n, mask_mode, scaling = _softmax_config(seed)
+    g = torch.Generator().manual_seed(seed)
+    l = (torch.randn(B, H, n, generator=g) * 6).half()
+    mask = None
+    if mask_mode == "b1":
+        mask = torch.zeros(B, 1, 1, n)
+        mask[0, 0, 0, : n // 3] = float("-inf")
+    elif mask_mode == "bh":
+        mask = torch.randn(B, H, n, generator=g)
+    w = gemv.softmax_scale_mask(l.to(gpu), scaling, None if mask is None else mask.to(gpu))
+    ref = l.double() * scaling
+    if mask is not None:
+        ref = ref + (mask[:, :, 0, :] if mask.dim() == 4 else mask).double()
+    ref = torch.softmax(ref, -1)
+    assert w.shape == (B, H, n)
+    err = torch.max(torch.abs(w.cpu().double() - ref)).item()
+    assert err < 6e-4, (B, H, n, mask_mode, scaling, err)
