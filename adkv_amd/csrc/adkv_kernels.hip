@@ -1329,8 +1329,9 @@ __global__ __launch_bounds__(NT) void softmax_kernel(
 
 // Unmasked rows of up to 1024 * NV * 8 elements (139 264 with NV = 17), one 1024-thread workgroup
 // per row: the row stays in registers AS FP16 (NV 16-byte vectors per thread), so it is read once
-// and written once; maximum, sum and weights are three walks over registers.  Two such workgroups
-// fit a CU (128 registers per lane); few and very long rows are better cut into chunks.
+// and written once; maximum, sum and weights are three walks over registers.  Up to 9 vectors
+// per thread two such workgroups fit a CU (64 registers per lane), beyond that one (104 registers
+// with 17 vectors); few and very long rows are better cut into chunks.
 // scaling must be non-zero: elements past the end of the row are held as the infinity that
 // scaling turns into -inf.
 constexpr int SM_REG_NV = 17;
