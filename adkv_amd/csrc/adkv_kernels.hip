@@ -1146,6 +1146,85 @@ __global__ __launch_bounds__(256) void ov_finalize_wide_kernel(const float *__re
 }
 
 // ---------------------------------------------------------------------------------------------
+// Rotary position embedding of q and k in one launch   (llama_adkv.py:336-338 calls transformers'
+// apply_rotary_pos_emb: x * cos + rotate_half(x) * sin, ten elementwise launches)
+// ---------------------------------------------------------------------------------------------
+// Every operation is rounded to the activations' type the way torch's elementwise kernels round
+// it (operands widened to fp32, one fp32 operation, result rounded to nearest even), so the
+// output equals that of the torch expression bit for bit.  A row is one (batch, token, head)
+// vector of D values; a lane takes two adjacent values of the first half and their partners in
+// the second.
+template <bool BF16>
+__device__ __forceinline__ float act_to_f32(uint32_t bits16)
+{
+    if (BF16)
+        return __uint_as_float(bits16 << 16);
+    return (float)__builtin_bit_cast(h1, (uint16_t)bits16);
+}
+template <bool BF16>
+__device__ __forceinline__ uint32_t f32_to_act(float f)
+{
+    if (BF16) {
+        const uint32_t u = __float_as_uint(f);
+        if ((u & 0x7FFFFFFFu) > 0x7F800000u)
+            return 0x7FC0u; // torch's bfloat16 NaN
+        return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+    }
+    return (uint32_t)__builtin_bit_cast(uint16_t, (h1)f);
+}
+// r(r(x*c) + r(y*s)) with y already negated where rotate_half negates
+template <bool BF16>
+__device__ __forceinline__ uint32_t rope_one(uint32_t x, uint32_t c, uint32_t y, bool neg_y, uint32_t s)
+{
+    const float a = act_to_f32<BF16>(f32_to_act<BF16>(act_to_f32<BF16>(x) * act_to_f32<BF16>(c)));
+    const float yy = neg_y ? -act_to_f32<BF16>(y) : act_to_f32<BF16>(y);
+    const float b = act_to_f32<BF16>(f32_to_act<BF16>(yy * act_to_f32<BF16>(s)));
+    return f32_to_act<BF16>(a + b);
+}
+
+struct RopeSide {
+    const uint16_t *x;
+    uint16_t *out;
+    long sb, sh, st; // element strides of x over batch, head, token (channels contiguous)
+    int heads;
+};
+
+// grid: (lanes of one token's Hq + H rows in workgroups of 256, token, batch)
+template <bool BF16>
+__global__ __launch_bounds__(256) void rope_kernel(RopeSide q, RopeSide k, const uint16_t *__restrict__ cos,
+                                                   const uint16_t *__restrict__ sin, long cb, long ct,
+                                                   int T, int D, int t0, int b0)
+{
+    const unsigned lpr = (unsigned)D >> 2;                   // lanes per row
+    const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+    const unsigned hh = idx / lpr;
+    if (hh >= (unsigned)(q.heads + k.heads))
+        return;
+    const int i = (int)(idx - hh * lpr) * 2;                 // first of this lane's two channels
+    const int t = t0 + (int)blockIdx.y;
+    const long b = (long)b0 + (long)blockIdx.z;
+    const RopeSide &sd = hh < (unsigned)q.heads ? q : k;
+    const int h = hh < (unsigned)q.heads ? (int)hh : (int)hh - q.heads;
+    const uint16_t *x = sd.x + b * sd.sb + h * sd.sh + t * sd.st;
+    uint16_t *o = sd.out + ((b * sd.heads + h) * T + t) * D;
+    const uint16_t *c = cos + b * cb + t * ct, *s = sin + b * cb + t * ct;
+    const int half = D >> 1;
+    const uint32_t x1 = *reinterpret_cast<const uint32_t *>(x + i);
+    const uint32_t x2 = *reinterpret_cast<const uint32_t *>(x + half + i);
+    const uint32_t c1 = *reinterpret_cast<const uint32_t *>(c + i);
+    const uint32_t c2 = *reinterpret_cast<const uint32_t *>(c + half + i);
+    const uint32_t s1 = *reinterpret_cast<const uint32_t *>(s + i);
+    const uint32_t s2 = *reinterpret_cast<const uint32_t *>(s + half + i);
+    // first half: x1*cos + (-x2)*sin; second half: x2*cos + x1*sin
+    const uint32_t lo0 = rope_one<BF16>(x1 & 0xFFFFu, c1 & 0xFFFFu, x2 & 0xFFFFu, true, s1 & 0xFFFFu);
+    const uint32_t lo1 = rope_one<BF16>(x1 >> 16, c1 >> 16, x2 >> 16, true, s1 >> 16);
+    const uint32_t hi0 = rope_one<BF16>(x2 & 0xFFFFu, c2 & 0xFFFFu, x1 & 0xFFFFu, false, s2 & 0xFFFFu);
+    const uint32_t hi1 = rope_one<BF16>(x2 >> 16, c2 >> 16, x1 >> 16, false, s2 >> 16);
+    *reinterpret_cast<uint32_t *>(o + i) = lo0 | (lo1 << 16);
+    *reinterpret_cast<uint32_t *>(o + half + i) = hi0 | (hi1 << 16);
+}
+
+// ---------------------------------------------------------------------------------------------
 // softmax(float(logits)*scaling + mask) -> fp16   (llama_adkv.py:266-271)
 // ---------------------------------------------------------------------------------------------
 constexpr int SM_BLOCK = 256;
@@ -1808,7 +1887,7 @@ static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval, int b
 
 extern "C" {
 
-int adkv_abi_version(void) { return 13; }
+int adkv_abi_version(void) { return 14; }
 
 void adkv_set_mha_kernel(int use_matrix_cores)
 {
@@ -2464,6 +2543,41 @@ int adkv_softmax(const void *logits, void *weights, const void *mask,
 {
     return adkv_softmax_ex(logits, weights, mask, rows, n, 0, rows_per_mask_row, scaling, nullptr, 0,
                            stream);
+}
+
+int adkv_rope_qk(const void *q, const void *k, const void *cos, const void *sin, void *q_out, void *k_out,
+                 int B, int Hq, int H, int T, int D,
+                 int64_t q_sb, int64_t q_sh, int64_t q_st, int64_t k_sb, int64_t k_sh, int64_t k_st,
+                 int64_t cs_sb, int64_t cs_st, int bf16, void *stream)
+{
+    if (!q || !k || !cos || !sin || !q_out || !k_out)
+        return ADKV_E_NULL;
+    if (B <= 0 || Hq <= 0 || H <= 0 || T <= 0 || D <= 0 || (D & 3))
+        return ADKV_E_SHAPE;
+    // 4-byte accesses: every base and every stride a multiple of two elements
+    if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)cos | (uintptr_t)sin | (uintptr_t)q_out | (uintptr_t)k_out) & 3)
+        return ADKV_E_ALIGN;
+    if ((q_sb | q_sh | q_st | k_sb | k_sh | k_st | cs_sb | cs_st) & 1)
+        return ADKV_E_ALIGN;
+    if ((long)(Hq + H) * (D >> 2) > (long)INT32_MAX)
+        return ADKV_E_SHAPE;
+    const RopeSide qs = {(const uint16_t *)q, (uint16_t *)q_out, (long)q_sb, (long)q_sh, (long)q_st, Hq};
+    const RopeSide ks = {(const uint16_t *)k, (uint16_t *)k_out, (long)k_sb, (long)k_sh, (long)k_st, H};
+    const unsigned gx = (unsigned)(((long)(Hq + H) * (D >> 2) + 255) / 256);
+    constexpr int GMAX = 65535; // grid limit of the token and batch axes: longer ones take several launches
+    for (int b0 = 0; b0 < B; b0 += GMAX)
+        for (int t0 = 0; t0 < T; t0 += GMAX) {
+            const dim3 grid(gx, (unsigned)min(T - t0, GMAX), (unsigned)min(B - b0, GMAX));
+            if (bf16)
+                hipLaunchKernelGGL(rope_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, qs, ks,
+                                   (const uint16_t *)cos, (const uint16_t *)sin, (long)cs_sb, (long)cs_st, T, D,
+                                   t0, b0);
+            else
+                hipLaunchKernelGGL(rope_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, qs, ks,
+                                   (const uint16_t *)cos, (const uint16_t *)sin, (long)cs_sb, (long)cs_st, T, D,
+                                   t0, b0);
+        }
+    return check_launch();
 }
 
 static int64_t pad256(int64_t n) { return (n + 255) & ~(int64_t)255; }

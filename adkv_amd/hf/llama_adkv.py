@@ -23,6 +23,7 @@ from transformers.models.llama.modeling_llama import (
 )
 from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
 
+from ..kernel.gemv import rope_qk
 from .cache import (CAP_LEN, INIT_SEQ_LEN, SCALE_MAX, SCALE_MIN, KVCache_ADKV,  # noqa: F401
                     KVCacheLayer_ADKV)
 
@@ -63,7 +64,12 @@ class LlamaAttention_ADKV(LlamaAttention):
         k = self.k_proj(hidden_states).view(split).transpose(1, 2)
         v = self.v_proj(hidden_states).view(split).transpose(1, 2)
         cos, sin = position_embeddings
-        q, k = apply_rotary_pos_emb(q, k, cos, sin)
+        if (q.is_cuda and q.dtype in (torch.float16, torch.bfloat16) and cos.dtype == q.dtype
+                and cos.dim() == 3 and self.head_dim % 4 == 0):
+            # one launch instead of apply_rotary_pos_emb's ten, same values bit for bit
+            q, k = rope_qk(q, k, cos, sin)
+        else:
+            q, k = apply_rotary_pos_emb(q, k, cos, sin)
 
         layer_cache = None
         if use_cache and past_key_values is not None:

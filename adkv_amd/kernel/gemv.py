@@ -440,6 +440,47 @@ def append_kv_pair(
     _lib.check(rc, "append_kv_pair")
 
 
+def rope_qk(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor
+            ) -> tuple[torch.Tensor, torch.Tensor]:
+    """Rotary position embedding of ``q [B, Hq, T, D]`` and ``k [B, H, T, D]`` in one launch.
+
+    Bit-identical to ``transformers``' ``apply_rotary_pos_emb(q, k, cos, sin)`` as the attention
+    module calls it (src/adkv/hf/llama_adkv.py:336-338): ``x*cos + rotate_half(x)*sin`` with each
+    of the three operations rounded to the tensors' type.  fp16 or bf16, all four tensors of one
+    type; ``cos`` / ``sin``: ``[B, T, D]`` (or ``[1, T, D]``).  Any batch / head / token strides with
+    contiguous channels are read in place; the results are contiguous.
+    """
+    _chk(q.dim() == 4 and k.dim() == 4 and cos.dim() == 3 and sin.dim() == 3,
+         "q, k must be [B, H, T, D] and cos, sin [B, T, D]")
+    B, Hq, T, D = q.shape
+    H = k.shape[1]
+    _chk(k.shape[0] == B and k.shape[2] == T and k.shape[3] == D, "q and k disagree in shape")
+    _chk(q.dtype in (torch.float16, torch.bfloat16), "q must be float16 or bfloat16")
+    _chk(k.dtype == q.dtype and cos.dtype == q.dtype and sin.dtype == q.dtype,
+         "q, k, cos, sin must share one dtype")
+    _chk(cos.shape == sin.shape and cos.shape[1] == T and cos.shape[2] == D and cos.shape[0] in (1, B),
+         "cos, sin must be [B, T, D] or [1, T, D]")
+    _chk(D % 4 == 0 and B * Hq * T * D > 0, "head dim must be a positive multiple of 4")
+    dev = _need_device(q, k, cos, sin)
+
+    def rows(t):        # channels contiguous, even strides, 4-byte aligned base: read in place
+        ok = t.stride(-1) == 1 and all(st % 2 == 0 for st in t.stride()[:-1]) and t.data_ptr() % 4 == 0
+        return t if ok else t.contiguous()
+    q_, k_, c_, s_ = rows(q), rows(k), rows(cos), rows(sin)
+    if s_.stride() != c_.stride():
+        c_, s_ = c_.contiguous(), s_.contiguous()
+    q_out = torch.empty((B, Hq, T, D), dtype=q.dtype, device=dev)
+    k_out = torch.empty((B, H, T, D), dtype=q.dtype, device=dev)
+    with _lib.device_guard(dev):
+        rc = _lib.lib().adkv_rope_qk(
+            q_.data_ptr(), k_.data_ptr(), c_.data_ptr(), s_.data_ptr(), q_out.data_ptr(), k_out.data_ptr(),
+            B, Hq, H, T, D, q_.stride(0), q_.stride(1), q_.stride(2), k_.stride(0), k_.stride(1), k_.stride(2),
+            c_.stride(0) if c_.shape[0] == B and B > 1 else 0, c_.stride(1),
+            1 if q.dtype == torch.bfloat16 else 0, _lib.current_stream_ptr(dev))
+    _lib.check(rc, "rope_qk")
+    return q_out, k_out
+
+
 def softmax_scale_mask(logits: torch.Tensor, scaling: float,
                        mask: torch.Tensor | None = None) -> torch.Tensor:
     """``softmax(logits.float()*scaling + mask) -> fp16`` in one launch.

@@ -316,6 +316,22 @@ int adkv_quant_f32(const void *x, void *xhat, void *codes, void *zp_state, void 
                    int B, int T, int C, int64_t stride_b, int64_t stride_t, int x_dtype,
                    int lower_limit, int upper_limit, float sc_min, float sc_max, void *stream);
 
+/*
+ * Rotary position embedding of the query and key rows in one launch: x * cos + rotate_half(x) * sin
+ * with every operation rounded to the activations' type as torch rounds it, bit-identical to
+ * transformers' apply_rotary_pos_emb that the attention module calls before the cache
+ * (src/adkv/hf/llama_adkv.py:336-338; ten elementwise launches there).
+ *   q [B, Hq, T, D], k [B, H, T, D]: fp16 (bf16 = 0) or bfloat16 (bf16 = 1), channels contiguous,
+ *       element strides over batch / head / token given (the [B, T, H*D] projection output viewed
+ *       head-first needs no copy);  cos, sin [B, T, D] in the same type, strides over batch / token
+ *       (0 over the batch for a shared table);  q_out, k_out: contiguous [B, Hq, T, D] / [B, H, T, D].
+ *   D a multiple of 4; every pointer 4-byte aligned and every stride even.
+ */
+int adkv_rope_qk(const void *q, const void *k, const void *cos, const void *sin, void *q_out, void *k_out,
+                 int B, int Hq, int H, int T, int D,
+                 int64_t q_sb, int64_t q_sh, int64_t q_st, int64_t k_sb, int64_t k_sh, int64_t k_st,
+                 int64_t cs_sb, int64_t cs_st, int bf16, void *stream);
+
 /* ---- comparator, not part of the drop-in boundary ----
  * fp16-KV single-query attention (split-K flash decoding), standing in for the uncompressed fp16
  * cache that ADKV's memory and latency claims are made against (tools/memory_comparison_fig.py:46-56

@@ -569,3 +569,36 @@ def test_cache_layer_grouped_queries_two_bit_and_bf16(gpu, oracle, bits, G, dtyp
         n = oracle.n_super(T0 + steps)
     assert np.array_equal(layer.key_states.cpu().numpy()[:, :, :n], ko[:, :, :n])
     assert np.array_equal(layer.value_states.cpu().numpy()[:, :, :n], vo[:, :, :n])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,Hq,H,T,D,shared_table", [(3, 4, 2, 1, 128, False), (2, 8, 8, 5, 64, True),
+                                                     (1, 2, 1, 33, 256, False), (130, 32, 32, 1, 128, False),
+                                                     (1, 1, 1, 65537, 8, True)])
+def test_rope_equals_transformers_bit_for_bit(gpu, dtype, B, Hq, H, T, D, shared_table):
+    """The one-launch rotary embedding returns the very bits of transformers' apply_rotary_pos_emb
+    (what the reference's attention module calls, llama_adkv.py:336-338) on the same device and
+    type: projection-shaped inputs read through their head-first views, values spread over the
+    type's range so that products land on rounding ties, small and subnormal results included."""
+    from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
+    from adkv_amd.kernel import gemv
+    g = torch.Generator().manual_seed(B * 1000 + T * 10 + D)
+    scale = torch.tensor([1.0, 37.5, 2.0 ** -9, 2.0 ** -13])[torch.randint(0, 4, (B, T, 1), generator=g)]
+    qp = (torch.randn(B, T, Hq * D, generator=g) * scale).to(dtype).to(gpu)
+    kp = (torch.randn(B, T, H * D, generator=g) * scale).to(dtype).to(gpu)
+    q = qp.view(B, T, Hq, D).transpose(1, 2)
+    k = kp.view(B, T, H, D).transpose(1, 2)
+    pos = torch.rand(1 if shared_table else B, T, 1, generator=g) * 4000.0
+    inv = 10000.0 ** (-torch.arange(0, D, 2).float() / D)
+    ang = torch.cat([pos * inv, pos * inv], dim=-1)
+    cos, sin = ang.cos().to(dtype).to(gpu), ang.sin().to(dtype).to(gpu)
+    want_q, want_k = apply_rotary_pos_emb(q, k, cos, sin)
+    got_q, got_k = gemv.rope_qk(q, k, cos, sin)
+    assert got_q.is_contiguous() and got_k.is_contiguous()
+    as_bits = lambda t: t.contiguous().view(torch.int16).cpu()
+    assert torch.equal(as_bits(got_q), as_bits(want_q))
+    assert torch.equal(as_bits(got_k), as_bits(want_k))
+    # packed inputs and a table that is a slice (odd storage offset in bytes / 4 is fine, strides even)
+    got_q2, _ = gemv.rope_qk(q.contiguous(), k.contiguous(), cos, sin)
+    assert torch.equal(as_bits(got_q2), as_bits(want_q))
