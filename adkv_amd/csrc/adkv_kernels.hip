@@ -1146,7 +1146,7 @@ __global__ __launch_bounds__(256) void ov_finalize_wide_kernel(const float *__re
 }
 
 // ---------------------------------------------------------------------------------------------
-// Rotary position embedding of q and k in one launch   (llama_adkv.py:336-338 calls transformers'
+// Rotary position embedding of q and k in one launch   (llama_adkv.py:336-337 calls transformers'
 // apply_rotary_pos_emb: x * cos + rotate_half(x) * sin, ten elementwise launches)
 // ---------------------------------------------------------------------------------------------
 // Every operation is rounded to the activations' type the way torch's elementwise kernels round

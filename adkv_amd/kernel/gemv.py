@@ -445,7 +445,7 @@ def rope_qk(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tens
     """Rotary position embedding of ``q [B, Hq, T, D]`` and ``k [B, H, T, D]`` in one launch.
 
     Bit-identical to ``transformers``' ``apply_rotary_pos_emb(q, k, cos, sin)`` as the attention
-    module calls it (src/adkv/hf/llama_adkv.py:336-338): ``x*cos + rotate_half(x)*sin`` with each
+    module calls it (src/adkv/hf/llama_adkv.py:336-337): ``x*cos + rotate_half(x)*sin`` with each
     of the three operations rounded to the tensors' type.  fp16 or bf16, all four tensors of one
     type; ``cos`` / ``sin``: ``[B, T, D]`` (or ``[1, T, D]``).  Any batch / head / token strides with
     contiguous channels are read in place; the results are contiguous.

@@ -320,7 +320,7 @@ int adkv_quant_f32(const void *x, void *xhat, void *codes, void *zp_state, void 
  * Rotary position embedding of the query and key rows in one launch: x * cos + rotate_half(x) * sin
  * with every operation rounded to the activations' type as torch rounds it, bit-identical to
  * transformers' apply_rotary_pos_emb that the attention module calls before the cache
- * (src/adkv/hf/llama_adkv.py:336-338; ten elementwise launches there).
+ * (src/adkv/hf/llama_adkv.py:336-337; ten elementwise launches there).
  *   q [B, Hq, T, D], k [B, H, T, D]: fp16 (bf16 = 0) or bfloat16 (bf16 = 1), channels contiguous,
  *       element strides over batch / head / token given (the [B, T, H*D] projection output viewed
  *       head-first needs no copy);  cos, sin [B, T, D] in the same type, strides over batch / token

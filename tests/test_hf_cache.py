@@ -578,7 +578,7 @@ def test_cache_layer_grouped_queries_two_bit_and_bf16(gpu, oracle, bits, G, dtyp
                                                      (1, 1, 1, 65537, 8, True)])
 def test_rope_equals_transformers_bit_for_bit(gpu, dtype, B, Hq, H, T, D, shared_table):
     """The one-launch rotary embedding returns the very bits of transformers' apply_rotary_pos_emb
-    (what the reference's attention module calls, llama_adkv.py:336-338) on the same device and
+    (what the reference's attention module calls, llama_adkv.py:336-337) on the same device and
     type: projection-shaped inputs read through their head-first views, values spread over the
     type's range so that products land on rounding ties, small and subnormal results included."""
     from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
