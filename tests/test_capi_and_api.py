@@ -77,6 +77,19 @@ def test_paired_append_and_fused_decode_validation_needs_no_device():
     assert L.adkv_decode_step(*fused) == -6                                # activation dtype must be f16 / bf16
 
 
+def test_rotary_embedding_validation_needs_no_device():
+    """adkv_rope_qk rejects NULL pointers, head dims that are no multiple of 4, unaligned bases and
+    odd strides on the host, before any launch."""
+    L = _lib.lib()
+    one = ctypes.c_void_p(16)
+    rope = lambda ptrs=None, D=128, strides=None: (ptrs or [one] * 6) + [2, 4, 2, 1, D] + \
+        (strides or [4 * D, D, 4 * D, 2 * D, D, 2 * D, D, D]) + [0, None]
+    assert L.adkv_rope_qk(*rope(ptrs=[one, None, one, one, one, one])) == -1
+    assert L.adkv_rope_qk(*rope(D=126)) == -3
+    assert L.adkv_rope_qk(*rope(ptrs=[ctypes.c_void_p(18)] + [one] * 5)) == -5
+    assert L.adkv_rope_qk(*rope(strides=[513, 128, 512, 256, 128, 256, 128, 128])) == -5
+
+
 def test_row_strides_of_projection_outputs():
     """A [B, T, H, D] projection output viewed head-first is handed over with its strides; layouts
     the library cannot read in place (odd strides, channel stride 2) are packed first."""
