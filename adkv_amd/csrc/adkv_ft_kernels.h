@@ -83,23 +83,14 @@ __device__ __forceinline__ uint2 ft_get(const uint2 *tab, uint32_t bytes, uint32
     // [0, j, bytes.byte[k], lane*8]: selector bytes 0-3 pick from lane_copy, 4-7 from bytes, 0x0C is zero
     const uint32_t sel = (j ? 0x0C010000u : 0x0C0C0000u) | ((4u + (uint32_t)k) << 8);
     const uint32_t addr = __builtin_amdgcn_perm(bytes, lane_copy, sel);
-#ifdef ADKV_ABLATE_NO_LOOKUP
-    return make_uint2(addr | 0x3c003c00u, 0x3c003c00u); // timing only: no LDS read, results are wrong
-#else
     return *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(tab) + addr);
-#endif
 }
 
-// Which supergroup the main loops prefetch.  ADKV_ABLATE_CODE_WINDOW=m (a measurement aid, see
-// tools/ablate.py; results are wrong) keeps every unit inside its first m+1 supergroups, so the
-// same instruction stream runs with its code bytes coming from a cache instead of from HBM.
+// Which supergroup the main loops prefetch: PF ahead, clamped to the segment's last one (the load
+// is unconditional; a load inside a branch makes the next wait cover every load in flight).
 __device__ __forceinline__ int ft_prefetch_index(int sg, int nfull)
 {
-#ifdef ADKV_ABLATE_CODE_WINDOW
-    return min(sg & (ADKV_ABLATE_CODE_WINDOW), nfull - 1);
-#else
     return min(sg + PF, nfull - 1);
-#endif
 }
 
 // The main loop needs zp, sc and alpha only (the table holds what beta and the target give); the
@@ -286,9 +277,9 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
 // forward_ov  (gemv.cu:946-1178), per-head table
 // ---------------------------------------------------------------------------------------------
 //
-// MM != 0: the contraction runs on the matrix cores.  v_mfma_f32_4x4x4_16B_f16 multiplies, in each
-// group of four lanes, the 4x4 matrix whose row i is lane i's A operand with the matrix whose
-// column r is lane r's B operand, and lane r receives column r of the product.  With
+// The contraction runs on the matrix cores.  v_mfma_f32_4x4x4_16B_f16 multiplies, in each group of
+// four lanes, the 4x4 matrix whose row i is lane i's A operand with the matrix whose column r is
+// lane r's B operand, and lane r receives column r of the product.  With
 //   B of lane r = (x_A[t], x_B[t], x_A[t+1], x_B[t+1])   the lane's channel pair at two tokens, which
 //                                                        is two consecutive registers as they are,
 //   A of lane 0 = (w[t], 0, w[t+1], 0),  A of lane 1 = (0, w[t], 0, w[t+1]),  A of lanes 2, 3 = 0,
@@ -296,14 +287,12 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
 // outputs, nothing crosses lanes, products exact and sums in fp32 as in the vector form.  One
 // instruction per (pair, two tokens) replaces four mixed-precision multiply-adds; a matrix
 // instruction takes one issue slot and then runs beside the vector pipe.  The weights reach the A
-// layout with two v_perm_b32 per token pair and per-lane selectors.
-//   MM == 2 (shipped): x = r16(q*sc + zp), the reference's dequantised value (gemv.cu:1085-1086).
-//   MM == 1: the product is linear, so one instruction takes the two q*sc registers and a second
-//   one the two zero-points and the packed add goes as well; outputs then differ by the skipped
-//   roundings (up to half an fp16 ulp of the largest value), for 1 % of the kernel's time.
+// layout with two v_perm_b32 per token pair and per-lane selectors.  x = r16(q*sc + zp), the
+// reference's dequantised value (gemv.cu:1085-1086).  (The product is linear, so contracting q*sc
+// and zp separately would save the packed add; the outputs would then lack that rounding, up to
+// half an fp16 ulp of the largest value, for 1 % of the kernel's time: not done.)
 // A non-finite cached value makes both outputs of its channel PAIR non-finite (0 * inf inside the
-// product); the vector form confines it to its own channel.
-template <int MM>
+// product); the vector form of ov_kernel's two-channel lanes confines it to its own channel.
 __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
     const h1 *__restrict__ attn, uint4 *__restrict__ cache, const h1 *__restrict__ v_new,
     h1 *__restrict__ out, float *__restrict__ partial,
@@ -368,50 +357,25 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
         }
         return;
     }
-    auto token = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2], const uint4 wv) {
-        const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
-        const h2 wp = as_h2(ww[t >> 1]);
-        const float wt = (t & 1) ? (float)wp.y : (float)wp.x;
-#pragma unroll
-        for (int p = 0; p < G::NP; p++) {
-            Pair &s = st[p];
-            const h2 qs = as_h2(e[p][t].x) * s.sc;
-            const h2 vd = qs + s.zp;
-            acc[2 * p] = __builtin_fmaf(wt, (float)vd.x, acc[2 * p]);
-            acc[2 * p + 1] = __builtin_fmaf(wt, (float)vd.y, acc[2 * p + 1]);
-            update_pair_f(s, as_h2(e[p][t].y), qs);
-        }
-#pragma unroll
-        for (int p = 0; p < G::NP; p++)
-            e[p][t] = ft_get(tab, nb[p][t & 1], lane_copy, t >> 1, p);
-        __builtin_amdgcn_sched_barrier(0);
-    };
-
     // two tokens of the current supergroup on the matrix cores, then the lookups of the same two
     // slots of the next one
     auto token2 = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2], const uint4 wv) {
         const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
         const uint32_t w2 = ww[t >> 1];
         const h4v a = as_h4(__builtin_amdgcn_perm(w2, w2, sel_a0), __builtin_amdgcn_perm(w2, w2, sel_a1));
-        uint32_t qs[G::NP][2], z[G::NP][2];
+        uint32_t vd[G::NP][2];
 #pragma unroll
         for (int k = 0; k < 2; k++)
 #pragma unroll
             for (int p = 0; p < G::NP; p++) {
                 Pair &s = st[p];
-                const h2 x = as_h2(e[p][t + k].x) * s.sc;
-                qs[p][k] = as_u32(MM == 2 ? x + s.zp : x);
-                z[p][k] = as_u32(s.zp);
-                update_pair_f(s, as_h2(e[p][t + k].y), x);
+                const h2 qs = as_h2(e[p][t + k].x) * s.sc;
+                vd[p][k] = as_u32(qs + s.zp);
+                update_pair_f(s, as_h2(e[p][t + k].y), qs);
             }
 #pragma unroll
         for (int p = 0; p < G::NP; p++)
-            acc4[p] = __builtin_amdgcn_mfma_f32_4x4x4f16(a, as_h4(qs[p][0], qs[p][1]), acc4[p], 0, 0, 0);
-        if (MM == 1) {
-#pragma unroll
-            for (int p = 0; p < G::NP; p++)
-                acc4[p] = __builtin_amdgcn_mfma_f32_4x4x4f16(a, as_h4(z[p][0], z[p][1]), acc4[p], 0, 0, 0);
-        }
+            acc4[p] = __builtin_amdgcn_mfma_f32_4x4x4f16(a, as_h4(vd[p][0], vd[p][1]), acc4[p], 0, 0, 0);
 #pragma unroll
         for (int k = 0; k < 2; k++)
 #pragma unroll
@@ -436,24 +400,16 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
         const int sgp = ft_prefetch_index(sg, nfull);
         buf[i][0] = cb[(size_t)sgp * G::VPS];
         __builtin_amdgcn_sched_barrier(0);
-        if (MM) {
 #pragma unroll
-            for (int t = 0; t < 8; t += 2)
-                token2(t, lk, nb, wbuf[i]);
-        } else {
-#pragma unroll
-            for (int t = 0; t < 8; t++)
-                token(t, lk, nb, wbuf[i]);
-        }
+        for (int t = 0; t < 8; t += 2)
+            token2(t, lk, nb, wbuf[i]);
         wbuf[i] = load_w(sgp); // reloaded once its last token is done (see ov_kernel)
     };
     rotate_over<PF>(nfull, body);
-    if (MM) {
 #pragma unroll
-        for (int p = 0; p < G::NP; p++) {
-            acc[2 * p] = acc4[p].x;
-            acc[2 * p + 1] = acc4[p].y;
-        }
+    for (int p = 0; p < G::NP; p++) {
+        acc[2 * p] = acc4[p].x;
+        acc[2 * p + 1] = acc4[p].y;
     }
 
     if (last) {

@@ -30,19 +30,7 @@
 
 namespace adkv {
 
-#ifndef ADKV_PF
-#define ADKV_PF 4
-#endif
-constexpr int PF = ADKV_PF; // supergroups in flight per lane
-// How the per-head-table OV kernel contracts: 2 = on the matrix cores over the rounded dequantised
-// values (shipped); 1 = on the matrix cores over q*sc and zp separately, without their fp16 sum;
-// 0 = vector form.  0 and 1 are built by tools/ablate.py only.
-#ifndef ADKV_FT_OV_MM
-#define ADKV_FT_OV_MM 2
-#endif
-#ifndef ADKV_MFMA_DEFAULT
-#define ADKV_MFMA_DEFAULT 0
-#endif
+constexpr int PF = 4; // supergroups in flight per lane (2, 6 and 8 were measured: no difference)
 
 template <int D, int CPL>
 struct Geo {
@@ -1818,7 +1806,7 @@ static int mha_kernel_default()
 {
     static const int from_env = [] {
         const char *e = getenv("ADKV_MFMA");
-        return (e ? atoi(e) : ADKV_MFMA_DEFAULT) != 0 ? 1 : 0;
+        return (e ? atoi(e) : 0) != 0 ? 1 : 0;
     }();
     return from_env;
 }
@@ -1860,17 +1848,6 @@ static bool use_head_table(int B, int H, int GQ, int bits, int D, const Seg &seg
     else
         t_shared = (double)((waves_shared + N_SIMD - 1) / N_SIMD) / WAVES_PER_SIMD_TARGET;
     return t_ft <= t_shared;
-}
-
-// ADKV_ENCODE_CPL=1/2 pins the encoder's channels per lane (a measurement aid); read once.
-static int encode_cpl_override()
-{
-    static const int from_env = [] {
-        const char *e = getenv("ADKV_ENCODE_CPL");
-        const int v = e ? atoi(e) : 0;
-        return (v == 1 || v == 2) ? v : 0;
-    }();
-    return from_env;
 }
 
 static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval, int bits = 4)
@@ -1980,8 +1957,6 @@ static int encode_common(void *cache, const void *kv_new,
     const long channels = (long)BH * D;
     const long tensors = second ? 2 : 1;
     int cpl = tensors * channels > 2L * 64 * N_SIMD + 32768 ? 2 : 1;
-    if (const int forced = encode_cpl_override())
-        cpl = forced;
     const long lanes = channels / cpl;
     const dim3 grid((unsigned)((lanes + 255) / 256), (unsigned)tensors), block(256);
     EncTensor first;
@@ -2268,22 +2243,25 @@ static int forward_ov_impl(const void *attn, void *v_cache, const void *v_new, v
     seg.act_bf16 = act_bf16;
     if (ld)
         seg.row_pitch = ld;
-    if (seg.nseg > 1) {
+    const bool matrix_cores = D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha());
+    const bool head_table = !matrix_cores && use_head_table(B, H, GQ, bits, D, seg);
+    // per-head table, two or four segments: the waves of one sequence pair sit in the same
+    // workgroup (interleave_segment) and add their partial outputs there; no second launch and
+    // nothing in the workspace
+    seg.combine = (head_table && (seg.nseg == 2 || seg.nseg == 4)) ? 1 : 0;
+    if (seg.nseg > 1 && !seg.combine) {
         if (!workspace || workspace_bytes < (int64_t)seg.nseg * BH * GQ * D * 4)
             return ADKV_E_WORKSPACE;
         if ((uintptr_t)workspace & 15)
             return ADKV_E_ALIGN;
     }
-    if (D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha())) {
+    if (matrix_cores) {
         ADKV_DISPATCH_GQ(ov_gqa_kernel, false, (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new,
                          (h1 *)out, (float *)workspace, (const h1 *)zp, (const h1 *)sc,
                          (const h1 *)alpha, (const h1 *)beta, (const h1 *)tgt, BH, H, T, n_super_cap,
                          (h1 *)state_out, seg);
-    } else if (use_head_table(B, H, GQ, bits, D, seg)) {
-        // two or four segments: the waves of one (sequence pair) sit in the same workgroup
-        // (interleave_segment) and add their partial outputs there, no second launch
-        seg.combine = (seg.nseg == 2 || seg.nseg == 4) ? 1 : 0;
-        hipLaunchKernelGGL(ov_ft_kernel<ADKV_FT_OV_MM>, dim3((unsigned)(H * ft_wgs_per_head(B, seg.nseg))),
+    } else if (head_table) {
+        hipLaunchKernelGGL(ov_ft_kernel, dim3((unsigned)(H * ft_wgs_per_head(B, seg.nseg))),
                            dim3(FT_BLK), 0, st, (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new, (h1 *)out,
                            (float *)workspace, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,
                            (const h1 *)beta, (const h1 *)tgt, B, H, T, n_super_cap, (h1 *)state_out, seg);
@@ -2370,10 +2348,19 @@ int adkv_forward_ov_noalloc(const void *attn, void *v_cache, const void *v_new, 
                             void *stream)
 {
     // what the segment plan of this launch needs, priced before anything touches the device
+    // (nothing when the kernel adds its two or four segments inside the workgroup)
     int64_t need = 0;
     if (ckpt != nullptr && B > 0 && H > 0 && Hq > 0 && Hq % H == 0 && T >= 0 && n_ckpt_cap > 0 &&
-        ckpt_interval > 0)
-        need = adkv_forward_ov_gqa_workspace_bytes(B, Hq, H, T, D, n_ckpt_cap, ckpt_interval);
+        ckpt_interval > 0 && (D == 128 || D == 256 || D == 512)) {
+        int dummy = 0;
+        const Seg seg = plan_segments(&dummy, n_ckpt_cap, ckpt_interval, B * H, T, D);
+        const int GQ = Hq / H;
+        const bool matrix_cores = D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha());
+        const bool in_workgroup = !matrix_cores && (seg.nseg == 2 || seg.nseg == 4) &&
+                                  use_head_table(B, H, GQ, bits, D, seg);
+        if (seg.nseg > 1 && !in_workgroup)
+            need = (int64_t)seg.nseg * B * Hq * D * 4;
+    }
     if (need > adkv_static_scratch_bytes())
         return ADKV_E_SCRATCH_LIMIT;
     float *ws = nullptr;

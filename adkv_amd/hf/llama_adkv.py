@@ -64,9 +64,12 @@ class LlamaAttention_ADKV(LlamaAttention):
         k = self.k_proj(hidden_states).view(split).transpose(1, 2)
         v = self.v_proj(hidden_states).view(split).transpose(1, 2)
         cos, sin = position_embeddings
+        wants_grad = torch.is_grad_enabled() and (q.requires_grad or k.requires_grad)
         if (q.is_cuda and q.dtype in (torch.float16, torch.bfloat16) and cos.dtype == q.dtype
-                and cos.dim() == 3 and self.head_dim % 4 == 0):
-            # one launch instead of apply_rotary_pos_emb's ten, same values bit for bit
+                and cos.dim() == 3 and self.head_dim % 4 == 0 and not wants_grad):
+            # one launch instead of apply_rotary_pos_emb's ten, same values bit for bit.  The
+            # kernel has no backward pass: whenever autograd is recording, the differentiable
+            # expression the reference calls (llama_adkv.py:336-337) runs instead.
             q, k = rope_qk(q, k, cos, sin)
         else:
             q, k = apply_rotary_pos_emb(q, k, cos, sin)

@@ -55,6 +55,10 @@ def parse():
                          "rocprofv3 FETCH_SIZE/WRITE_SIZE readings by)")
     ap.add_argument("--graph", action="store_true",
                     help="also replay the step from HIP graphs and report that time beside the headline")
+    ap.add_argument("--bf16", action="store_true",
+                    help="decode workload: q, the new token and the output in bfloat16")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="default decode run only: skip the short cfg3 / cfg5 / cfg1 runs reported under `secondary`")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fp16-comparator", action="store_true",
                     help="skip timing the fp16-KV decode kernel beside the ADKV step")
@@ -148,7 +152,7 @@ def fp16_comparator(args, dev, adkv_ms):
             "adkv_speedup": ms / adkv_ms}
 
 
-def encode_main(args):
+def encode_record(args, B, T, steps, warmup, cpu=True):
     """cfg3: one step = prefill-quantise B x ctx tokens of K (one launch); afterwards 256 timed
     single-token appends.  tokens quantised / s = B*ctx / t_prefill."""
     import numpy as np
@@ -158,8 +162,6 @@ def encode_main(args):
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    B = 8 if args.batch == 128 else args.batch
-    T = 32768 if args.ctx == 4096 else args.ctx
     H, D, S = args.heads, args.dim, (args.ckpt_interval or 256)
     n_app = 256
     p = synth.make_params(H, D).to(dev)
@@ -173,18 +175,18 @@ def encode_main(args):
     def prefill():
         gemv.append_kv(cache, xp, *p.astuple(), 0, state, ckpt=ck, ckpt_interval=S)
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         prefill()
     torch.cuda.synchronize()
     marks = []
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         e0, e1 = ev(), ev()
         e0.record(); prefill(); e1.record()
         marks.append((e0, e1))
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    ms_step = wall * 1e3 / args.steps
+    ms_step = wall * 1e3 / steps
     k_ms = sum(a.elapsed_time(b) for a, b in marks) / len(marks)
 
     toks = [x[:, :, T + i:T + i + 1].contiguous() for i in range(n_app)]
@@ -210,10 +212,10 @@ def encode_main(args):
     torch.cuda.synchronize()
     p0, p1 = ev(), ev()
     p0.record()
-    for _ in range(args.steps):
+    for _ in range(steps):
         prefill_pair()
     p1.record(); torch.cuda.synchronize()
-    pair_ms = p0.elapsed_time(p1) / args.steps
+    pair_ms = p0.elapsed_time(p1) / steps
     pair_same = bool(torch.equal(cache_k2[:, :, :T // 8], cache[:, :, :T // 8]))
 
     # bit-exactness of the codes: two sampled heads against the oracle, whole stream
@@ -230,7 +232,7 @@ def encode_main(args):
     res = {
         "metric": "streaming quantiser tokens quantised/sec (B*ctx / prefill time, one K tensor)",
         "value": B * T / (ms_step * 1e-3), "unit": "tokens/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "steps": steps, "warmup": warmup, "ms_per_step": ms_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": f"cfg3 streaming quantise: prefill B={B} H={H} d={D} ctx={T} fp16 -> 4-bit codes, "
@@ -247,7 +249,7 @@ def encode_main(args):
                      # (profiles/encode_cfg3_and_decode_cfg5_pmc_traffic.md); default workload only
                      "traffic": 2.7015e9 if (B, H, D, T, S) == (8, 32, 128, 32768, 256) else None},
     }
-    if not args.no_cpu_baseline:
+    if cpu:
         hs, Ts = 2, 4096
         xs = np16(x[:1, :hs, :Ts])
         c = O.alloc_cache(1, hs, Ts, D)
@@ -257,10 +259,10 @@ def encode_main(args):
         res["cpu_baseline"] = {"value": Ts / (dt * H / hs), "unit": "tokens/s", "cores": 1, "kind": "port",
                                "sample": f"C oracle encode, 1 sequence x {hs} of {H} heads x {Ts} tokens "
                                          f"in {dt:.2f} s; scaled linearly to {H} heads"}
-    print(json.dumps(res))
+    return res
 
 
-def quant_f32_main(args):
+def quant_f32_record(args, B, T, steps, warmup):
     """cfg1: the fp32 (train / eval) recurrence over one sequence of 32 heads x 128 channels and
     1024 tokens, K-shaped input with outlier channels.  A step is one pass over the sequence."""
     import numpy as np
@@ -270,8 +272,6 @@ def quant_f32_main(args):
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    B = 1 if args.batch == 128 else args.batch
-    T = 1024 if args.ctx == 4096 else args.ctx
     H, D = args.heads, args.dim
     C = H * D
     p = synth.make_params(H, D, dtype=torch.float32)
@@ -289,17 +289,17 @@ def quant_f32_main(args):
         return quant_f32(xg, al, be, tg, -8, 7, smin, smax, zp_state=zp, sc_state=sc,
                          zp_init=zp_i, sc_init=sc_i, out=out, want_codes=True)
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     marks = []
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         e0, e1 = ev(), ev()
         e0.record(); _, codes, _, _ = step(); e1.record()
         marks.append((e0, e1))
     torch.cuda.synchronize()
-    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_step = (time.perf_counter() - t0) * 1e3 / steps
     k_ms = sum(a.elapsed_time(b) for a, b in marks) / len(marks)
 
     from oracle import oracle as O
@@ -314,7 +314,7 @@ def quant_f32_main(args):
     res = {
         "metric": "fp32-recurrence tokens quantised/sec (B*T / pass time, one tensor)",
         "value": B * T / (ms_step * 1e-3), "unit": "tokens/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "steps": steps, "warmup": warmup, "ms_per_step": ms_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": f"cfg1 fp32 recurrence: B={B} T={T} C={C} ({H} heads x {D}), 4-bit range, "
@@ -327,34 +327,20 @@ def quant_f32_main(args):
         "cpu_baseline": {"value": B * T / cpu_s, "unit": "tokens/s", "cores": 1, "kind": "port",
                          "sample": f"C oracle adkv_o_quant_f32 over the whole workload in {cpu_s:.2f} s"},
     }
-    print(json.dumps(res))
+    return res
 
 
-def main():
-    args = parse()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build measures one GPU only (the path shards over batch/heads with no "
-              "exchange; nothing multi-GPU is built). Run with --gpus 1.", file=sys.stderr)
-        sys.exit(2)
-
-    if args.workload == "encode":
-        return encode_main(args)
-    if args.workload == "quant_f32":
-        return quant_f32_main(args)
-
+def decode_record(args, B, Hq, H, D, T, bits, S, NL, steps, warmup, headline=True, bf16=False):
+    """Times `steps` decode_step calls (the product path) over NL rotating layer caches and returns
+    the bench record.  headline=False leaves out the comparator, the CPU baseline and the graph
+    replay (the secondary records of the default run)."""
     import torch
     from adkv_amd import synth
     from adkv_amd.kernel import gemv
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    B, Hq, D, T = args.batch, args.heads, args.dim, args.ctx
-    H = args.kv_heads or Hq          # KV heads own the caches and parameters
-    smin, smax = math.exp(-4.0), math.exp(4.0)
-    NL = args.layer_buffers
-
-    S = args.ckpt_interval
-    bits = args.bits
+    act = torch.bfloat16 if bf16 else torch.float16   # q, the new token and the output
     ncap = T // S + 1 if S else 0
     kps, vps, kcs, vcs, kks, vks = [], [], [], [], [], []
     state = torch.zeros(B, H, D, 2, dtype=torch.float16, device=dev)
@@ -375,14 +361,14 @@ def main():
         kks.append(kk); vks.append(vk)
         if NL > 8:
             torch.cuda.empty_cache()   # many resident layer caches: keep the input scratch from fragmenting
-    q = synth.make_q(B, Hq, D, device=dev)
-    k_new = synth.make_k(B, H, 1, D, seed=11, dtype=torch.float16, device=dev, t0=T)
-    v_new = synth.make_v(B, H, 1, D, seed=12, dtype=torch.float16, device=dev)
+    q = synth.make_q(B, Hq, D, device=dev).to(act)
+    k_new = synth.make_k(B, H, 1, D, seed=11, dtype=torch.float16, device=dev, t0=T).to(act)
+    v_new = synth.make_v(B, H, 1, D, seed=12, dtype=torch.float16, device=dev).to(act)
     scaling = D ** -0.5
     torch.cuda.synchronize()
     torch.cuda.empty_cache()
 
-    if args.calibrate_copy:
+    if args.calibrate_copy and headline:
         a = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
         b = torch.empty_like(a)
         for _ in range(3):
@@ -403,25 +389,25 @@ def main():
 
     # four events per timed step, recorded by the library around the stages of the fused call
     marks = []
-    for _ in range(args.steps):
+    for _ in range(steps):
         e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
         for x in e:
             x.record()                     # creates the underlying hipEvent_t
         marks.append(e)
     arr4 = _lib.C.c_void_p * 4
 
-    for i in range(args.warmup):
+    for i in range(warmup):
         fused(i % NL)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
+    for i in range(steps):
         L.adkv_set_stage_events(arr4(*[x.cuda_event for x in marks[i]]))
         fused(i % NL)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     L.adkv_set_stage_events(None)
 
-    ms_step = wall * 1e3 / args.steps
+    ms_step = wall * 1e3 / steps
     qk_ms = sum(e[0].elapsed_time(e[1]) for e in marks) / len(marks)
     sm_ms = sum(e[1].elapsed_time(e[2]) for e in marks) / len(marks)
     ov_ms = sum(e[2].elapsed_time(e[3]) for e in marks) / len(marks)
@@ -429,7 +415,7 @@ def main():
 
     # the same step replayed from HIP graphs (one per layer cache): no host work between launches
     graph_ms = None
-    if args.graph:
+    if args.graph and headline:
         graphs = []
         side = torch.cuda.Stream()
         for l in range(NL):
@@ -441,14 +427,14 @@ def main():
                     fused(l)
             graphs.append(g)
         torch.cuda.synchronize()
-        for i in range(args.warmup):
+        for i in range(warmup):
             graphs[i % NL].replay()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for i in range(args.steps):
+        for i in range(steps):
             graphs[i % NL].replay()
         torch.cuda.synchronize()
-        graph_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        graph_ms = (time.perf_counter() - t0) * 1e3 / steps
 
     code_bytes = B * H * T * D * bits / 8.0             # one tensor's codes: bytes per QK launch
     achieved = code_bytes / (qk_ms * 1e-3) / 1e9
@@ -468,8 +454,8 @@ def main():
         "value": tokens_s,
         "unit": "tokens/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": ms_step,
         "higher_is_better": True,
         "scaling": "weak",
@@ -504,13 +490,13 @@ def main():
                         "note": "forward_ov stage incl. the partial-sum kernel"},
     }
     # what the memory system itself delivers for these kernels' access pattern with nothing else
-    # running (tools/hbm_streams, recorded in profiles/hbm_pattern_ceiling.json)
+    # running (a loads-only probe; result and method in profiles/hbm_pattern_ceiling.json)
     try:
         with open(os.path.join(ROOT, "profiles", "hbm_pattern_ceiling.json")) as f:
             ceil = next(iter(json.load(f).values()))
         res["roofline"]["pattern_ceiling"] = {"GBps": ceil["best_GBps"], "frac_of_peak": ceil["best_GBps"] / HBM_PEAK_GBPS,
                                               "achieved_over_ceiling": achieved / ceil["best_GBps"],
-                                              "note": "loads only, same access pattern: python -m adkv_amd.tools.hbm_streams"}
+                                              "note": "loads only, same access pattern; method and table in profiles/decode_cfg2_ablation.md"}
     except (OSError, ValueError, StopIteration, KeyError):
         pass
     if graph_ms is not None:
@@ -532,11 +518,82 @@ def main():
                                     "note": "SQ_INSTS_VALU per launch from profiles/valu_issue.json; duration live"}
     except (OSError, ValueError):
         pass
-    if not args.no_fp16_comparator and D == 128 and H == Hq and bits == 4:
+    if headline and not args.no_fp16_comparator and D == 128 and H == Hq and bits == 4:
         res["fp16_kv_comparator"] = fp16_comparator(args, dev, ms_step)
-    if not args.no_cpu_baseline and H == Hq and bits == 4:
+    if headline and not args.no_cpu_baseline and H == Hq and bits == 4:
         res["cpu_baseline"] = cpu_baseline(args, T, D)
+    del kcs, vcs, kks, vks, ws
+    torch.cuda.empty_cache()
+    return res
+
+
+
+def secondary_records(args):
+    """Short runs of the other named workloads in the same process, so that one default run shows
+    them all: the streaming quantiser (cfg3), the long-context grouped-query 2-bit decode (cfg5) and
+    the fp32 recurrence (cfg1).  Each record is what `--workload ...` prints with fewer steps and
+    without the host baselines; a failure in one is reported in its place and does not touch the
+    headline."""
+    import torch
+    out = {}
+
+    def run(name, fn):
+        try:
+            out[name] = fn()
+        except Exception as e:  # noqa: BLE001 - reported, the headline line must still print
+            out[name] = {"error": f"{type(e).__name__}: {e}"}
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
+
+    def cfg3():
+        r = encode_record(args, 8, 32768, steps=5, warmup=2, cpu=False)
+        return {"workload": r["config"]["workload"], "ms_per_tensor": r["ms_per_step"],
+                "tokens_quantised_per_s": r["value"], "append_us_per_token_step": r["append_us_per_token_step"],
+                "kv_pair": r["kv_pair"], "codes_bit_exact_vs_oracle": r["codes_bit_exact_vs_oracle"],
+                "roofline": r["roofline"]}
+
+    def cfg5():
+        r = decode_record(args, 16, 32, 8, 128, 131072, 2, 256, 2, steps=6, warmup=2, headline=False, bf16=True)
+        return {"workload": r["config"]["workload"], "ms_per_step": r["ms_per_step"], "tokens_per_s": r["value"],
+                "kernel_ms": r["kernel_ms"], "roofline": r["roofline"],
+                **({"roofline_valu": r["roofline_valu"]} if "roofline_valu" in r else {})}
+
+    def cfg1():
+        r = quant_f32_record(args, 1, 1024, steps=20, warmup=3)
+        return {"workload": r["config"]["workload"], "ms_per_pass": r["ms_per_step"], "tokens_per_s": r["value"],
+                "bit_exact_vs_oracle": r["bit_exact_vs_oracle"], "roofline": r["roofline"],
+                "cpu_baseline": r["cpu_baseline"]}
+
+    run("cfg3_streaming_quantiser", cfg3)
+    run("cfg5_long_context_gqa_2bit", cfg5)
+    run("cfg1_fp32_recurrence", cfg1)
+    return out
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (the path shards over batch/heads with no "
+              "exchange; nothing multi-GPU is built). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    if args.workload == "encode":
+        res = encode_record(args, 8 if args.batch == 128 else args.batch, 32768 if args.ctx == 4096 else args.ctx,
+                            args.steps, args.warmup, cpu=not args.no_cpu_baseline)
+    elif args.workload == "quant_f32":
+        res = quant_f32_record(args, 1 if args.batch == 128 else args.batch,
+                               1024 if args.ctx == 4096 else args.ctx, args.steps, args.warmup)
+    else:
+        Hq = args.heads
+        res = decode_record(args, args.batch, Hq, args.kv_heads or Hq, args.dim, args.ctx, args.bits,
+                            args.ckpt_interval, args.layer_buffers, args.steps, args.warmup, bf16=args.bf16)
+        default_shape = (args.batch, Hq, args.kv_heads or Hq, args.dim, args.ctx, args.bits) == \
+            (128, 32, 32, 128, 4096, 4)
+        if default_shape and not args.no_secondary:
+            res["secondary"] = secondary_records(args)
     print(json.dumps(res))
+
+
 
 
 if __name__ == "__main__":

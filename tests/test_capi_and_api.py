@@ -77,6 +77,27 @@ def test_paired_append_and_fused_decode_validation_needs_no_device():
     assert L.adkv_decode_step(*fused) == -6                                # activation dtype must be f16 / bf16
 
 
+def test_static_scratch_entry_points_return_a_code_without_a_device():
+    """adkv_init() and adkv_forward_ov_noalloc resolve the address of the library's static device
+    array with HIP calls.  Where no GPU is present those calls fail; the library must hand that
+    back as ADKV_E_DEVICE (with the HIP code kept for adkv_last_hip_error), never abort.  On a
+    machine with a GPU adkv_init() succeeds and this test has nothing to show."""
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present: adkv_init() succeeds here")
+    L = _lib.lib()
+    rc = L.adkv_init()
+    assert rc == -9 and b"device" in L.adkv_strerror(rc).lower()
+    assert L.adkv_last_hip_error() != 0
+    one = ctypes.c_void_p(256)
+    # a launch that fits the static array: the size check passes, the address lookup reports the failure
+    rc = L.adkv_forward_ov_noalloc(*([one] * 9), 1, 2, 2, 600, 128, 80, 4, 0, None, one, 10, 64, None)
+    assert rc == -9
+    # one that does not fit is refused before any HIP call
+    rc = L.adkv_forward_ov_noalloc(*([one] * 9), 96, 64, 8, 131072, 128, 8200, 4, 0, None, one, 513, 256, None)
+    assert rc == -8
+
+
 def test_rotary_embedding_validation_needs_no_device():
     """adkv_rope_qk rejects NULL pointers, head dims that are no multiple of 4, unaligned bases and
     odd strides on the host, before any launch."""

@@ -391,6 +391,154 @@ def test_tiny_llama_decode_path_matches_oracle_and_dense_model(gpu, oracle, tmp_
         assert err <= 2e-2, (i, err)
 
 
+def _check_decode_calls_in_model_dtype(oracle, model, calls, params16, pad, prompt_len):
+    """_check_decode_calls_against_oracle for a model whose weights are fp16 or bf16: the
+    projections are the module's own linear layers applied to the recorded hidden states and the
+    rotary embedding is the textbook expression evaluated in the model's dtype (each product and
+    the sum rounded to that dtype, as torch's elementwise kernels do), so q, k and v carry exactly
+    the bits the module hands to its cache; they are rounded to fp16 (a no-op for an fp16 model,
+    torch's .to(float16) for a bf16 one: llama_adkv.py:248-250) and given to the oracle.
+    Tolerance on the context that reached o_proj: 2e-3, plus half a bf16 ulp of the value for a
+    bf16 model (the kernel's fp16 result is rounded to bf16 on the way out, llama_adkv.py:274)."""
+    cfg = model.config
+    Hq, H, D = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    G = Hq // H
+    scaling = D ** -0.5
+    dt = model.dtype
+    caches, T = {}, {}
+    n_decode = 0
+    for c in calls:
+        att = model.model.layers[c["layer"]].self_attn
+        hs = c["hidden"]
+        assert hs.dtype == dt
+        B, Tq, _ = hs.shape
+        split = lambda x, n: x.view(B, Tq, n, D).transpose(1, 2)
+        with torch.no_grad():
+            q = _rope(split(att.q_proj(hs), Hq), c["cos"], c["sin"])
+            k = _rope(split(att.k_proj(hs), H), c["cos"], c["sin"])
+            v = split(att.v_proj(hs), H)
+        assert q.dtype == dt and k.dtype == dt
+        q16, k16, v16 = (_np16(t.to(torch.float16)) for t in (q, k, v))
+        kpn, vpn = params16[c["layer"]]
+        if c["layer"] not in caches:
+            assert Tq == prompt_len
+            ko = oracle.alloc_cache(B, H, 256, D)
+            vo = oracle.alloc_cache(B, H, 256, D)
+            oracle.encode_kv_f16(ko, k16, *kpn)
+            oracle.encode_kv_f16(vo, v16, *vpn)
+            caches[c["layer"]], T[c["layer"]] = (ko, vo), Tq
+            continue
+        assert Tq == 1
+        ko, vo = caches[c["layer"]]
+        t = T[c["layer"]]
+        mask = np.zeros((B, 1, t + 1), np.float32)
+        for b in range(B):
+            mask[b, 0, :pad[b]] = -np.inf
+        ctx = np.zeros((B, Hq, D))
+        qn = q16.reshape(B, H, G, D)
+        for j in range(G):
+            kc, vc = ko.copy(), vo.copy()
+            o, _, _ = oracle.decode_step_f16(qn[:, :, j], kc, vc, k16, v16, kpn, vpn, t, scaling, mask=mask)
+            ctx.reshape(B, H, G, D)[:, :, j] = o
+        caches[c["layer"]], T[c["layer"]] = (kc, vc), t + 1
+        got_ctx = c["ctx"].float().cpu().numpy().reshape(B, Hq, D)
+        tol = 2e-3 + (2.0 ** -9 * np.abs(ctx) if dt == torch.bfloat16 else 0.0)
+        assert np.all(np.abs(got_ctx - ctx) <= tol), (c["layer"], t, float(np.max(np.abs(got_ctx - ctx))))
+        want_out = torch.from_numpy(ctx.reshape(B, 1, Hq * D)).float().to(hs.device) @ att.o_proj.weight.detach().float().T
+        assert torch.allclose(c["out"].float(), want_out, atol=5e-3, rtol=2.0 ** -7), (c["layer"], t)
+        n_decode += 1
+    return caches, T, n_decode
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,heads,kv_heads", [(torch.float16, 2, 2), (torch.float16, 4, 2),
+                                                  (torch.bfloat16, 2, 2)])
+def test_tiny_llama_half_precision_decode_path_matches_oracle(gpu, oracle, tmp_path, monkeypatch, dtype,
+                                                              heads, kv_heads):
+    """The attention module on the route a half-precision model takes: the one-launch rotary
+    embedding (adkv_rope_qk) and the branch of KVCacheLayer_ADKV.decode that hands q, k, v to the
+    kernels without a conversion.  Same tiny random-init Llama, left-padded batch and calibration
+    files as the fp32 test above; every decode call of every attention module is recomputed from
+    its input hidden states with the oracle as the attention, and the packed caches at the end
+    are the oracle's byte for byte."""
+    pytest.importorskip("transformers")
+    from adkv_amd import calib
+    from adkv_amd.hf import llama_adkv as M
+
+    cfg = _tiny_cfg(heads, kv_heads)
+    torch.manual_seed(0)
+    model = M.LlamaForCausalLM_ADKV(cfg).to(gpu).to(dtype).eval()
+    H, D = kv_heads, 128
+    raw = _tiny_raw_calibration(2, H * D, seed=11)
+    calib.save_calibration(tmp_path, raw)
+    model.load_adkv_config(calib.load_calibration(tmp_path, 2, hidden_size=H * D))
+    params16 = _deployment_params16(raw, H, D)
+
+    fused_calls = []
+    real_rope = M.rope_qk
+    monkeypatch.setattr(M, "rope_qk", lambda *a, **k: (fused_calls.append(1), real_rope(*a, **k))[1])
+
+    P, new = 12, 8
+    pad = [0, 3]
+    ids = torch.randint(1, 128, (2, P), generator=torch.Generator().manual_seed(3))
+    amask = torch.ones(2, P, dtype=torch.long)
+    for b, n in enumerate(pad):
+        ids[b, :n] = 0
+        amask[b, :n] = 0
+    ids, amask = ids.to(gpu), amask.to(gpu)
+    tap = _AttentionTap(model)
+    with torch.no_grad():
+        out = model.generate(ids, attention_mask=amask, max_new_tokens=new, do_sample=False, pad_token_id=0)
+    tap.close()
+    assert out.shape == (2, P + new)
+    assert len(fused_calls) == 2 * new                   # every attention call took the fused rotary embedding
+    caches, T, n_decode = _check_decode_calls_in_model_dtype(oracle, model, tap.calls, params16, pad, P)
+    assert n_decode == 2 * (new - 1) and all(t == P + new - 1 for t in T.values())
+    cache = tap.cache
+    assert cache is not None and cache.get_seq_length() == P + new - 1
+    n = oracle.n_super(P + new - 1)
+    for L in range(2):
+        assert np.array_equal(cache[L].key_states.cpu().numpy()[:, :, :n], caches[L][0][:, :, :n]), L
+        assert np.array_equal(cache[L].value_states.cpu().numpy()[:, :, :n], caches[L][1][:, :, :n]), L
+
+
+def test_rotary_embedding_keeps_gradients(monkeypatch):
+    """Under autograd the attention module must not take the fused rotary-embedding kernel (it has
+    no backward pass): the differentiable expression runs and q_proj / k_proj receive gradients.
+    Checked on the CPU by making the fused path look eligible and failing the test if it is called."""
+    pytest.importorskip("transformers")
+    from adkv_amd.hf import llama_adkv as M
+
+    def boom(*a, **k):
+        raise AssertionError("fused rotary embedding called while gradients are recorded")
+
+    monkeypatch.setattr(M, "rope_qk", boom)
+    cfg = _tiny_cfg(2, 2)
+    torch.manual_seed(0)
+    model = M.LlamaForCausalLM_ADKV(cfg).to(torch.bfloat16).train()
+    att = model.model.layers[0].self_attn
+
+    ids = torch.randint(1, 128, (1, 6))
+    # `is_cuda` decides the branch; pretend the projections live on a GPU for that test only
+    real_forward = M.LlamaAttention_ADKV.forward
+    seen = []
+
+    def forward(self, hidden_states, *a, **k):
+        seen.append(torch.is_grad_enabled() and hidden_states.requires_grad)
+        return real_forward(self, hidden_states, *a, **k)
+
+    monkeypatch.setattr(M.LlamaAttention_ADKV, "forward", forward)
+    monkeypatch.setattr(torch.Tensor, "is_cuda", property(lambda self: True))
+    try:
+        loss = model(ids, use_cache=False).logits.float().pow(2).mean()
+    finally:
+        monkeypatch.undo()
+    loss.backward()
+    assert seen and all(seen)
+    for lin in (att.q_proj, att.k_proj, att.v_proj, att.o_proj):
+        assert lin.weight.grad is not None and float(lin.weight.grad.float().abs().sum()) > 0.0
+
+
 @pytest.mark.gpu
 def test_tiny_llama_follow_up_chunk_equals_single_token_steps(gpu):
     """A second multi-token call on top of a cache that already holds codes (a follow-up turn):

@@ -89,3 +89,67 @@ def test_noalloc_rejects_launches_beyond_the_static_scratch(gpu):
     assert rc == -8 and b"static" in L.adkv_strerror(rc)
     # the largest benchmark shape (16 sequences, 32 query heads over 8 KV heads, 131072 tokens) fits
     assert L.adkv_forward_ov_gqa_workspace_bytes(16, 32, 8, 131072, 128, 513, 256) <= L.adkv_static_scratch_bytes()
+
+
+def test_noalloc_call_is_capturable_in_a_graph(gpu):
+    """Stream capture fails on any allocation, so capturing one adkv_forward_ov_noalloc call (after
+    adkv_init() has resolved the array's address) shows that the call allocates nothing; every
+    replay, with the program's own eager work between replays, reproduces the eager result."""
+    L = _lib.lib()
+    assert L.adkv_init() == 0
+    c = _case(gpu, B=3, H=4, G=1, T=1031, S=64, bits=4, seed=7)         # 17 segments through the array
+    want = _run(L, c, noalloc=False)
+    dev = c["cache"].device
+    cache0, ck0 = c["cache"].clone(), c["ck"].clone()
+    cache, ck = cache0.clone(), ck0.clone()
+    out = torch.zeros((c["B"], c["Hq"], c["D"]), dtype=torch.float16, device=dev)
+    st = torch.zeros(c["B"], c["H"], c["D"], 2, dtype=torch.float16, device=dev)
+    pp = [t.data_ptr() for t in c["p"].astuple()]
+    head = [c["attn"].data_ptr(), cache.data_ptr(), c["v_new"].data_ptr(), out.data_ptr(), *pp,
+            c["B"], c["Hq"], c["H"], c["T"], c["D"], cache.shape[2], c["bits"], 0,
+            st.data_ptr(), ck.data_ptr(), c["ncap"], c["S"]]
+
+    def call():
+        rc = L.adkv_forward_ov_noalloc(*head, _lib.current_stream_ptr(dev))
+        assert rc == 0, L.adkv_strerror(rc)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()                                          # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for rep in range(3):
+        out.zero_()
+        st.zero_()
+        cache.copy_(cache0)
+        ck.copy_(ck0)
+        graph.replay()
+        junk = (c["attn"].float() * 1.5).sum()          # eager work between replays
+        torch.cuda.synchronize()
+        assert torch.isfinite(junk)
+        for a, b, name in zip((out, cache, ck, st), want, ("out", "cache", "checkpoints", "state")):
+            assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), (rep, name)
+
+
+def test_noalloc_accepts_launches_that_sum_their_segments_in_the_workgroup(gpu):
+    """The per-head-table kernel adds two or four segments inside its workgroups and touches no
+    scratch: such a launch is never refused for its size.  Forced here on a small shape (the
+    kernels take it by themselves only for launches of hundreds of workgroups)."""
+    L = _lib.lib()
+    c = _case(gpu, B=4, H=2, G=1, T=40, S=32, bits=4, seed=8)           # two segments
+    L.adkv_set_mha_kernel(2)
+    try:
+        got = _run(L, c, noalloc=True)
+    finally:
+        L.adkv_set_mha_kernel(-1)
+    # the same launch through the shared-table kernels and a workspace: same codes, state and
+    # checkpoints; outputs one fp16 ulp apart at most (different summation order)
+    want = _run(L, c, noalloc=False)
+    for a, b, name in zip(got[1:], want[1:], ("cache", "checkpoints", "state")):
+        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), name
+    d = (got[0].float() - want[0].float()).abs()
+    assert torch.all(d <= 2.0 ** -10 * torch.clamp(want[0].float().abs(), min=2.0 ** -4))
