@@ -13,7 +13,7 @@ import torch  # noqa: F401  (loads libamdhip64 first)
 
 _DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_DIR, "libadkv_hip.so")
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 _vp, _i, _f = C.c_void_p, C.c_int, C.c_float
 
@@ -47,6 +47,7 @@ PROTOTYPES = {
                                                                             C.c_int64, _vp]),
     "adkv_set_stage_events": (None, [_vp]),
     "adkv_decode_kernel_name": (C.c_char_p, [_i] * 8),
+    "adkv_decode_segments": (_i, [_i] * 8 + [_vp, _i, _vp]),
     "adkv_rope_qk": (_i, [_vp] * 6 + [_i] * 5 + [C.c_int64] * 8 + [_i, _vp]),
     "adkv_quant_f32": (_i, [_vp] * 12 + [_i] * 3 + [C.c_int64, C.c_int64] + [_i] * 3 + [_f, _f, _vp]),
     "adkv_fp16_decode_workspace_bytes": (C.c_int64, [_i] * 3),

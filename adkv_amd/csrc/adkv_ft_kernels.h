@@ -35,15 +35,13 @@ __host__ __device__ inline int ft_wgs_per_head(int B, int nseg)
 }
 
 struct FtUnit {
-    int h, seg, bx, lh, c0;
+    int seg, bx, lh, c0;
     bool active, wave_active;
-    __device__ __forceinline__ FtUnit(int B, int H, int nseg)
+    // h: KV head; vw: virtual workgroup within the head (16 waves' worth of the head's units)
+    __device__ __forceinline__ FtUnit(int B, int H, int nseg, int h, int vw)
     {
         const int pps = ft_pairs_per_seg(B);
-        const int wph = ft_wgs_per_head(B, nseg);
-        h = (int)blockIdx.x / wph;
-        const int w = __builtin_amdgcn_readfirstlane(((int)blockIdx.x % wph) * FT_WAVES +
-                                                     (int)(threadIdx.x >> 6)); // wave within the head
+        const int w = __builtin_amdgcn_readfirstlane(vw * FT_WAVES + (int)(threadIdx.x >> 6)); // wave within the head
         int sg, pair;
         interleave_segment(w, nseg, sg, pair);
         const int lane = threadIdx.x & 63;
@@ -86,6 +84,15 @@ __device__ __forceinline__ uint2 ft_get(const uint2 *tab, uint32_t bytes, uint32
     return *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(tab) + addr);
 }
 
+// The code stream is read exactly once: a non-temporal load keeps it from displacing the logits
+// and weights (which the softmax and the next kernel read back) in the caches.
+typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 ft_load_codes(const uint4 *p)
+{
+    const u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v *>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 // Which supergroup the main loops prefetch: PF ahead, clamped to the segment's last one (the load
 // is unconditional; a load inside a branch makes the next wait cover every load in flight).
 __device__ __forceinline__ int ft_prefetch_index(int sg, int nfull)
@@ -106,7 +113,7 @@ __device__ __forceinline__ void ft_init_pairs(Pair *st, const h1 *zp, const h1 *
         st[p].al = *reinterpret_cast<const h2 *>(al + pi);
     }
     if (seg > 0) {
-        const int j = seg * (sa.seg_tokens / sa.ckpt_interval) - 1;
+        const int j = seg_begin(sa, seg) / sa.ckpt_interval - 1;
         load_state<4>(sa.ckpt + (((size_t)bx * sa.n_ckpt_cap + j) * 128 + c0) * 2, st);
     }
 }
@@ -132,6 +139,11 @@ __device__ __forceinline__ void update_pair_f(Pair &p, h2 f, h2 qs)
 // ---------------------------------------------------------------------------------------------
 // forward_qk  (gemv.cu:435-815), per-head table
 // ---------------------------------------------------------------------------------------------
+//
+// A workgroup serves one head and walks through one or more VIRTUAL workgroups of that head
+// (sa.phys_per_head apart), each 16 waves' worth of (sequence pair, segment) units, without a
+// barrier between them: the table is built once, and a wave that finishes its unit goes straight
+// on to its unit of the next virtual workgroup.
 __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
     const h1 *__restrict__ q, uint4 *__restrict__ cache, const h1 *__restrict__ k_new,
     h1 *__restrict__ out,
@@ -142,135 +154,140 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
     constexpr int D = 128, CPL = 4;
     using G = Geo<D, CPL>;
     __shared__ uint2 tab[FT_TABLE_WORDS64]; // the only LDS object: sits at offset 0
-    const FtUnit un(B, H, sa.nseg);
-
+    const int h = (int)blockIdx.x / sa.phys_per_head;
+    const int pw = (int)blockIdx.x % sa.phys_per_head;
+    const int wph = ft_wgs_per_head(B, sa.nseg);
     const int lane = threadIdx.x & 63;
-    const uint32_t lane_copy = 0x100u | ((uint32_t)un.lh * 8u);
-    const int bx = un.bx, lh = un.lh, c0 = un.c0, h = un.h;
-    const bool active = un.active;
-    const bool last = un.seg == sa.nseg - 1;
-
-    Pair st[G::NP];
-    h2 qv[G::NP];
-    ft_init_pairs(st, zp, sc, al, h, bx, c0, un.seg, sa);
-#pragma unroll
-    for (int p = 0; p < G::NP; p++)
-        qv[p] = load_act2(q + (size_t)bx * D + c0 + 2 * p, sa.act_bf16);
-
-    const int t0 = un.seg * sa.seg_tokens;
-    const int t1 = last ? T : t0 + sa.seg_tokens;
-    uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh;
-    const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;
-    h1 *ob = out + (size_t)bx * sa.row_pitch + t0;
-    const int nfull = (t1 - t0) >> 3;
     const int tk = token_of_lane(lane);
-    const bool storer = active && (lane & 3) == 0;
-
-    // The first code words, like the parameters and the query above, are requested BEFORE the
-    // table is built, so that their latency runs beside the fill instead of after it (padding
-    // waves have valid, clamped addresses and simply drop what they loaded).
-    uint4 buf[PF][1];
-#pragma unroll
-    for (int i = 0; i < PF; i++)
-        buf[i][0] = (i < nfull) ? cb[(size_t)i * G::VPS] : make_uint4(0, 0, 0, 0);
-    ft_fill(tab, be, tg, un.h);
+    // The table is built before the loop: a barrier under a condition inside it, even a uniform
+    // one, costs the loop body some twenty registers and spills.
+    ft_fill(tab, be, tg, h);
     __syncthreads();
-    if (!un.wave_active)
-        return; // padding waves of the head's last workgroup
 
-    auto finish = [&](const float *part, int sg, int ntok) {
-        const float s = reduce8_head32(part);
-        if (storer && tk < ntok)
-            ob[sg * 8 + tk] = (h1)s;
-    };
+    for (int vw = pw; vw < wph; vw += sa.phys_per_head) {
+        const FtUnit un(B, H, sa.nseg, h, vw);
+        const uint32_t lane_copy = 0x100u | ((uint32_t)un.lh * 8u);
+        const int bx = un.bx, lh = un.lh, c0 = un.c0;
+        const bool active = un.active;
+        const bool last = un.seg == sa.nseg - 1;
 
-    // one token of the current supergroup, then the lookups of the same slot of the next one
-    auto token = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2], float &out_t) {
-        float acc;
-#pragma unroll
-        for (int p = 0; p < G::NP; p++) {
-            Pair &s = st[p];
-            const h2 qs = as_h2(e[p][t].x) * s.sc;
-            const h2 kh = qs + s.zp;
-            if (p == 0)
-                acc = dot2_from_zero(qv[p], kh);
-            else
-                acc = __builtin_amdgcn_fdot2(qv[p], kh, acc, false);
-            update_pair_f(s, as_h2(e[p][t].y), qs);
-        }
-        out_t = acc;
+        Pair st[G::NP];
+        h2 qv[G::NP];
+        ft_init_pairs(st, zp, sc, al, h, bx, c0, un.seg, sa);
 #pragma unroll
         for (int p = 0; p < G::NP; p++)
-            e[p][t] = ft_get(tab, nb[p][t & 1], lane_copy, t >> 1, p);
-        __builtin_amdgcn_sched_barrier(0);
-    };
+            qv[p] = load_act2(q + (size_t)bx * D + c0 + 2 * p, sa.act_bf16);
 
-    uint2 lk[G::NP][8];
-    uint32_t nb[G::NP][2];
-    float part[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (nfull > 0) {
-        pair_bytes_of<D, CPL>(buf[0], nb);
+        const int t0 = seg_begin(sa, un.seg);
+        const int t1 = last ? T : seg_end(sa, un.seg);
+        uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh;
+        const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;
+        h1 *ob = out + (size_t)bx * sa.row_pitch + t0;
+        const int nfull = (t1 - t0) >> 3;
+        const bool storer = active && (lane & 3) == 0;
+
+        // (padding waves have valid, clamped addresses and simply drop what they loaded)
+        uint4 buf[PF][1];
 #pragma unroll
-        for (int t = 0; t < 8; t++)
+        for (int i = 0; i < PF; i++)
+            buf[i][0] = (i < nfull) ? ft_load_codes(cb + (size_t)i * G::VPS) : make_uint4(0, 0, 0, 0);
+        if (!un.wave_active)
+            continue; // padding waves of the head's last virtual workgroup
+
+        auto finish = [&](const float *part, int sg, int ntok) {
+            const float s = reduce8_head32(part);
+            if (storer && tk < ntok)
+                ob[sg * 8 + tk] = (h1)s;
+        };
+
+        // one token of the current supergroup, then the lookups of the same slot of the next one
+        auto token = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2], float &out_t) {
+            float acc;
+#pragma unroll
+            for (int p = 0; p < G::NP; p++) {
+                Pair &s = st[p];
+                const h2 qs = as_h2(e[p][t].x) * s.sc;
+                const h2 kh = qs + s.zp;
+                if (p == 0)
+                    acc = dot2_from_zero(qv[p], kh);
+                else
+                    acc = __builtin_amdgcn_fdot2(qv[p], kh, acc, false);
+                update_pair_f(s, as_h2(e[p][t].y), qs);
+            }
+            out_t = acc;
 #pragma unroll
             for (int p = 0; p < G::NP; p++)
-                lk[p][t] = ft_get(tab, nb[p][t & 1], lane_copy, t >> 1, p);
-    }
-    // One supergroup; i = its buffer in the rotation.  Nothing conditional: the trip count is
-    // wave-uniform, the prefetch index is clamped, and the reduction of the previous supergroup
-    // (done here, between the lookups' issue and their first use) stores nothing for sg == 0.
-    auto body = [&](int sg, auto ic) {
-        constexpr int i = decltype(ic)::value;
-        pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
-        buf[i][0] = cb[(size_t)ft_prefetch_index(sg, nfull) * G::VPS];
-        __builtin_amdgcn_sched_barrier(0);
-        finish(part, sg - 1, sg > 0 ? 8 : 0);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int t = 0; t < 8; t++)
-            token(t, lk, nb, part[t]);
-    };
-    rotate_over<PF>(nfull, body);
-    if (nfull > 0)
-        finish(part, nfull - 1, 8);
-    if (!last)
-        return;
+                e[p][t] = ft_get(tab, nb[p][t & 1], lane_copy, t >> 1, p);
+            __builtin_amdgcn_sched_barrier(0);
+        };
 
-    // ragged tail: T % 8 tokens of the last supergroup (gemv.cu:648-654); plain arithmetic
-    ft_load_beta(st, be, tg, h, c0);
-    const int ntail = (t1 - t0) & 7;
-    if (ntail) {
-        float tp[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-        uint32_t w[4];
-        vec_words(cb[(size_t)nfull * G::VPS], w);
+        uint2 lk[G::NP][8];
+        uint32_t nb[G::NP][2];
+        float part[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (nfull > 0) {
+            pair_bytes_of<D, CPL>(buf[0], nb);
 #pragma unroll
-        for (int pp = 0; pp < 2; pp++) {
-            Pair &s = st[pp];
-            for (int tt = 0; tt < ntail; tt++) {
-                const h2 qc = extract_pair<4>(w[2 * pp], w[2 * pp + 1], tt);
-                const h2 qs = qc * s.sc;
-                const float d = __builtin_amdgcn_fdot2(qv[pp], qs + s.zp, 0.0f, false);
+            for (int t = 0; t < 8; t++)
 #pragma unroll
-                for (int k = 0; k < 8; k++)
-                    tp[k] += (k == tt) ? d : 0.0f;
-                update_pair(s, qc, qs);
-            }
+                for (int p = 0; p < G::NP; p++)
+                    lk[p][t] = ft_get(tab, nb[p][t & 1], lane_copy, t >> 1, p);
         }
-        finish(tp, nfull, ntail);
-    }
-
-    if (active)
-        publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
-
-    h2 deq[G::NP];
-    append_new_token<D, CPL>(cbh, T, k_new + (size_t)bx * D + c0, st, deq, active, sa.act_bf16);
-    float self = 0.0f;
+        // One supergroup; i = its buffer in the rotation.  Nothing conditional: the trip count is
+        // wave-uniform, the prefetch index is clamped, and the reduction of the previous supergroup
+        // (done here, between the lookups' issue and their first use) stores nothing for sg == 0.
+        auto body = [&](int sg, auto ic) {
+            constexpr int i = decltype(ic)::value;
+            pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
+            buf[i][0] = ft_load_codes(cb + (size_t)ft_prefetch_index(sg, nfull) * G::VPS);
+            __builtin_amdgcn_sched_barrier(0);
+            finish(part, sg - 1, sg > 0 ? 8 : 0);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int p = 0; p < G::NP; p++)
-        self = __builtin_amdgcn_fdot2(qv[p], deq[p], self, false);
-    self = head_allreduce<G::LPH>(self);
-    if (active && lh == 0)
-        out[(size_t)bx * sa.row_pitch + T] = (h1)self;
+            for (int t = 0; t < 8; t++)
+                token(t, lk, nb, part[t]);
+        };
+        rotate_over<PF>(nfull, body);
+        if (nfull > 0)
+            finish(part, nfull - 1, 8);
+        if (!last)
+            continue;
+
+        // ragged tail: T % 8 tokens of the last supergroup (gemv.cu:648-654); plain arithmetic
+        ft_load_beta(st, be, tg, h, c0);
+        const int ntail = (t1 - t0) & 7;
+        if (ntail) {
+            float tp[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            uint32_t w[4];
+            vec_words(cb[(size_t)nfull * G::VPS], w);
+#pragma unroll
+            for (int pp = 0; pp < 2; pp++) {
+                Pair &s = st[pp];
+                for (int tt = 0; tt < ntail; tt++) {
+                    const h2 qc = extract_pair<4>(w[2 * pp], w[2 * pp + 1], tt);
+                    const h2 qs = qc * s.sc;
+                    const float d = __builtin_amdgcn_fdot2(qv[pp], qs + s.zp, 0.0f, false);
+#pragma unroll
+                    for (int k = 0; k < 8; k++)
+                        tp[k] += (k == tt) ? d : 0.0f;
+                    update_pair(s, qc, qs);
+                }
+            }
+            finish(tp, nfull, ntail);
+        }
+
+        if (active)
+            publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
+
+        h2 deq[G::NP];
+        append_new_token<D, CPL>(cbh, T, k_new + (size_t)bx * D + c0, st, deq, active, sa.act_bf16);
+        float self = 0.0f;
+#pragma unroll
+        for (int p = 0; p < G::NP; p++)
+            self = __builtin_amdgcn_fdot2(qv[p], deq[p], self, false);
+        self = head_allreduce<G::LPH>(self);
+        if (active && lh == 0)
+            out[(size_t)bx * sa.row_pitch + T] = (h1)self;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -293,6 +310,11 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
 // half an fp16 ulp of the largest value, for 1 % of the kernel's time: not done.)
 // A non-finite cached value makes both outputs of its channel PAIR non-finite (0 * inf inside the
 // product); the vector form of ov_kernel's two-channel lanes confines it to its own channel.
+//
+// One virtual workgroup per workgroup (forward_ov gains nothing from uneven segments, so its plan
+// never needs more).  sa.combine: the two or four segments of a sequence pair sit in the same
+// workgroup and are added there; otherwise every segment stores its fp32 partial sums for
+// ov_finalize_kernel.
 __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
     const h1 *__restrict__ attn, uint4 *__restrict__ cache, const h1 *__restrict__ v_new,
     h1 *__restrict__ out, float *__restrict__ partial,
@@ -303,178 +325,180 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
     constexpr int D = 128, CPL = 4;
     using G = Geo<D, CPL>;
     __shared__ uint2 tab[FT_TABLE_WORDS64];
-    const FtUnit un(B, H, sa.nseg);
-
-    const uint32_t lane_copy = 0x100u | ((uint32_t)un.lh * 8u);
-    const int bx = un.bx, lh = un.lh, c0 = un.c0, h = un.h;
-    const bool active = un.active;
-    const bool last = un.seg == sa.nseg - 1;
+    const int wph = ft_wgs_per_head(B, sa.nseg);
+    const int h = (int)blockIdx.x / wph;
     const int BH = B * H;
-
-    Pair st[G::NP];
-    float acc[CPL];
-    f4v acc4[G::NP];
-    ft_init_pairs(st, zp, sc, al, h, bx, c0, un.seg, sa);
-#pragma unroll
-    for (int c = 0; c < CPL; c++)
-        acc[c] = 0.0f;
-#pragma unroll
-    for (int p = 0; p < G::NP; p++)
-        acc4[p] = (f4v){0.0f, 0.0f, 0.0f, 0.0f};
     // selectors that turn the word (w[t], w[t+1]) into this lane's two A registers
     const int role = threadIdx.x & 3;
     const uint32_t sel_a0 = role == 0 ? 0x0C0C0100u : role == 1 ? 0x01000C0Cu : 0x0C0C0C0Cu;
     const uint32_t sel_a1 = role == 0 ? 0x0C0C0302u : role == 1 ? 0x03020C0Cu : 0x0C0C0C0Cu;
+    {
+        const FtUnit un(B, H, sa.nseg, h, (int)blockIdx.x % wph);
+        const uint32_t lane_copy = 0x100u | ((uint32_t)un.lh * 8u);
+        const int bx = un.bx, lh = un.lh, c0 = un.c0;
+        const bool active = un.active;
+        const bool last = un.seg == sa.nseg - 1;
 
-    const int t0 = un.seg * sa.seg_tokens;
-    const int t1 = last ? T : t0 + sa.seg_tokens;
-    uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh;
-    const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;
-    const h1 *wrow = attn + (size_t)bx * sa.row_pitch;
-    const h1 *wb = wrow + t0;
-    const int nfull = (t1 - t0) >> 3;
-
-    auto load_w = [&](int sg) {
-        uint4 r;
-        __builtin_memcpy(&r, wb + (size_t)sg * 8, 16); // row base is only 2-byte aligned
-        return r;
-    };
-    // the first code words and weights, like the parameters above, are requested before the
-    // table is built (see qk_ft_kernel)
-    uint4 buf[PF][1];
-    uint4 wbuf[PF];
-#pragma unroll
-    for (int i = 0; i < PF; i++) {
-        buf[i][0] = (i < nfull) ? cb[(size_t)i * G::VPS] : make_uint4(0, 0, 0, 0);
-        wbuf[i] = (i < nfull) ? load_w(i) : make_uint4(0, 0, 0, 0);
-    }
-    ft_fill(tab, be, tg, un.h);
-    __syncthreads();
-    if (!un.wave_active) {
-        if (sa.combine) { // the two barriers of the in-workgroup sum below
-            __syncthreads();
-            __syncthreads();
-        }
-        return;
-    }
-    // two tokens of the current supergroup on the matrix cores, then the lookups of the same two
-    // slots of the next one
-    auto token2 = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2], const uint4 wv) {
-        const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
-        const uint32_t w2 = ww[t >> 1];
-        const h4v a = as_h4(__builtin_amdgcn_perm(w2, w2, sel_a0), __builtin_amdgcn_perm(w2, w2, sel_a1));
-        uint32_t vd[G::NP][2];
-#pragma unroll
-        for (int k = 0; k < 2; k++)
-#pragma unroll
-            for (int p = 0; p < G::NP; p++) {
-                Pair &s = st[p];
-                const h2 qs = as_h2(e[p][t + k].x) * s.sc;
-                vd[p][k] = as_u32(qs + s.zp);
-                update_pair_f(s, as_h2(e[p][t + k].y), qs);
-            }
+        Pair st[G::NP];
+        float acc[CPL];
+        f4v acc4[G::NP];
+        ft_init_pairs(st, zp, sc, al, h, bx, c0, un.seg, sa);
 #pragma unroll
         for (int p = 0; p < G::NP; p++)
-            acc4[p] = __builtin_amdgcn_mfma_f32_4x4x4f16(a, as_h4(vd[p][0], vd[p][1]), acc4[p], 0, 0, 0);
-#pragma unroll
-        for (int k = 0; k < 2; k++)
-#pragma unroll
-            for (int p = 0; p < G::NP; p++)
-                e[p][t + k] = ft_get(tab, nb[p][(t + k) & 1], lane_copy, (t + k) >> 1, p);
-        __builtin_amdgcn_sched_barrier(0);
-    };
+            acc4[p] = (f4v){0.0f, 0.0f, 0.0f, 0.0f};
 
-    uint2 lk[G::NP][8];
-    uint32_t nb[G::NP][2];
-    if (nfull > 0) {
-        pair_bytes_of<D, CPL>(buf[0], nb);
-#pragma unroll
-        for (int t = 0; t < 8; t++)
-#pragma unroll
-            for (int p = 0; p < G::NP; p++)
-                lk[p][t] = ft_get(tab, nb[p][t & 1], lane_copy, t >> 1, p);
-    }
-    auto body = [&](int sg, auto ic) {
-        constexpr int i = decltype(ic)::value;
-        pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
-        const int sgp = ft_prefetch_index(sg, nfull);
-        buf[i][0] = cb[(size_t)sgp * G::VPS];
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int t = 0; t < 8; t += 2)
-            token2(t, lk, nb, wbuf[i]);
-        wbuf[i] = load_w(sgp); // reloaded once its last token is done (see ov_kernel)
-    };
-    rotate_over<PF>(nfull, body);
-#pragma unroll
-    for (int p = 0; p < G::NP; p++) {
-        acc[2 * p] = acc4[p].x;
-        acc[2 * p + 1] = acc4[p].y;
-    }
+        const int t0 = seg_begin(sa, un.seg);
+        const int t1 = last ? T : seg_end(sa, un.seg);
+        uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh;
+        const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;
+        const h1 *wrow = attn + (size_t)bx * sa.row_pitch;
+        const h1 *wb = wrow + t0;
+        const int nfull = (t1 - t0) >> 3;
 
-    if (last) {
-        ft_load_beta(st, be, tg, h, c0);
-        const int ntail = (t1 - t0) & 7;
-        if (ntail) {
-            uint32_t w[4];
-            vec_words(cb[(size_t)nfull * G::VPS], w);
+        auto load_w = [&](int sg) {
+            uint4 r;
+            __builtin_memcpy(&r, wb + (size_t)sg * 8, 16); // row base is only 2-byte aligned
+            return r;
+        };
+        // the first code words and weights, like the parameters above, are requested before the
+        // table is built, so that their latency runs beside the fill instead of after it
+        uint4 buf[PF][1];
+        uint4 wbuf[PF];
 #pragma unroll
-            for (int pp = 0; pp < 2; pp++) {
-                Pair &s = st[pp];
-                for (int tt = 0; tt < ntail; tt++) {
-                    const h2 qc = extract_pair<4>(w[2 * pp], w[2 * pp + 1], tt);
-                    const h2 qs = qc * s.sc;
-                    const h2 vd = qs + s.zp;
-                    const float wt = (float)wb[nfull * 8 + tt];
-                    acc[2 * pp] = __builtin_fmaf(wt, (float)vd.x, acc[2 * pp]);
-                    acc[2 * pp + 1] = __builtin_fmaf(wt, (float)vd.y, acc[2 * pp + 1]);
-                    update_pair(s, qc, qs);
-                }
-            }
+        for (int i = 0; i < PF; i++) {
+            buf[i][0] = (i < nfull) ? ft_load_codes(cb + (size_t)i * G::VPS) : make_uint4(0, 0, 0, 0);
+            wbuf[i] = (i < nfull) ? load_w(i) : make_uint4(0, 0, 0, 0);
         }
-        if (active)
-            publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
-        h2 deq[G::NP];
-        append_new_token<D, CPL>(cbh, T, v_new + (size_t)bx * D + c0, st, deq, active, sa.act_bf16);
-        const float wT = (float)wrow[T];
+        ft_fill(tab, be, tg, h);
+        __syncthreads();
+        if (!un.wave_active) {
+            if (sa.combine) { // the two barriers of the in-workgroup sum below
+                __syncthreads();
+                __syncthreads();
+            }
+            return;
+        }
+
+        // two tokens of the current supergroup on the matrix cores, then the lookups of the same two
+        // slots of the next one
+        auto token2 = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2], const uint4 wv) {
+            const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+            const uint32_t w2 = ww[t >> 1];
+            const h4v a = as_h4(__builtin_amdgcn_perm(w2, w2, sel_a0), __builtin_amdgcn_perm(w2, w2, sel_a1));
+            uint32_t vd[G::NP][2];
+#pragma unroll
+            for (int k = 0; k < 2; k++)
+#pragma unroll
+                for (int p = 0; p < G::NP; p++) {
+                    Pair &s = st[p];
+                    const h2 qs = as_h2(e[p][t + k].x) * s.sc;
+                    vd[p][k] = as_u32(qs + s.zp);
+                    update_pair_f(s, as_h2(e[p][t + k].y), qs);
+                }
+#pragma unroll
+            for (int p = 0; p < G::NP; p++)
+                acc4[p] = __builtin_amdgcn_mfma_f32_4x4x4f16(a, as_h4(vd[p][0], vd[p][1]), acc4[p], 0, 0, 0);
+#pragma unroll
+            for (int k = 0; k < 2; k++)
+#pragma unroll
+                for (int p = 0; p < G::NP; p++)
+                    e[p][t + k] = ft_get(tab, nb[p][(t + k) & 1], lane_copy, (t + k) >> 1, p);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+
+        uint2 lk[G::NP][8];
+        uint32_t nb[G::NP][2];
+        if (nfull > 0) {
+            pair_bytes_of<D, CPL>(buf[0], nb);
+#pragma unroll
+            for (int t = 0; t < 8; t++)
+#pragma unroll
+                for (int p = 0; p < G::NP; p++)
+                    lk[p][t] = ft_get(tab, nb[p][t & 1], lane_copy, t >> 1, p);
+        }
+        auto body = [&](int sg, auto ic) {
+            constexpr int i = decltype(ic)::value;
+            pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
+            const int sgp = ft_prefetch_index(sg, nfull);
+            buf[i][0] = ft_load_codes(cb + (size_t)sgp * G::VPS);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < 8; t += 2)
+                token2(t, lk, nb, wbuf[i]);
+            wbuf[i] = load_w(sgp); // reloaded once its last token is done (see ov_kernel)
+        };
+        rotate_over<PF>(nfull, body);
 #pragma unroll
         for (int p = 0; p < G::NP; p++) {
-            acc[2 * p] = __builtin_fmaf(wT, (float)deq[p].x, acc[2 * p]);
-            acc[2 * p + 1] = __builtin_fmaf(wT, (float)deq[p].y, acc[2 * p + 1]);
+            acc[2 * p] = acc4[p].x;
+            acc[2 * p + 1] = acc4[p].y;
         }
-    }
-    if (sa.combine) {
-        // nseg is 2 or 4: the waves holding the other segments of these sequences are 4, 8, 12
-        // waves away in this workgroup (interleave_segment: quad q takes segment q mod nseg).  The
-        // table is finished with once every wave is here; its first 16 KB take the partial sums,
-        // and the wave of segment 0 adds them in segment order (what ov_finalize_kernel does).
-        __syncthreads();
-        float4 *red = reinterpret_cast<float4 *>(tab);
-        const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
-        red[wv * 64 + lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
-        __syncthreads();
-        if (un.seg != 0 || !active)
+
+        if (last) {
+            ft_load_beta(st, be, tg, h, c0);
+            const int ntail = (t1 - t0) & 7;
+            if (ntail) {
+                uint32_t w[4];
+                vec_words(cb[(size_t)nfull * G::VPS], w);
+#pragma unroll
+                for (int pp = 0; pp < 2; pp++) {
+                    Pair &s = st[pp];
+                    for (int tt = 0; tt < ntail; tt++) {
+                        const h2 qc = extract_pair<4>(w[2 * pp], w[2 * pp + 1], tt);
+                        const h2 qs = qc * s.sc;
+                        const h2 vd = qs + s.zp;
+                        const float wt = (float)wb[nfull * 8 + tt];
+                        acc[2 * pp] = __builtin_fmaf(wt, (float)vd.x, acc[2 * pp]);
+                        acc[2 * pp + 1] = __builtin_fmaf(wt, (float)vd.y, acc[2 * pp + 1]);
+                        update_pair(s, qc, qs);
+                    }
+                }
+            }
+            if (active)
+                publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
+            h2 deq[G::NP];
+            append_new_token<D, CPL>(cbh, T, v_new + (size_t)bx * D + c0, st, deq, active, sa.act_bf16);
+            const float wT = (float)wrow[T];
+#pragma unroll
+            for (int p = 0; p < G::NP; p++) {
+                acc[2 * p] = __builtin_fmaf(wT, (float)deq[p].x, acc[2 * p]);
+                acc[2 * p + 1] = __builtin_fmaf(wT, (float)deq[p].y, acc[2 * p + 1]);
+            }
+        }
+        if (sa.combine) {
+            // nseg is 2 or 4: the waves holding
+            // the other segments of these sequences are 4, 8, 12 waves away (interleave_segment:
+            // quad q takes segment q mod nseg).  The table is finished with once every wave is
+            // here; its first 16 KB take the partial sums, and the wave of segment 0 adds them in
+            // segment order (what ov_finalize_kernel does).
+            __syncthreads();
+            float4 *red = reinterpret_cast<float4 *>(tab);
+            const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+            red[wv * 64 + lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+            __syncthreads();
+            if (un.seg != 0 || !active)
+                return;
+            for (int s = 1; s < sa.nseg; s++) {
+                const float4 p = red[(wv + 4 * s) * 64 + lane];
+                acc[0] += p.x;
+                acc[1] += p.y;
+                acc[2] += p.z;
+                acc[3] += p.w;
+            }
+        }
+        if (!active)
             return;
-        for (int s = 1; s < sa.nseg; s++) {
-            const float4 p = red[(wv + 4 * s) * 64 + lane];
-            acc[0] += p.x;
-            acc[1] += p.y;
-            acc[2] += p.z;
-            acc[3] += p.w;
+        if (sa.nseg == 1 || sa.combine) {
+            h1 *o = out + (size_t)bx * D + c0;
+#pragma unroll
+            for (int p = 0; p < G::NP; p++)
+                store_act2(o + 2 * p, acc[2 * p], acc[2 * p + 1], sa.act_bf16);
+        } else {
+            float2 *o = reinterpret_cast<float2 *>(partial + ((size_t)un.seg * BH + bx) * D + c0);
+#pragma unroll
+            for (int p = 0; p < G::NP; p++)
+                o[p] = make_float2(acc[2 * p], acc[2 * p + 1]);
         }
-    }
-    if (!active)
-        return;
-    if (sa.nseg == 1 || sa.combine) {
-        h1 *o = out + (size_t)bx * D + c0;
-#pragma unroll
-        for (int p = 0; p < G::NP; p++)
-            store_act2(o + 2 * p, acc[2 * p], acc[2 * p + 1], sa.act_bf16);
-    } else {
-        float2 *o = reinterpret_cast<float2 *>(partial + ((size_t)un.seg * BH + bx) * D + c0);
-#pragma unroll
-        for (int p = 0; p < G::NP; p++)
-            o[p] = make_float2(acc[2 * p], acc[2 * p + 1]);
     }
 }
 

@@ -72,7 +72,60 @@ struct Seg {
     long row_pitch;     // elements between rows of the logits / attention-weight matrix (>= T + 1)
     int act_bf16;       // q, the new token and the output are bfloat16 (see load_act2 / store_act2)
     int combine;        // ov_ft_kernel: the segments' partial outputs are added inside the workgroup
+    // Per-head-table kernels only.  groups > 0: the context's `intervals` checkpoint intervals are
+    // cut into `groups` groups of four segments of unequal length (uneven_cut).  phys_per_head:
+    // workgroups launched per KV head; each walks through the head's virtual workgroups pw,
+    // pw + phys_per_head, ... one after the other (same table, no barrier between them).
+    int groups;
+    int intervals;
+    int phys_per_head;
+    unsigned skew;      // shares of the four wave slots, oldest first, one byte each, in sixteenths
 };
+
+__host__ __device__ inline int ft_skew(unsigned skew, int k) { return (int)((skew >> (8 * k)) & 0xFFu); }
+constexpr unsigned pack_skew(unsigned a, unsigned b, unsigned c, unsigned d) { return a | (b << 8) | (c << 16) | (d << 24); }
+
+// First checkpoint interval of segment `seg` (seg == 4*groups: one past the last) when `intervals`
+// intervals are cut into `groups` groups of four uneven segments.  Group g covers
+// [intervals*g/groups, intervals*(g+1)/groups); inside it the shares are rounded down, every
+// segment gets at least one interval, and what is left goes to the oldest slots first.  Needs at
+// least four intervals per group.  The same function plans on the host and indexes on the device.
+__host__ __device__ inline int uneven_cut(int seg, int groups, int intervals, unsigned skew)
+{
+    const int g = seg >> 2, k = seg & 3;
+    const int lo = (int)((long)intervals * g / groups);
+    if (k == 0)
+        return lo;
+    const int n = (int)((long)intervals * (g + 1) / groups) - lo;
+    int part[4], left = n;
+    for (int i = 0; i < 4; i++) {
+        part[i] = n * ft_skew(skew, i) / 16;
+        if (part[i] < 1)
+            part[i] = 1;
+        left -= part[i];
+    }
+    for (int i = 0; left > 0; i = (i + 1) & 3, left--)
+        part[i]++;
+    for (int i = 0; left < 0; i = (i + 1) & 3) // only when n is tiny: take from the longest
+        if (part[i] > 1) {
+            part[i]--;
+            left++;
+        }
+    int c = lo;
+    for (int i = 0; i < k; i++)
+        c += part[i];
+    return c;
+}
+
+// first token of segment `seg` / of the one after it
+__host__ __device__ inline int seg_begin(const Seg &sa, int seg)
+{
+    return sa.groups ? uneven_cut(seg, sa.groups, sa.intervals, sa.skew) * sa.ckpt_interval : seg * sa.seg_tokens;
+}
+__host__ __device__ inline int seg_end(const Seg &sa, int seg)
+{
+    return sa.groups ? uneven_cut(seg + 1, sa.groups, sa.intervals, sa.skew) * sa.ckpt_interval : (seg + 1) * sa.seg_tokens;
+}
 
 __device__ __forceinline__ float wave_xor_add(float v, int mask)
 {
@@ -1680,6 +1733,10 @@ static Seg plan_segments(void *ckpt, int n_ckpt_cap, int ckpt_interval, int BH, 
     s.row_pitch = T + 1;
     s.act_bf16 = 0;
     s.combine = 0;
+    s.groups = 0;
+    s.intervals = 0;
+    s.phys_per_head = 0;
+    s.skew = 0;
     if (!ckpt || ckpt_interval <= 0 || T <= ckpt_interval)
         return s;
     const int avail = (T + ckpt_interval - 1) / ckpt_interval;               // finest split
@@ -1850,6 +1907,89 @@ static bool use_head_table(int B, int H, int GQ, int bits, int D, const Seg &seg
     return t_ft <= t_shared;
 }
 
+// The plan of a launch that takes the per-head-table kernels.
+//
+// A SIMD issues from its OLDEST resident wave whenever that wave has an instruction ready (wave
+// priorities set by the program do not change that on this chip), and one wave alone keeps the
+// vector pipe only about half busy.  Four waves with equal shares of work therefore finish one
+// after the other (measured at B=128, 32 heads, 4096 tokens in two even segments: the four waves of
+// a SIMD are done after 131, 188, 261 and 327 us) and the pipe idles more and more towards the end.
+// So the shares are made UNEVEN, in the proportions in which the four slots of a SIMD actually
+// progress while all are resident (FT_SKEW, oldest first): a workgroup's waves 4k..4k+3 are slot k
+// of its four SIMDs, interleave_segment gives quad k of a workgroup segment k of a group of four,
+// and the context of every sequence is cut into groups of four such segments, at checkpoints.
+//
+// That needs four segments where the even plan has one or two, hence more workgroups than CUs;
+// a second round of workgroups costs a table build, a launch gap and a second ragged end (12 % at
+// the shape above).  Instead each launched workgroup walks through several VIRTUAL workgroups of
+// its head one after the other (phys_per_head apart) with no barrier between them.
+//
+// Measured at B=128, 32 heads, 4096 tokens, checkpoints every 256 (medians of interleaved runs on
+// one device, us): forward_qk 300-303 with two even segments, 297 with four even ones walked as
+// two virtual workgroups, 280-285 with shares 7:5:2:2 (8:4:2:2 and 6:6:3:1 within 3 us of that,
+// 9:4:2:1 302); forward_ov 261 with two even segments added inside the workgroup, 262-266 with the
+// best uneven shares (6:5:3:2, 7:5:2:2) plus the 4 us kernel that then adds the partial sums: no
+// gain, so forward_ov keeps its even plan.
+// Shares of a SIMD's work given to its four wave slots, oldest first, in sixteenths of a group's
+// checkpoint intervals: measured on the headline shape, one setting per kernel.
+constexpr unsigned FT_SKEW_QK = pack_skew(7, 5, 2, 2);
+constexpr unsigned FT_SKEW_OV = 0; // 0: even segments.  forward_ov gains nothing from uneven ones (see plan_head_table)
+constexpr int FT_MIN_GROUP = 8;  // checkpoint intervals a group needs for its shares to differ
+constexpr int FT_MAX_GROUPS = 16;
+
+static void plan_head_table(Seg &seg, int B, int H, int T, unsigned skew)
+{
+    seg.groups = 0;
+    seg.skew = skew;
+    seg.phys_per_head = ft_wgs_per_head(B, seg.nseg);
+    if (!seg.ckpt || seg.ckpt_interval <= 0 || skew == 0)
+        return;
+    const int iv = seg.ckpt_interval;
+    const int avail = (T + iv - 1) / iv;
+    // groups of four segments: as many as give every SIMD its four waves, FT_MIN_GROUP intervals or more each
+    const long waves_per_group = (long)H * 4 * pad4(ft_pairs_per_seg(B));
+    long G = ((long)N_SIMD * WAVES_PER_SIMD_TARGET + waves_per_group - 1) / waves_per_group;
+    if (G > avail / FT_MIN_GROUP)
+        G = avail / FT_MIN_GROUP;
+    if (G > FT_MAX_GROUPS)
+        G = FT_MAX_GROUPS;
+    if (G < 1)
+        return;
+    // segment s > 0 starts from checkpoint cut(s) - 1
+    if (uneven_cut((int)(4 * G - 1), (int)G, avail, skew) - 1 >= seg.n_ckpt_cap)
+        return;
+    seg.groups = (int)G;
+    seg.intervals = avail;
+    seg.nseg = (int)(4 * G);
+    seg.seg_tokens = iv; // not read by the kernels of an uneven plan
+    // workgroups per head: the fewest rounds of 256 workgroups times virtual workgroups each
+    const int W = ft_wgs_per_head(B, seg.nseg);
+    int best = W;
+    long best_cost = -1;
+    for (int P = 1; P <= W; P++) {
+        const long cost = (((long)H * P + 255) / 256) * ((W + P - 1) / P);
+        if (best_cost < 0 || cost < best_cost) {
+            best = P;
+            best_cost = cost;
+        }
+    }
+    seg.phys_per_head = best;
+}
+
+// How many segments the forward_ov partial sums of a launch can have under either plan (what a
+// workspace must be sized for: the kernel family can be switched between sizing and launch).
+static int max_plan_segments(void *ckpt, int n_ckpt_cap, int ckpt_interval, int B, int H, int T, int D)
+{
+    Seg seg = plan_segments(ckpt, n_ckpt_cap, ckpt_interval, B * H, T, D);
+    int n = seg.nseg;
+    if (D == 128) {
+        plan_head_table(seg, B, H, T, FT_SKEW_QK);
+        if (seg.nseg > n)
+            n = seg.nseg;
+    }
+    return n;
+}
+
 static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval, int bits = 4)
 {
     if (!ckpt)
@@ -1864,7 +2004,7 @@ static int check_ckpt(const void *ckpt, int n_ckpt_cap, int ckpt_interval, int b
 
 extern "C" {
 
-int adkv_abi_version(void) { return 14; }
+int adkv_abi_version(void) { return 15; }
 
 void adkv_set_mha_kernel(int use_matrix_cores)
 {
@@ -1948,6 +2088,10 @@ static int encode_common(void *cache, const void *kv_new,
     seg.row_pitch = T + 1;
     seg.act_bf16 = 0;
     seg.combine = 0;
+    seg.groups = 0;
+    seg.intervals = 0;
+    seg.phys_per_head = 0;
+    seg.skew = 0;
     // Lane width, measured on an MI355X (4096 tokens, ms for 65 536 / 131 072 / 196 608 / 262 144 /
     // 524 288 channels): one channel per lane 0.29 / 0.44 / 0.60 / 0.74 / 1.38, two 0.43 / 0.44 /
     // 0.55 / 0.60 / 1.17, four 0.78 / 0.78 / 0.78 / 0.79 / 1.18.  Up to two waves per SIMD the
@@ -2094,8 +2238,12 @@ static const char *decode_kernel_name(int B, int Hq, int H, int T, int D, int bi
         return threads >= 1024L * 256 ? "gqa_kernel, 16-wave workgroups (matrix cores)"
                                       : "gqa_kernel, 8-wave workgroups (matrix cores)";
     }
-    if (use_head_table(B, H, GQ, bits, D, seg))
-        return "ft_kernel (per-head table, 16-wave workgroups)";
+    if (use_head_table(B, H, GQ, bits, D, seg)) {
+        Seg s2 = seg;
+        plan_head_table(s2, B, H, T, FT_SKEW_QK);
+        return s2.groups ? "ft_kernel (per-head table, 16-wave workgroups, uneven segments)"
+                         : "ft_kernel (per-head table, 16-wave workgroups)";
+    }
     if (D == 128) {
         const long units = padded_units<32>(B * H, seg.nseg);
         if (units / 2 <= N_SIMD)
@@ -2147,7 +2295,8 @@ static int forward_qk_impl(const void *q, void *k_cache, const void *k_new, void
         return check_launch();
     }
     if (use_head_table(B, H, GQ, bits, D, seg)) {
-        hipLaunchKernelGGL(qk_ft_kernel, dim3((unsigned)(H * ft_wgs_per_head(B, seg.nseg))), dim3(FT_BLK), 0, st,
+        plan_head_table(seg, B, H, T, FT_SKEW_QK);
+        hipLaunchKernelGGL(qk_ft_kernel, dim3((unsigned)(H * seg.phys_per_head)), dim3(FT_BLK), 0, st,
                            (const h1 *)q, (uint4 *)k_cache, (const h1 *)k_new, (h1 *)logits,
                            (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha, (const h1 *)beta,
                            (const h1 *)tgt, B, H, T, n_super_cap, (h1 *)state_out, seg);
@@ -2165,6 +2314,40 @@ const char *adkv_decode_kernel_name(int B, int Hq, int H, int T, int D, int bits
                                     int ckpt_interval)
 {
     return decode_kernel_name(B, Hq, H, T, D, bits, n_ckpt_cap, ckpt_interval);
+}
+
+int adkv_decode_segments(int B, int Hq, int H, int T, int D, int bits, int n_ckpt_cap,
+                         int ckpt_interval, int *bounds, int max_bounds, int *info)
+{
+    if (B <= 0 || H <= 0 || Hq <= 0 || Hq % H || T < 0 || (D != 128 && D != 256 && D != 512) ||
+        (bits != 2 && bits != 4))
+        return -1;
+    const int GQ = Hq / H;
+    if ((GQ > 1 || bits != 4) && D != 128)
+        return -1;
+    int dummy = 0;
+    Seg seg = plan_segments(n_ckpt_cap > 0 && ckpt_interval > 0 ? &dummy : nullptr, n_ckpt_cap,
+                            ckpt_interval, B * H, T, D);
+    const bool matrix_cores = D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha());
+    const bool head_table = !matrix_cores && use_head_table(B, H, GQ, bits, D, seg);
+    long wgs = 0;
+    int virt = 1;
+    if (head_table) {
+        plan_head_table(seg, B, H, T, FT_SKEW_QK);
+        const int W = ft_wgs_per_head(B, seg.nseg);
+        wgs = (long)H * seg.phys_per_head;
+        virt = (W + seg.phys_per_head - 1) / seg.phys_per_head;
+    }
+    if (bounds != nullptr && max_bounds > seg.nseg) {
+        for (int s = 0; s < seg.nseg; s++)
+            bounds[s] = seg_begin(seg, s);
+        bounds[seg.nseg] = T;
+    }
+    if (info != nullptr) {
+        info[0] = (int)wgs; // 0: not a per-head-table launch (workgroup count follows the kernel's shape)
+        info[1] = virt;
+    }
+    return seg.nseg;
 }
 
 int adkv_forward_qk_gqa(const void *q, void *k_cache, const void *k_new, void *logits,
@@ -2204,8 +2387,8 @@ int64_t adkv_forward_ov_workspace_bytes(int B, int H, int T, int D, int n_ckpt_c
     if (B <= 0 || H <= 0 || T < 0 || n_ckpt_cap <= 0 || ckpt_interval <= 0)
         return 0;
     int dummy = 0;
-    const Seg seg = plan_segments(&dummy, n_ckpt_cap, ckpt_interval, B * H, T, D);
-    return seg.nseg > 1 ? (int64_t)seg.nseg * B * H * D * 4 : 0;
+    const int nseg = max_plan_segments(&dummy, n_ckpt_cap, ckpt_interval, B, H, T, D);
+    return nseg > 1 ? (int64_t)nseg * B * H * D * 4 : 0;
 }
 
 } // extern "C"
@@ -2245,10 +2428,13 @@ static int forward_ov_impl(const void *attn, void *v_cache, const void *v_new, v
         seg.row_pitch = ld;
     const bool matrix_cores = D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha());
     const bool head_table = !matrix_cores && use_head_table(B, H, GQ, bits, D, seg);
-    // per-head table, two or four segments: the waves of one sequence pair sit in the same
-    // workgroup (interleave_segment) and add their partial outputs there; no second launch and
-    // nothing in the workspace
-    seg.combine = (head_table && (seg.nseg == 2 || seg.nseg == 4)) ? 1 : 0;
+    if (head_table)
+        plan_head_table(seg, B, H, T, FT_SKEW_OV);
+    // per-head table, two or four segments, one virtual workgroup per workgroup: the waves of one
+    // sequence pair sit in the same workgroup (interleave_segment) and add their partial outputs
+    // there; no second launch and nothing in the workspace
+    seg.combine = (head_table && (seg.nseg == 2 || seg.nseg == 4) &&
+                   seg.phys_per_head == ft_wgs_per_head(B, seg.nseg)) ? 1 : 0;
     if (seg.nseg > 1 && !seg.combine) {
         if (!workspace || workspace_bytes < (int64_t)seg.nseg * BH * GQ * D * 4)
             return ADKV_E_WORKSPACE;
@@ -2353,11 +2539,14 @@ int adkv_forward_ov_noalloc(const void *attn, void *v_cache, const void *v_new, 
     if (ckpt != nullptr && B > 0 && H > 0 && Hq > 0 && Hq % H == 0 && T >= 0 && n_ckpt_cap > 0 &&
         ckpt_interval > 0 && (D == 128 || D == 256 || D == 512)) {
         int dummy = 0;
-        const Seg seg = plan_segments(&dummy, n_ckpt_cap, ckpt_interval, B * H, T, D);
+        Seg seg = plan_segments(&dummy, n_ckpt_cap, ckpt_interval, B * H, T, D);
         const int GQ = Hq / H;
         const bool matrix_cores = D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha());
-        const bool in_workgroup = !matrix_cores && (seg.nseg == 2 || seg.nseg == 4) &&
-                                  use_head_table(B, H, GQ, bits, D, seg);
+        bool in_workgroup = false;
+        if (!matrix_cores && use_head_table(B, H, GQ, bits, D, seg)) {
+            plan_head_table(seg, B, H, T, FT_SKEW_OV);
+            in_workgroup = (seg.nseg == 2 || seg.nseg == 4) && seg.phys_per_head == ft_wgs_per_head(B, seg.nseg);
+        }
         if (seg.nseg > 1 && !in_workgroup)
             need = (int64_t)seg.nseg * B * Hq * D * 4;
     }

@@ -56,6 +56,20 @@ class LlamaAttention_ADKV(LlamaAttention):
     def _adkv_params(self, side: str) -> tuple[torch.Tensor, ...]:
         return tuple(getattr(self, f"{side}_{name}") for name in ADKV_PARAM_FIELDS)
 
+    def _apply(self, fn, recurse=True):
+        # model.to(torch.bfloat16) / .half() casts every floating-point buffer.  The recurrence is
+        # fp16 whatever the weights are (the kernels take fp16 parameters only, as the reference's
+        # do: gemv.cu:375-382), and a round trip through bfloat16 would drop three mantissa bits of
+        # the calibrated values: these ten buffers follow the module's device, never its dtype.
+        names = [f"{side}_{name}" for side in ("key", "value") for name in ADKV_PARAM_FIELDS]
+        kept = {n: self._buffers[n] for n in names if self._buffers.get(n) is not None}
+        super()._apply(fn, recurse)
+        for n, old in kept.items():
+            new = self._buffers[n]
+            if new.dtype != torch.float16:
+                self._buffers[n] = old.to(device=new.device)
+        return self
+
     def forward(self, hidden_states, position_embeddings=None, attention_mask=None,
                 past_key_values=None, cache_position=None, use_cache: bool = True, **kwargs):
         lead = hidden_states.shape[:-1]

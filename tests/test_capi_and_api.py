@@ -57,7 +57,9 @@ def test_argument_validation_in_c_abi_needs_no_device():
     assert L.adkv_forward_ov_workspace_bytes(1, 1, 64, 128, 8, 16) == 4 * 1 * 1 * 128 * 4
     ov = [one] * 9 + [1, 1, 64, 128, 16, None, one, 8, 16, None, 0, None]
     assert L.adkv_forward_ov_ex(*ov) == -7
-    assert L.adkv_forward_ov_workspace_bytes(128, 32, 4096, 128, 17, 256) == 2 * 128 * 32 * 128 * 4
+    # the headline shape: forward_qk is cut into four uneven segments under the per-head-table plan,
+    # forward_ov into two even ones; the size covers either plan, whichever kernel family is selected
+    assert L.adkv_forward_ov_workspace_bytes(128, 32, 4096, 128, 17, 256) == 4 * 128 * 32 * 128 * 4
 
 
 def test_paired_append_and_fused_decode_validation_needs_no_device():
@@ -75,6 +77,38 @@ def test_paired_append_and_fused_decode_validation_needs_no_device():
     fused = [one] * 5 + [arr5, arr5, None, 1, 1.0, one, None, 0, 1, 1, 1, 8, 128, 2, 4, 0,
              None, None, 0, 0, one, 1 << 20, None]
     assert L.adkv_decode_step(*fused) == -6                                # activation dtype must be f16 / bf16
+
+
+def test_segment_plans_cut_at_checkpoints_and_cover_the_context():
+    """adkv_decode_segments: boundaries start at 0, end at T, increase strictly, inner ones lie on
+    checkpoints that exist (index below n_ckpt_cap); uneven plans give the oldest wave slot of a
+    SIMD the longest segment of its group of four.  Host logic only."""
+    L = _lib.lib()
+    for (B, Hq, H, T, D, bits, S) in [(128, 32, 32, 4096, 128, 4, 256), (64, 32, 32, 4096, 128, 4, 256),
+                                      (352, 32, 32, 4096, 128, 4, 256), (32, 32, 32, 4097, 128, 4, 128),
+                                      (34, 32, 32, 3000, 128, 4, 64), (128, 32, 32, 640, 128, 4, 256),
+                                      (16, 32, 8, 131072, 128, 2, 256), (1, 32, 32, 32768, 128, 4, 256),
+                                      (128, 32, 32, 4096, 128, 4, 0), (3, 5, 5, 1000, 256, 4, 8)]:
+        ncap = T // S + 1 if S else 0
+        b = (ctypes.c_int * 600)()
+        info = (ctypes.c_int * 2)()
+        n = L.adkv_decode_segments(B, Hq, H, T, D, bits, ncap, S, b, 600, info)
+        assert n >= 1, (B, T)
+        bounds = list(b[:n + 1])
+        assert bounds[0] == 0 and bounds[-1] == T
+        assert all(x < y for x, y in zip(bounds, bounds[1:])), bounds
+        for x in bounds[1:-1]:
+            assert S and x % S == 0 and x // S - 1 < ncap, (bounds, S)
+        name = L.adkv_decode_kernel_name(B, Hq, H, T, D, bits, ncap, S).decode()
+        if "uneven" in name:
+            assert n % 4 == 0 and info[0] > 0 and info[1] >= 1
+            for g in range(n // 4):
+                lens = [bounds[4 * g + k + 1] - bounds[4 * g + k] for k in range(4)]
+                assert lens[0] >= lens[1] >= lens[2] >= lens[3] - S, lens      # the last may hold a ragged tail
+    assert L.adkv_decode_segments(1, 3, 2, 10, 128, 4, 0, 0, None, 0, None) == -1        # 3 query heads over 2
+    # the headline shape: shares 7 : 5 : 2 : 2 of 16 intervals, 256 workgroups walking two virtual ones each
+    n = L.adkv_decode_segments(128, 32, 32, 4096, 128, 4, 17, 256, b, 600, info)
+    assert n == 4 and list(b[:5]) == [0, 1792, 3072, 3584, 4096] and list(info) == [256, 2]
 
 
 def test_static_scratch_entry_points_return_a_code_without_a_device():

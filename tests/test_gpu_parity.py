@@ -816,6 +816,78 @@ def test_per_head_table_kernels(gpu, oracle, B, H, T, S):
         _lib.lib().adkv_set_mha_kernel(-1)
 
 
+@pytest.mark.parametrize("B,H,T,S", [(18, 64, 203, 8),     # two virtual workgroups per workgroup
+                                     (34, 64, 203, 8)])    # ten per head over four workgroups: 3, 3, 2, 2
+def test_virtual_workgroups_with_uneven_segments(gpu, oracle, B, H, T, S):
+    """The per-head-table kernels on a plan that only big launches get by themselves: segments of
+    unequal length (the four wave slots of a SIMD get unequal shares), several virtual workgroups
+    walked through by each launched workgroup, partial outputs through the workspace.  Forced on
+    a mid-sized shape.  Appended codes equal a one-shot encode of T+1 tokens; state, checkpoints,
+    logits and outputs equal those of the shared-table kernels (which cut the context evenly);
+    sampled (sequence, head) pairs are held to the oracle."""
+    from adkv_amd import _lib
+    import ctypes
+    L = _lib.lib()
+    D = 128
+    x, p = _inputs(B, H, T + 1, D, seed=21)
+    pg = [t.to(gpu) for t in p.astuple()]
+    xg = x.to(gpu)
+    ncap = (T + 8) // S + 1
+    full = synth.alloc_cache(B, H, T + 9, D, gpu)
+    gemv.encode_kv(full, xg, *pg, SMIN, SMAX)
+    cache = synth.alloc_cache(B, H, T + 9, D, gpu)
+    ck = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=gpu)
+    st_enc = torch.zeros(B, H, D, 2, dtype=torch.float16, device=gpu)
+    gemv.encode_kv(cache, xg[:, :, :T].contiguous(), *pg, SMIN, SMAX, state_out=st_enc, ckpt=ck, ckpt_interval=S)
+    g = torch.Generator().manual_seed(4)
+    q = torch.randn(B, H, 1, D, generator=g).half().to(gpu)
+    attn = torch.softmax(2.0 * torch.randn(B, H, T + 1, generator=g), dim=-1).half().to(gpu)
+    xn = xg[:, :, T:].contiguous()
+
+    def run(mode):
+        L.adkv_set_mha_kernel(mode)
+        try:
+            kc, vc, ckk, ckv = cache.clone(), cache.clone(), ck.clone(), ck.clone()
+            sk, sv = torch.zeros_like(st_enc), torch.zeros_like(st_enc)
+            lg = gemv.forward_qk(q, kc, xn, *pg, T, SMIN, SMAX, state_out=sk, ckpt=ckk, ckpt_interval=S)
+            o = gemv.forward_ov(attn, vc, xn, *pg, SMIN, SMAX, state_out=sv, ckpt=ckv, ckpt_interval=S)
+            torch.cuda.synchronize()
+            return lg, o, kc, vc, ckk, ckv, sk, sv
+        finally:
+            L.adkv_set_mha_kernel(-1)
+
+    L.adkv_set_mha_kernel(2)
+    try:
+        b = (ctypes.c_int * 80)()
+        info = (ctypes.c_int * 2)()
+        n = L.adkv_decode_segments(B, H, H, T, D, 4, ncap, S, b, 80, info)
+        name = L.adkv_decode_kernel_name(B, H, H, T, D, 4, ncap, S).decode()
+    finally:
+        L.adkv_set_mha_kernel(-1)
+    assert "uneven" in name and n in (4, 8) and info[1] >= 2, (name, n, list(info))
+    lens = [b[i + 1] - b[i] for i in range(n)]
+    assert len(set(lens)) > 2, lens                                     # really uneven
+
+    got, want = run(2), run(0)
+    for a, w, what in zip(got[2:], want[2:], ("K cache", "V cache", "K checkpoints", "V checkpoints", "K state", "V state")):
+        assert torch.equal(a.view(torch.uint8), w.view(torch.uint8)), what
+    assert torch.equal(got[2], full) and torch.equal(got[3], full)
+    assert torch.equal(got[6].view(torch.int16), st_enc.view(torch.int16))
+    for a, w in ((got[0], want[0]), (got[1], want[1])):                  # summation order differs: one ulp
+        d = torch.abs(a.float() - w.float())
+        assert torch.all(d <= 2.0 ** -10 * torch.clamp(w.float().abs(), min=2.0 ** -4))
+    pn = [_np16(t) for t in p.astuple()]
+    for (bb, h) in [(0, 0), (B - 1, H - 1), (B // 2, 17), (7, 40), (B - 2, 1)]:
+        ph = [a[h:h + 1] for a in pn]
+        sub = cache[bb:bb + 1, h:h + 1].cpu().numpy().copy()
+        lw, _ = oracle.forward_qk_f16(_np16(q[bb:bb + 1, h:h + 1]), sub.copy(), _np16(xn[bb:bb + 1, h:h + 1]), *ph, T)
+        gl = _np16(got[0][bb:bb + 1, h:h + 1]).astype(np.float64)
+        assert np.all(np.abs(gl - lw) <= _ulp16(lw) + 1e-3), (bb, h)
+        ow, _ = oracle.forward_ov_f16(_np16(attn[bb:bb + 1, h:h + 1]), sub.copy(), _np16(xn[bb:bb + 1, h:h + 1]), *ph)
+        go = _np16(got[1][bb:bb + 1, h:h + 1]).astype(np.float64)
+        assert np.all(np.abs(go - ow) <= _ulp16(ow) + 1e-3), (bb, h)
+
+
 @pytest.mark.parametrize("B,H,T,S", [(2, 3, 0, 0), (1, 2, 7, 0), (2, 2, 130, 0), (2, 3, 530, 64)])
 def test_matrix_core_kernels_for_equal_heads(gpu, oracle, B, H, T, S):
     """The same matrix-core kernels with one query head per KV head (selected by the tuning knob)

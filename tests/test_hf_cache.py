@@ -502,6 +502,23 @@ def test_tiny_llama_half_precision_decode_path_matches_oracle(gpu, oracle, tmp_p
         assert np.array_equal(cache[L].value_states.cpu().numpy()[:, :, :n], caches[L][1][:, :, :n]), L
 
 
+def test_parameter_buffers_stay_fp16_when_the_model_changes_dtype():
+    """model.to(torch.bfloat16) casts floating-point buffers; the ten ADKV parameter buffers of an
+    attention module must keep fp16 and their exact values (the kernels take fp16 parameters only,
+    and bfloat16 would drop three mantissa bits of a calibrated value)."""
+    pytest.importorskip("transformers")
+    from adkv_amd.hf.llama_adkv import LlamaForCausalLM_ADKV
+    model = LlamaForCausalLM_ADKV(_tiny_cfg(2, 2))
+    att = model.model.layers[0].self_attn
+    att.key_alpha.fill_(0.9501953125)            # not representable in bfloat16
+    att.value_beta.fill_(0.0400390625)
+    model = model.to(torch.bfloat16)
+    assert att.q_proj.weight.dtype == torch.bfloat16
+    assert att.key_alpha.dtype == torch.float16 and float(att.key_alpha[0]) == 0.9501953125
+    model = model.float().half()
+    assert att.value_beta.dtype == torch.float16 and float(att.value_beta[3]) == 0.0400390625
+
+
 def test_rotary_embedding_keeps_gradients(monkeypatch):
     """Under autograd the attention module must not take the fused rotary-embedding kernel (it has
     no backward pass): the differentiable expression runs and q_proj / k_proj receive gradients.
