@@ -84,15 +84,6 @@ __device__ __forceinline__ uint2 ft_get(const uint2 *tab, uint32_t bytes, uint32
     return *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(tab) + addr);
 }
 
-// The code stream is read exactly once: a non-temporal load keeps it from displacing the logits
-// and weights (which the softmax and the next kernel read back) in the caches.
-typedef uint32_t u4v __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ uint4 ft_load_codes(const uint4 *p)
-{
-    const u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v *>(p));
-    return make_uint4(v.x, v.y, v.z, v.w);
-}
-
 // Which supergroup the main loops prefetch: PF ahead, clamped to the segment's last one (the load
 // is unconditional; a load inside a branch makes the next wait cover every load in flight).
 __device__ __forceinline__ int ft_prefetch_index(int sg, int nfull)
@@ -190,7 +181,7 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
         uint4 buf[PF][1];
 #pragma unroll
         for (int i = 0; i < PF; i++)
-            buf[i][0] = (i < nfull) ? ft_load_codes(cb + (size_t)i * G::VPS) : make_uint4(0, 0, 0, 0);
+            buf[i][0] = (i < nfull) ? load_codes(cb + (size_t)i * G::VPS) : make_uint4(0, 0, 0, 0);
         if (!un.wave_active)
             continue; // padding waves of the head's last virtual workgroup
 
@@ -238,7 +229,7 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
         auto body = [&](int sg, auto ic) {
             constexpr int i = decltype(ic)::value;
             pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
-            buf[i][0] = ft_load_codes(cb + (size_t)ft_prefetch_index(sg, nfull) * G::VPS);
+            buf[i][0] = load_codes(cb + (size_t)ft_prefetch_index(sg, nfull) * G::VPS);
             __builtin_amdgcn_sched_barrier(0);
             finish(part, sg - 1, sg > 0 ? 8 : 0);
             __builtin_amdgcn_sched_barrier(0);
@@ -366,7 +357,7 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
         uint4 wbuf[PF];
 #pragma unroll
         for (int i = 0; i < PF; i++) {
-            buf[i][0] = (i < nfull) ? ft_load_codes(cb + (size_t)i * G::VPS) : make_uint4(0, 0, 0, 0);
+            buf[i][0] = (i < nfull) ? load_codes(cb + (size_t)i * G::VPS) : make_uint4(0, 0, 0, 0);
             wbuf[i] = (i < nfull) ? load_w(i) : make_uint4(0, 0, 0, 0);
         }
         ft_fill(tab, be, tg, h);
@@ -420,7 +411,7 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
             constexpr int i = decltype(ic)::value;
             pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
             const int sgp = ft_prefetch_index(sg, nfull);
-            buf[i][0] = ft_load_codes(cb + (size_t)sgp * G::VPS);
+            buf[i][0] = load_codes(cb + (size_t)sgp * G::VPS);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int t = 0; t < 8; t += 2)

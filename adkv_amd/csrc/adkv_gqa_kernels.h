@@ -174,8 +174,8 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
     }
     const uint2 *arow = tile + (tg4 * 4 + r) * TILE_ROW64 + (lane >> 5) * 32 + qd * 8;
 
-    const int t0 = un.seg * sa.seg_tokens;
-    const int t1 = last ? T : t0 + sa.seg_tokens;
+    const int t0 = seg_begin(sa, un.seg);
+    const int t1 = last ? T : seg_end(sa, un.seg);
     uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV;
     const uint4 *cb = cbh + (size_t)(t0 / TPW) * G::VPS;
     const int nfull = (t1 - t0) / TPW;
@@ -233,7 +233,7 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
     uint2 areg[8] = {}; // read (and discarded) once before the first unit has filled it
 #pragma unroll
     for (int i = 0; i < GPF; i++)
-        buf[i] = (i < nfull) ? cb[(size_t)i * G::VPS] : make_uint4(0, 0, 0, 0);
+        buf[i] = (i < nfull) ? load_codes(cb + (size_t)i * G::VPS) : make_uint4(0, 0, 0, 0);
     if (nfull > 0) {
         code_bytes<BITS>(buf[0], nbc);
         lk.fill(lut, nbc, lane_copy, 0);
@@ -245,7 +245,7 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
         code_bytes<BITS>(buf[(i + 1) % GPF], nbn);
         // unconditional, clamped to the segment's last supergroup: a load inside a branch makes
         // the next wait cover every load in flight, this one included
-        buf[i] = cb[(size_t)min(sg + GPF, nfull - 1) * G::VPS];
+        buf[i] = load_codes(cb + (size_t)min(sg + GPF, nfull - 1) * G::VPS);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int hf = 0; hf < UPS; hf++) {
@@ -351,8 +351,8 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
         for (int c = 0; c < CPL; c++)
             acc[n][c] = (f4v){0.0f, 0.0f, 0.0f, 0.0f};
 
-    const int t0 = un.seg * sa.seg_tokens;
-    const int t1 = last ? T : t0 + sa.seg_tokens;
+    const int t0 = seg_begin(sa, un.seg);
+    const int t1 = last ? T : seg_end(sa, un.seg);
     uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh * G::NV;
     const uint4 *cb = cbh + (size_t)(t0 / TPW) * G::VPS;
     const int nfull = (t1 - t0) / TPW;
@@ -410,7 +410,7 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
     uint32_t nbc[G::NP][2], nbn[G::NP][2];
 #pragma unroll
     for (int i = 0; i < GPF; i++)
-        buf[i] = (i < nfull) ? cb[(size_t)i * G::VPS] : make_uint4(0, 0, 0, 0);
+        buf[i] = (i < nfull) ? load_codes(cb + (size_t)i * G::VPS) : make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int i = 0; i < WPF; i++)
 #pragma unroll
@@ -424,7 +424,7 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
     auto body = [&](int sg, auto ic) {
         constexpr int i = decltype(ic)::value;
         code_bytes<BITS>(buf[(i + 1) % GPF], nbn);
-        buf[i] = cb[(size_t)min(sg + GPF, nfull - 1) * G::VPS]; // unconditional: see qk_gqa_kernel
+        buf[i] = load_codes(cb + (size_t)min(sg + GPF, nfull - 1) * G::VPS); // unconditional: see qk_gqa_kernel
 #pragma unroll
         for (int hf = 0; hf < UPS; hf++) {
             const int unit = sg * UPS + hf;

@@ -60,6 +60,22 @@ template <typename V> __device__ __forceinline__ V vec_zero();
 template <> __device__ __forceinline__ uint4 vec_zero<uint4>() { return make_uint4(0, 0, 0, 0); }
 template <> __device__ __forceinline__ uint2 vec_zero<uint2>() { return make_uint2(0, 0); }
 
+// The code stream is read exactly once: a non-temporal load keeps it from displacing the logits
+// and weights (which the softmax and the next kernel read back) in the caches.  Measured on the
+// headline shape: forward_qk -1 %, forward_ov -3 %, the softmax between them -12 %.
+typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+typedef uint32_t u2v32 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint4 load_codes(const uint4 *p)
+{
+    const u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v *>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint2 load_codes(const uint2 *p)
+{
+    const u2v32 v = __builtin_nontemporal_load(reinterpret_cast<const u2v32 *>(p));
+    return make_uint2(v.x, v.y);
+}
+
 // How the time axis is cut.  seg_tokens is a multiple of ckpt_interval (itself a multiple of 8);
 // segment s covers tokens [s*seg_tokens, min((s+1)*seg_tokens, T)) and starts from checkpoint
 // s*seg_tokens/ckpt_interval - 1 (segment 0 starts from the initial parameters).
@@ -345,7 +361,7 @@ __device__ __forceinline__ void init_pairs(Pair *st, const h1 *zp, const h1 *sc,
     for (int p = 0; p < CPL / 2; p++)
         load_pair(st[p], zp, sc, al, be, tg, h * D + c0 + 2 * p);
     if (seg > 0) {
-        const int j = seg * (sa.seg_tokens / sa.ckpt_interval) - 1;
+        const int j = seg_begin(sa, seg) / sa.ckpt_interval - 1;
         load_state<CPL>(sa.ckpt + (((size_t)bx * sa.n_ckpt_cap + j) * D + c0) * 2, st);
     }
 }
@@ -788,8 +804,8 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
     for (int p = 0; p < G::NP; p++)
         qv[p] = load_act2(q + (size_t)bx * D + c0 + 2 * p, sa.act_bf16);
 
-    const int t0 = un.seg * sa.seg_tokens;
-    const int t1 = last ? T : t0 + sa.seg_tokens;
+    const int t0 = seg_begin(sa, un.seg);
+    const int t1 = last ? T : seg_end(sa, un.seg);
     using Vec = typename G::Vec;
     Vec *cbh = reinterpret_cast<Vec *>(cache) + (size_t)bx * n_super_cap * G::VPS + lh * G::NV; // this head, this lane
     const Vec *cb = cbh + (size_t)(t0 >> 3) * G::VPS;                                           // this segment
@@ -840,7 +856,7 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
     for (int i = 0; i < PF; i++) {
 #pragma unroll
         for (int v = 0; v < G::NV; v++)
-            buf[i][v] = (i < nfull) ? cb[(size_t)i * G::VPS + v] : vec_zero<Vec>();
+            buf[i][v] = (i < nfull) ? load_codes(cb + (size_t)i * G::VPS + v) : vec_zero<Vec>();
     }
     if (nfull > 0) {
         pair_bytes_of<D, CPL>(buf[0], nb);
@@ -863,7 +879,7 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
             const int sgp = min(sg + PF, nfull - 1);
 #pragma unroll
             for (int v = 0; v < G::NV; v++)
-                buf[i][v] = cb[(size_t)sgp * G::VPS + v];
+                buf[i][v] = load_codes(cb + (size_t)sgp * G::VPS + v);
         }
         __builtin_amdgcn_sched_barrier(0);
         finish(part, sg - 1, sg > 0 ? 8 : 0);
@@ -967,8 +983,8 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
     const uint32_t sel_a0 = role == 0 ? 0x0C0C0100u : role == 1 ? 0x01000C0Cu : 0x0C0C0C0Cu;
     const uint32_t sel_a1 = role == 0 ? 0x0C0C0302u : role == 1 ? 0x03020C0Cu : 0x0C0C0C0Cu;
 
-    const int t0 = un.seg * sa.seg_tokens;
-    const int t1 = last ? T : t0 + sa.seg_tokens;
+    const int t0 = seg_begin(sa, un.seg);
+    const int t1 = last ? T : seg_end(sa, un.seg);
     using Vec = typename G::Vec;
     Vec *cbh = reinterpret_cast<Vec *>(cache) + (size_t)bx * n_super_cap * G::VPS + lh * G::NV;
     const Vec *cb = cbh + (size_t)(t0 >> 3) * G::VPS;
@@ -1037,7 +1053,7 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
     for (int i = 0; i < PF; i++) {
 #pragma unroll
         for (int v = 0; v < G::NV; v++)
-            buf[i][v] = (i < nfull) ? cb[(size_t)i * G::VPS + v] : vec_zero<Vec>();
+            buf[i][v] = (i < nfull) ? load_codes(cb + (size_t)i * G::VPS + v) : vec_zero<Vec>();
         wbuf[i] = (i < nfull) ? load_w(i) : make_uint4(0, 0, 0, 0);
     }
     if (nfull > 0) {
@@ -1055,7 +1071,7 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
         const int sgp = min(sg + PF, nfull - 1);
 #pragma unroll
         for (int v = 0; v < G::NV; v++)
-            buf[i][v] = cb[(size_t)sgp * G::VPS + v];
+            buf[i][v] = load_codes(cb + (size_t)sgp * G::VPS + v);
         __builtin_amdgcn_sched_barrier(0);
         if (MM) {
 #pragma unroll
@@ -1934,6 +1950,11 @@ static bool use_head_table(int B, int H, int GQ, int bits, int D, const Seg &seg
 // checkpoint intervals: measured on the headline shape, one setting per kernel.
 constexpr unsigned FT_SKEW_QK = pack_skew(7, 5, 2, 2);
 constexpr unsigned FT_SKEW_OV = 0; // 0: even segments.  forward_ov gains nothing from uneven ones (see plan_head_table)
+// matrix-core kernels in 16-wave workgroups, measured on B=16, 32 query heads over 8 KV heads, 131072
+// tokens of 2-bit codes (64 segments, us): forward_qk 320 even, 299 with 6:5:3:2 (305 with 7:5:2:2,
+// 318 with 6:6:3:1, 330 with 8:4:2:2); forward_ov 265 even, 252 with 6:5:3:2 / 6:6:3:1 / 8:5:2:1
+constexpr unsigned GQA_SKEW_QK = pack_skew(6, 5, 3, 2);
+constexpr unsigned GQA_SKEW_OV = pack_skew(6, 5, 3, 2);
 constexpr int FT_MIN_GROUP = 8;  // checkpoint intervals a group needs for its shares to differ
 constexpr int FT_MAX_GROUPS = 16;
 
@@ -1974,6 +1995,26 @@ static void plan_head_table(Seg &seg, int B, int H, int T, unsigned skew)
         }
     }
     seg.phys_per_head = best;
+}
+
+// The same uneven shares for the kernels without virtual workgroups (matrix-core and shared-table
+// kernels in 16-wave workgroups, where a workgroup's quads of waves are the four slots of its
+// SIMDs as well): the even plan's segments, when their number is a multiple of four, are re-cut
+// in groups of four.  The segment count, and with it the workgroup count, stays what it was.
+static void plan_uneven(Seg &seg, int T, long threads, unsigned skew)
+{
+    seg.groups = 0;
+    seg.skew = skew;
+    if (skew == 0 || !seg.ckpt || seg.ckpt_interval <= 0 || threads < 1024L * 256 || seg.nseg < 4 || (seg.nseg & 3))
+        return;
+    const int avail = (T + seg.ckpt_interval - 1) / seg.ckpt_interval;
+    const int G = seg.nseg / 4;
+    if (G > FT_MAX_GROUPS || avail / G < FT_MIN_GROUP)
+        return;
+    if (uneven_cut(4 * G - 1, G, avail, skew) - 1 >= seg.n_ckpt_cap)
+        return;
+    seg.groups = G;
+    seg.intervals = avail;
 }
 
 // How many segments the forward_ov partial sums of a launch can have under either plan (what a
@@ -2288,6 +2329,8 @@ static int forward_qk_impl(const void *q, void *k_cache, const void *k_new, void
     if (ld)
         seg.row_pitch = ld;
     if (D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha())) {
+        if (GQ <= 4) // eight query heads per KV head may fall back to 8-wave workgroups
+            plan_uneven(seg, T, padded_units<32>(BH, seg.nseg) * 32, GQA_SKEW_QK);
         ADKV_DISPATCH_GQ(qk_gqa_kernel, true, (const h1 *)q, (uint4 *)k_cache, (const h1 *)k_new,
                          (h1 *)logits, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,
                          (const h1 *)beta, (const h1 *)tgt, BH, H, T, n_super_cap, (h1 *)state_out,
@@ -2332,6 +2375,8 @@ int adkv_decode_segments(int B, int Hq, int H, int T, int D, int bits, int n_ckp
     const bool head_table = !matrix_cores && use_head_table(B, H, GQ, bits, D, seg);
     long wgs = 0;
     int virt = 1;
+    if (matrix_cores && GQ <= 4)
+        plan_uneven(seg, T, padded_units<32>(B * H, seg.nseg) * 32, GQA_SKEW_QK);
     if (head_table) {
         plan_head_table(seg, B, H, T, FT_SKEW_QK);
         const int W = ft_wgs_per_head(B, seg.nseg);
@@ -2442,6 +2487,8 @@ static int forward_ov_impl(const void *attn, void *v_cache, const void *v_new, v
             return ADKV_E_ALIGN;
     }
     if (matrix_cores) {
+        if (GQ <= 4)
+            plan_uneven(seg, T, padded_units<32>(BH, seg.nseg) * 32, GQA_SKEW_OV);
         ADKV_DISPATCH_GQ(ov_gqa_kernel, false, (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new,
                          (h1 *)out, (float *)workspace, (const h1 *)zp, (const h1 *)sc,
                          (const h1 *)alpha, (const h1 *)beta, (const h1 *)tgt, BH, H, T, n_super_cap,
