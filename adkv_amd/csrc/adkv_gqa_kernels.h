@@ -28,8 +28,20 @@ namespace adkv {
 
 constexpr int GQA_D = 128;
 constexpr int GQA_CPL = 4;
-constexpr int TILE_ROW64 = 65;               // 8-byte words per token row: 2 heads x 32 lanes + 1 pad
+// The key tile of a wave: 8 token rows of 8-byte words (a lane's two channel pairs).  The LDS
+// serves an 8-byte access of 16 lanes per clock from 32 four-byte banks, so a group of 16 lanes has
+// to touch 16 different 8-byte slots modulo 16.  Writes: lane L of a head goes to column
+// tile_col(L) of its head's 36 columns, 16 consecutive lanes to 16 consecutive words.  Reads of the
+// matrix operands: lane (row r of 4, quarter qd of 4) reads word m of its quarter from token row
+// r, eight times; the second half of a head sits 4 words further (columns 20-35), so that the
+// quarters start at 0, 8, 20, 28 = 0, 8, 4, 12 modulo 16, and a row stride of 73 = 9 modulo 16
+// spreads the four rows over 0, 9, 2, 11: all 16 (row, quarter) slots differ.  (With 32 columns per
+// head and a stride of 65 quarters 0 and 2 met in the same banks: SQ_LDS_BANK_CONFLICT was a
+// quarter of the LDS's busy cycles, and this kernel keeps the LDS busier than the vector pipe.)
+constexpr int TILE_HEAD64 = 36;              // columns per head
+constexpr int TILE_ROW64 = 73;               // 8-byte words per token row: 2 heads x 36 columns + 1
 constexpr int TILE_WORDS64 = 8 * TILE_ROW64; // per wave
+__device__ __forceinline__ int tile_col(int lane_in_head) { return lane_in_head + 4 * (lane_in_head >> 4); }
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_mov(float v)
@@ -172,7 +184,8 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
             qb[n][m] = (g < GQ) ? four : make_uint2(0u, 0u);
         }
     }
-    const uint2 *arow = tile + (tg4 * 4 + r) * TILE_ROW64 + (lane >> 5) * 32 + qd * 8;
+    const uint2 *arow = tile + (tg4 * 4 + r) * TILE_ROW64 + (lane >> 5) * TILE_HEAD64 + tile_col(qd * 8);
+    const int wcol = (lane >> 5) * TILE_HEAD64 + tile_col(lane & 31); // where this lane's values go in a row
 
     const int t0 = seg_begin(sa, un.seg);
     const int t1 = last ? T : seg_end(sa, un.seg);
@@ -223,7 +236,7 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
             kh[p] = as_u32(qs + s.zp);
             update_pair_abs(s, qa, qs);
         }
-        tile[t * TILE_ROW64 + lane] = make_uint2(kh[0], kh[1]);
+        tile[t * TILE_ROW64 + wcol] = make_uint2(kh[0], kh[1]);
         lk.refill(lut, nbnext, lane_copy, t, next_half);
         __builtin_amdgcn_sched_barrier(0);
     };
@@ -291,7 +304,7 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
                 kh[pp] = as_u32(qs + s.zp);
                 update_pair(s, qc, qs);
             }
-            tile[row * TILE_ROW64 + lane] = make_uint2(kh[0], kh[1]);
+            tile[row * TILE_ROW64 + wcol] = make_uint2(kh[0], kh[1]);
             if (++row == 8) {
                 emit_read(areg);
                 emit_finish(areg, unit, 8);
@@ -304,7 +317,7 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
         publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
     h2 deq[G::NP];
     append_new_token<D, CPL, BITS>(cbh, T, k_new + (size_t)bx * D + c0, st, deq, active, sa.act_bf16);
-    tile[row * TILE_ROW64 + lane] = make_uint2(as_u32(deq[0]), as_u32(deq[1]));
+    tile[row * TILE_ROW64 + wcol] = make_uint2(as_u32(deq[0]), as_u32(deq[1]));
     emit_read(areg);
     emit_finish(areg, unit, row + 1);
 }
