@@ -1731,7 +1731,29 @@ static inline int lanes_per_head(int D) { return D == 128 ? 32 : 64; }
 
 // Waves a SIMD should hold for packed-f16 issue to run near full rate, and SIMDs on the device.
 constexpr int WAVES_PER_SIMD_TARGET = 4;
-constexpr int N_SIMD = 256 * 4;
+// Compute units of the device the calling thread is on, asked once per device (256 on an MI355X,
+// and that is what every measurement behind the plans below was taken on).  Without a device (the
+// planning entry points can be called on a host that has none) the MI355X's count is assumed.
+static int cus()
+{
+    constexpr int MAX_DEV = 64, MI355X_CUS = 256;
+    static std::atomic<int> cached[MAX_DEV];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEV) {
+        (void)hipGetLastError(); // not this call's error to report
+        return MI355X_CUS;
+    }
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            n = MI355X_CUS;
+        }
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+static int n_simd() { return 4 * cus(); }
 
 // Segment plan for a decode launch.  Starting from the fewest segments that give every SIMD its
 // target of waves, finer splits are taken when they shorten the launch: 16-wave workgroups run one
@@ -1757,7 +1779,7 @@ static Seg plan_segments(void *ckpt, int n_ckpt_cap, int ckpt_interval, int BH, 
         return s;
     const int avail = (T + ckpt_interval - 1) / ckpt_interval;               // finest split
     const int lph = lanes_per_head(D);
-    const long units_target = (long)N_SIMD * WAVES_PER_SIMD_TARGET * (64 / lph);
+    const long units_target = (long)n_simd() * WAVES_PER_SIMD_TARGET * (64 / lph);
     long want = (units_target + BH - 1) / BH;
     if (want < 1)
         want = 1;
@@ -1770,10 +1792,10 @@ static Seg plan_segments(void *ckpt, int n_ckpt_cap, int ckpt_interval, int BH, 
     auto cost = [&](int m) {
         const int nseg = (avail + m - 1) / m;
         const long threads = (lph == 32 ? padded_units<32>(BH, nseg) : padded_units<64>(BH, nseg)) * lph;
-        if (D == 512 || threads < 1024L * 256)
+        if (D == 512 || threads < 1024L * cus())
             return (double)m;                        // small workgroups: no round structure to model
         const long wgs = (threads + 1023) / 1024;
-        return (double)((wgs + 255) / 256) * m;
+        return (double)((wgs + cus() - 1) / cus()) * m;
     };
     int best = -1;
     double best_cost = 0.0;
@@ -1803,7 +1825,7 @@ static void launch_units(long threads, int big, F256 f256, FBIG fbig)
 {
     // 16-wave workgroups share one lookup table and let a CU hold 4 waves per SIMD; small launches
     // use 4-wave workgroups so that they still spread over the CUs
-    if (big > 256 && threads >= (long)big * 256)
+    if (big > 256 && threads >= (long)big * cus())
         fbig(dim3((unsigned)((threads + big - 1) / big)), dim3(big));
     else
         f256(dim3((unsigned)((threads + 255) / 256)), dim3(256));
@@ -1822,7 +1844,7 @@ static void launch_units(long threads, int big, F256 f256, FBIG fbig)
 #define ADKV_DISPATCH_D(KERNEL, ...)                  \
     switch (D) {                                      \
     case 128:                                         \
-        if (padded_units<32>(BH, seg.nseg) / 2 <= N_SIMD) \
+        if (padded_units<32>(BH, seg.nseg) / 2 <= n_simd()) \
             ADKV_LAUNCH(KERNEL, 128, 2, 256, __VA_ARGS__); \
         else                                          \
             ADKV_LAUNCH(KERNEL, 128, 4, 1024, __VA_ARGS__); \
@@ -1845,7 +1867,7 @@ static void launch_units(long threads, int big, F256 f256, FBIG fbig)
     do {                                                                                            \
         const long threads = padded_units<32>(BH, seg.nseg) * 32;                                   \
         constexpr int GBIG = (GQV <= 4 || BIG8) ? GQV : 1; /* unused instantiation otherwise */     \
-        if ((GQV <= 4 || BIG8) && threads >= 1024L * 256)                                           \
+        if ((GQV <= 4 || BIG8) && threads >= 1024L * cus())                                         \
             hipLaunchKernelGGL((KERNEL<BB, GBIG, 1024>), dim3((unsigned)((threads + 1023) / 1024)), \
                                dim3(1024), 0, st, __VA_ARGS__);                                     \
         else                                                                                        \
@@ -1911,15 +1933,15 @@ static bool use_head_table(int B, int H, int GQ, int bits, int D, const Seg &seg
     const long BH = (long)B * H;
     const long padded = padded_units<32>((int)BH, seg.nseg);
     const long waves_shared = padded / 2;
-    if (waves_shared <= N_SIMD)
+    if (waves_shared <= n_simd())
         return false;                                 // every wave a SIMD to itself: two-channel lanes
     const long wgs_ft = (long)H * ft_wgs_per_head(B, seg.nseg);
-    const double t_ft = 0.93 * (double)((wgs_ft + 255) / 256);
+    const double t_ft = 0.93 * (double)((wgs_ft + cus() - 1) / cus());
     double t_shared;
-    if (padded * 32 >= (long)FT_BLK * 256)
-        t_shared = (double)(((padded * 32 + FT_BLK - 1) / FT_BLK + 255) / 256);
+    if (padded * 32 >= (long)FT_BLK * cus())
+        t_shared = (double)(((padded * 32 + FT_BLK - 1) / FT_BLK + cus() - 1) / cus());
     else
-        t_shared = (double)((waves_shared + N_SIMD - 1) / N_SIMD) / WAVES_PER_SIMD_TARGET;
+        t_shared = (double)((waves_shared + n_simd() - 1) / n_simd()) / WAVES_PER_SIMD_TARGET;
     return t_ft <= t_shared;
 }
 
@@ -1969,7 +1991,7 @@ static void plan_head_table(Seg &seg, int B, int H, int T, unsigned skew)
     const int avail = (T + iv - 1) / iv;
     // groups of four segments: as many as give every SIMD its four waves, FT_MIN_GROUP intervals or more each
     const long waves_per_group = (long)H * 4 * pad4(ft_pairs_per_seg(B));
-    long G = ((long)N_SIMD * WAVES_PER_SIMD_TARGET + waves_per_group - 1) / waves_per_group;
+    long G = ((long)n_simd() * WAVES_PER_SIMD_TARGET + waves_per_group - 1) / waves_per_group;
     if (G > avail / FT_MIN_GROUP)
         G = avail / FT_MIN_GROUP;
     if (G > FT_MAX_GROUPS)
@@ -1988,7 +2010,7 @@ static void plan_head_table(Seg &seg, int B, int H, int T, unsigned skew)
     int best = W;
     long best_cost = -1;
     for (int P = 1; P <= W; P++) {
-        const long cost = (((long)H * P + 255) / 256) * ((W + P - 1) / P);
+        const long cost = (((long)H * P + cus() - 1) / cus()) * ((W + P - 1) / P);
         if (best_cost < 0 || cost < best_cost) {
             best = P;
             best_cost = cost;
@@ -2005,7 +2027,7 @@ static void plan_uneven(Seg &seg, int T, long threads, unsigned skew)
 {
     seg.groups = 0;
     seg.skew = skew;
-    if (skew == 0 || !seg.ckpt || seg.ckpt_interval <= 0 || threads < 1024L * 256 || seg.nseg < 4 || (seg.nseg & 3))
+    if (skew == 0 || !seg.ckpt || seg.ckpt_interval <= 0 || threads < 1024L * cus() || seg.nseg < 4 || (seg.nseg & 3))
         return;
     const int avail = (T + seg.ckpt_interval - 1) / seg.ckpt_interval;
     const int G = seg.nseg / 4;
@@ -2141,7 +2163,7 @@ static int encode_common(void *cache, const void *kv_new,
     // Four channels per lane never win and are not instantiated.
     const long channels = (long)BH * D;
     const long tensors = second ? 2 : 1;
-    int cpl = tensors * channels > 2L * 64 * N_SIMD + 32768 ? 2 : 1;
+    int cpl = tensors * channels > 2L * 64 * n_simd() + 32768 ? 2 : 1;
     const long lanes = channels / cpl;
     const dim3 grid((unsigned)((lanes + 255) / 256), (unsigned)tensors), block(256);
     EncTensor first;
@@ -2276,7 +2298,7 @@ static const char *decode_kernel_name(int B, int Hq, int H, int T, int D, int bi
                                   ckpt_interval, B * H, T, D);
     if (D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha())) {
         const long threads = padded_units<32>(B * H, seg.nseg) * 32;
-        return threads >= 1024L * 256 ? "gqa_kernel, 16-wave workgroups (matrix cores)"
+        return threads >= 1024L * cus() ? "gqa_kernel, 16-wave workgroups (matrix cores)"
                                       : "gqa_kernel, 8-wave workgroups (matrix cores)";
     }
     if (use_head_table(B, H, GQ, bits, D, seg)) {
@@ -2287,9 +2309,9 @@ static const char *decode_kernel_name(int B, int Hq, int H, int T, int D, int bi
     }
     if (D == 128) {
         const long units = padded_units<32>(B * H, seg.nseg);
-        if (units / 2 <= N_SIMD)
+        if (units / 2 <= n_simd())
             return "kernel<128,2,256> (shared table, two channels per lane)";
-        return units * 32 >= 1024L * 256 ? "kernel<128,4,1024> (shared table)" : "kernel<128,4,256> (shared table)";
+        return units * 32 >= 1024L * cus() ? "kernel<128,4,1024> (shared table)" : "kernel<128,4,256> (shared table)";
     }
     return D == 256 ? "kernel<256,4,*> (shared table)" : "kernel<512,8,256> (shared table)";
 }
