@@ -27,40 +27,52 @@ constexpr int FT_BLK = 1024;
 constexpr int FT_WAVES = FT_BLK / 64;
 constexpr int FT_TABLE_WORDS64 = 2 * LUT_ENTRIES * 32; // uint2 elements: 2 x 64 KB
 
+// A head is spread over LPH lanes of a wave: 32 lanes with four channels each, or 16 lanes that
+// make two passes of four channels (channels 4*lane.. in the first, 64 + 4*lane.. in the second)
+// over every supergroup.  A wave then holds upw = 64 / LPH sequences of one segment.
 // host and device: how the (head, segment, sequence) units of a launch are laid out
-__host__ __device__ inline int ft_pairs_per_seg(int B) { return (B + 1) >> 1; }
-__host__ __device__ inline int ft_wgs_per_head(int B, int nseg)
+__host__ __device__ inline int ft_waves_per_seg(int B, int upw) { return (B + upw - 1) / upw; }
+__host__ __device__ inline int ft_wgs_per_head(int B, int nseg, int upw)
 {
-    return (nseg * pad4(ft_pairs_per_seg(B)) + FT_WAVES - 1) / FT_WAVES;
+    return (nseg * pad4(ft_waves_per_seg(B, upw)) + FT_WAVES - 1) / FT_WAVES;
 }
 
+template <int LPH>
 struct FtUnit {
     int seg, bx, lh, c0;
     bool active, wave_active;
     // h: KV head; vw: virtual workgroup within the head (16 waves' worth of the head's units)
     __device__ __forceinline__ FtUnit(int B, int H, int nseg, int h, int vw)
     {
-        const int pps = ft_pairs_per_seg(B);
+        constexpr int UPW = 64 / LPH;
+        const int wps = ft_waves_per_seg(B, UPW);
         const int w = __builtin_amdgcn_readfirstlane(vw * FT_WAVES + (int)(threadIdx.x >> 6)); // wave within the head
-        int sg, pair;
-        interleave_segment(w, nseg, sg, pair);
+        int sg, wis;
+        interleave_segment(w, nseg, sg, wis);
         const int lane = threadIdx.x & 63;
-        const int b = pair * 2 + (lane >> 5);
-        lh = lane & 31;
+        const int b = wis * UPW + lane / LPH;
+        lh = lane % LPH;
         c0 = lh * 4;
-        wave_active = pair < pps;
+        wave_active = wis < wps;
         active = wave_active && b < B;
         seg = sg;
         bx = (b < B ? b : B - 1) * H + h;
     }
 };
 
-// table[j][code byte][lane] = (q pair, f pair) for channels 4*lane + 2j, 4*lane + 2j + 1 of head h
+// 32 lanes: table[j][code byte][lane] = (q pair, f pair) for channels 4*lane + 2j, 4*lane + 2j + 1
+// of head h.  16 lanes: table[pass][code byte][j][lane] for channels 64*pass + 4*lane + 2j, + 1: the
+// 16 lanes of a head read the 16 slots of one half of a 256-byte row, again whatever their codes.
+template <int LPH>
 __device__ __forceinline__ void ft_fill(uint2 *tab, const h1 *be, const h1 *tg, int h)
 {
     const int tid = threadIdx.x;
-    const int lh = tid & 31, j = (tid >> 5) & 1, cg = tid >> 6; // cg: 16 code bytes each
-    const int pi = h * 128 + 4 * lh + 2 * j;
+    const int cg = tid >> 6; // 16 code bytes each
+    const int lh = tid & (LPH - 1);
+    const int j = LPH == 32 ? (tid >> 5) & 1 : (tid >> 4) & 1;
+    const int pass = LPH == 32 ? 0 : (tid >> 5) & 1;
+    const int pi = h * 128 + 64 * pass + 4 * lh + 2 * j;
+    const int slot = LPH == 32 ? j * (LUT_ENTRIES * 32) + lh : pass * (LUT_ENTRIES * 32) + j * 16 + lh;
     const h2 b2 = *reinterpret_cast<const h2 *>(be + pi);
     const h2 t2 = *reinterpret_cast<const h2 *>(tg + pi);
     const h2 bt = b2 * t2;
@@ -70,25 +82,30 @@ __device__ __forceinline__ void ft_fill(uint2 *tab, const h1 *be, const h1 *tg, 
         const int code = cg * (LUT_ENTRIES / FT_WAVES) + i;
         const h2 q = (h2){(h1)((code & 15) - 8), (h1)((code >> 4) - 8)};
         const h2 f = pk_fma(b2, pk_abs(q), omt); // gemv.cu:163, first half
-        tab[j * (LUT_ENTRIES * 32) + code * 32 + lh] = make_uint2(as_u32(q), as_u32(f));
+        tab[slot + code * 32] = make_uint2(as_u32(q), as_u32(f));
     }
 }
 
-// lane_copy = (1 << 8) | (lane % 32) * 8.  Entry of byte k (0..3) of `bytes` in table j (0 / 1);
-// k and j must be compile-time constants after unrolling (the selector becomes a literal).
-__device__ __forceinline__ uint2 ft_get(const uint2 *tab, uint32_t bytes, uint32_t lane_copy, int k, int j)
+// The per-lane constant the table address is permuted from.
+template <int LPH>
+__device__ __forceinline__ uint32_t ft_lane_copy(int lh)
 {
-    // [0, j, bytes.byte[k], lane*8]: selector bytes 0-3 pick from lane_copy, 4-7 from bytes, 0x0C is zero
-    const uint32_t sel = (j ? 0x0C010000u : 0x0C0C0000u) | ((4u + (uint32_t)k) << 8);
-    const uint32_t addr = __builtin_amdgcn_perm(bytes, lane_copy, sel);
-    return *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(tab) + addr);
+    return LPH == 32 ? 0x100u | ((uint32_t)lh * 8u)
+                     : 0x10000u | ((128u + (uint32_t)lh * 8u) << 8) | ((uint32_t)lh * 8u);
 }
 
-// Which supergroup the main loops prefetch: PF ahead, clamped to the segment's last one (the load
-// is unconditional; a load inside a branch makes the next wait cover every load in flight).
-__device__ __forceinline__ int ft_prefetch_index(int sg, int nfull)
+// Entry of byte k (0..3) of `bytes` for pair j (0 / 1) of pass `pass`; k, j and pass must be
+// compile-time constants after unrolling (the selector becomes a literal).
+template <int LPH>
+__device__ __forceinline__ uint2 ft_get(const uint2 *tab, uint32_t bytes, uint32_t lane_copy, int k, int j, int pass)
 {
-    return min(sg + PF, nfull - 1);
+    // selector bytes 0-3 pick from lane_copy, 4-7 from bytes, 0x0C is zero
+    //   32 lanes: [0, j, bytes.byte[k], lane*8]
+    //   16 lanes: [0, pass, bytes.byte[k], j*128 + lane*8]
+    const uint32_t sel = LPH == 32 ? (j ? 0x0C010000u : 0x0C0C0000u) | ((4u + (uint32_t)k) << 8)
+                                   : (pass ? 0x0C020000u : 0x0C0C0000u) | ((4u + (uint32_t)k) << 8) | (j ? 1u : 0u);
+    const uint32_t addr = __builtin_amdgcn_perm(bytes, lane_copy, sel);
+    return *reinterpret_cast<const uint2 *>(reinterpret_cast<const char *>(tab) + addr);
 }
 
 // The main loop needs zp, sc and alpha only (the table holds what beta and the target give); the
@@ -132,9 +149,14 @@ __device__ __forceinline__ void update_pair_f(Pair &p, h2 f, h2 qs)
 // ---------------------------------------------------------------------------------------------
 //
 // A workgroup serves one head and walks through one or more VIRTUAL workgroups of that head
-// (sa.phys_per_head apart), each 16 waves' worth of (sequence pair, segment) units, without a
+// (sa.phys_per_head apart), each 16 waves' worth of (sequences, segment) units, without a
 // barrier between them: the table is built once, and a wave that finishes its unit goes straight
 // on to its unit of the next virtual workgroup.
+//
+// LPH = 16: a lane makes two passes over every supergroup (32 + 32 channel-pair tokens), so the
+// reduction of the eight partial logits, the store and the loop overhead are paid once per eight
+// channels instead of once per four.
+template <int LPH>
 __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
     const h1 *__restrict__ q, uint4 *__restrict__ cache, const h1 *__restrict__ k_new,
     h1 *__restrict__ out,
@@ -142,73 +164,81 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
     const h1 *__restrict__ be, const h1 *__restrict__ tg,
     int B, int H, int T, int n_super_cap, h1 *__restrict__ state_out, Seg sa)
 {
-    constexpr int D = 128, CPL = 4;
+    constexpr int D = 128, CPL = 4; // per pass
     using G = Geo<D, CPL>;
+    constexpr int NPASS = 32 / LPH, UPW = 64 / LPH;
+    constexpr int PFQ = PF / NPASS; // supergroups in flight: the same bytes per lane either way
     __shared__ uint2 tab[FT_TABLE_WORDS64]; // the only LDS object: sits at offset 0
     const int h = (int)blockIdx.x / sa.phys_per_head;
     const int pw = (int)blockIdx.x % sa.phys_per_head;
-    const int wph = ft_wgs_per_head(B, sa.nseg);
+    const int wph = ft_wgs_per_head(B, sa.nseg, UPW);
     const int lane = threadIdx.x & 63;
-    const int tk = token_of_lane(lane);
+    const int tk = LPH == 32 ? token_of_lane(lane) : token_of_lane16(lane);
     // The table is built before the loop: a barrier under a condition inside it, even a uniform
     // one, costs the loop body some twenty registers and spills.
-    ft_fill(tab, be, tg, h);
+    ft_fill<LPH>(tab, be, tg, h);
     __syncthreads();
 
     for (int vw = pw; vw < wph; vw += sa.phys_per_head) {
-        const FtUnit un(B, H, sa.nseg, h, vw);
-        const uint32_t lane_copy = 0x100u | ((uint32_t)un.lh * 8u);
+        const FtUnit<LPH> un(B, H, sa.nseg, h, vw);
+        const uint32_t lane_copy = ft_lane_copy<LPH>(un.lh);
         const int bx = un.bx, lh = un.lh, c0 = un.c0;
         const bool active = un.active;
         const bool last = un.seg == sa.nseg - 1;
 
-        Pair st[G::NP];
-        h2 qv[G::NP];
-        ft_init_pairs(st, zp, sc, al, h, bx, c0, un.seg, sa);
+        Pair st[NPASS * G::NP];
+        h2 qv[NPASS * G::NP];
 #pragma unroll
-        for (int p = 0; p < G::NP; p++)
-            qv[p] = load_act2(q + (size_t)bx * D + c0 + 2 * p, sa.act_bf16);
+        for (int ps = 0; ps < NPASS; ps++) {
+            ft_init_pairs(st + ps * G::NP, zp, sc, al, h, bx, c0 + 64 * ps, un.seg, sa);
+#pragma unroll
+            for (int p = 0; p < G::NP; p++)
+                qv[ps * G::NP + p] = load_act2(q + (size_t)bx * D + c0 + 64 * ps + 2 * p, sa.act_bf16);
+        }
 
         const int t0 = seg_begin(sa, un.seg);
         const int t1 = last ? T : seg_end(sa, un.seg);
-        uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh;
+        uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh; // pass ps: vector lh + LPH*ps
         const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;
         h1 *ob = out + (size_t)bx * sa.row_pitch + t0;
         const int nfull = (t1 - t0) >> 3;
-        const bool storer = active && (lane & 3) == 0;
+        const bool storer = active && (LPH == 32 ? (lane & 3) == 0 : (lane & 1) == 0);
 
         // (padding waves have valid, clamped addresses and simply drop what they loaded)
-        uint4 buf[PF][1];
+        uint4 buf[PFQ][NPASS];
 #pragma unroll
-        for (int i = 0; i < PF; i++)
-            buf[i][0] = (i < nfull) ? load_codes(cb + (size_t)i * G::VPS) : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < PFQ; i++)
+#pragma unroll
+            for (int ps = 0; ps < NPASS; ps++)
+                buf[i][ps] = (i < nfull) ? load_codes(cb + (size_t)i * G::VPS + LPH * ps) : make_uint4(0, 0, 0, 0);
         if (!un.wave_active)
             continue; // padding waves of the head's last virtual workgroup
 
         auto finish = [&](const float *part, int sg, int ntok) {
-            const float s = reduce8_head32(part);
+            const float s = LPH == 32 ? reduce8_head32(part) : reduce8_head16(part);
             if (storer && tk < ntok)
                 ob[sg * 8 + tk] = (h1)s;
         };
 
-        // one token of the current supergroup, then the lookups of the same slot of the next one
-        auto token = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2], float &out_t) {
-            float acc;
+        // one token of the current pass, then the lookups of the same slot of the next pass
+        auto token = [&](int t, auto pc, uint2 (*e)[8], const uint32_t (*nb)[2], float &out_t) {
+            constexpr int ps = decltype(pc)::value;
+            float acc = out_t;
 #pragma unroll
             for (int p = 0; p < G::NP; p++) {
-                Pair &s = st[p];
+                Pair &s = st[ps * G::NP + p];
                 const h2 qs = as_h2(e[p][t].x) * s.sc;
                 const h2 kh = qs + s.zp;
-                if (p == 0)
+                if (ps == 0 && p == 0)
                     acc = dot2_from_zero(qv[p], kh);
                 else
-                    acc = __builtin_amdgcn_fdot2(qv[p], kh, acc, false);
+                    acc = __builtin_amdgcn_fdot2(qv[ps * G::NP + p], kh, acc, false);
                 update_pair_f(s, as_h2(e[p][t].y), qs);
             }
             out_t = acc;
 #pragma unroll
             for (int p = 0; p < G::NP; p++)
-                e[p][t] = ft_get(tab, nb[p][t & 1], lane_copy, t >> 1, p);
+                e[p][t] = ft_get<LPH>(tab, nb[p][t & 1], lane_copy, t >> 1, p, (ps + 1) % NPASS);
             __builtin_amdgcn_sched_barrier(0);
         };
 
@@ -216,66 +246,83 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
         uint32_t nb[G::NP][2];
         float part[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         if (nfull > 0) {
-            pair_bytes_of<D, CPL>(buf[0], nb);
+            pair_bytes_of<D, CPL>(&buf[0][0], nb);
 #pragma unroll
             for (int t = 0; t < 8; t++)
 #pragma unroll
                 for (int p = 0; p < G::NP; p++)
-                    lk[p][t] = ft_get(tab, nb[p][t & 1], lane_copy, t >> 1, p);
+                    lk[p][t] = ft_get<LPH>(tab, nb[p][t & 1], lane_copy, t >> 1, p, 0);
         }
         // One supergroup; i = its buffer in the rotation.  Nothing conditional: the trip count is
-        // wave-uniform, the prefetch index is clamped, and the reduction of the previous supergroup
+        // wave-uniform, the prefetch index is clamped to the segment's last supergroup (the load is
+        // unconditional; a load inside a branch makes the next wait cover every load in flight), and the reduction of the previous supergroup
         // (done here, between the lookups' issue and their first use) stores nothing for sg == 0.
         auto body = [&](int sg, auto ic) {
             constexpr int i = decltype(ic)::value;
-            pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
-            buf[i][0] = load_codes(cb + (size_t)ft_prefetch_index(sg, nfull) * G::VPS);
-            __builtin_amdgcn_sched_barrier(0);
-            finish(part, sg - 1, sg > 0 ? 8 : 0);
-            __builtin_amdgcn_sched_barrier(0);
+            static_for<NPASS>([&](auto pc) {
+                constexpr int ps = decltype(pc)::value;
+                // the code bytes of the pass after this one: same supergroup, or the next one's first
+                if (ps + 1 < NPASS)
+                    pair_bytes_of<D, CPL>(&buf[i][(ps + 1) % NPASS], nb);
+                else
+                    pair_bytes_of<D, CPL>(&buf[(i + 1) % PFQ][0], nb);
+                buf[i][ps] = load_codes(cb + (size_t)min(sg + PFQ, nfull - 1) * G::VPS + LPH * ps);
+                __builtin_amdgcn_sched_barrier(0);
+                if (ps == 0) {
+                    finish(part, sg - 1, sg > 0 ? 8 : 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
 #pragma unroll
-            for (int t = 0; t < 8; t++)
-                token(t, lk, nb, part[t]);
+                for (int t = 0; t < 8; t++)
+                    token(t, pc, lk, nb, part[t]);
+            });
         };
-        rotate_over<PF>(nfull, body);
+        rotate_over<PFQ>(nfull, body);
         if (nfull > 0)
             finish(part, nfull - 1, 8);
         if (!last)
             continue;
 
         // ragged tail: T % 8 tokens of the last supergroup (gemv.cu:648-654); plain arithmetic
-        ft_load_beta(st, be, tg, h, c0);
         const int ntail = (t1 - t0) & 7;
-        if (ntail) {
-            float tp[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-            uint32_t w[4];
-            vec_words(cb[(size_t)nfull * G::VPS], w);
+        float tp[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-            for (int pp = 0; pp < 2; pp++) {
-                Pair &s = st[pp];
-                for (int tt = 0; tt < ntail; tt++) {
-                    const h2 qc = extract_pair<4>(w[2 * pp], w[2 * pp + 1], tt);
-                    const h2 qs = qc * s.sc;
-                    const float d = __builtin_amdgcn_fdot2(qv[pp], qs + s.zp, 0.0f, false);
+        for (int ps = 0; ps < NPASS; ps++) {
+            ft_load_beta(st + ps * G::NP, be, tg, h, c0 + 64 * ps);
+            if (ntail) {
+                uint32_t w[4];
+                vec_words(cb[(size_t)nfull * G::VPS + LPH * ps], w);
 #pragma unroll
-                    for (int k = 0; k < 8; k++)
-                        tp[k] += (k == tt) ? d : 0.0f;
-                    update_pair(s, qc, qs);
+                for (int pp = 0; pp < 2; pp++) {
+                    Pair &s = st[ps * G::NP + pp];
+                    for (int tt = 0; tt < ntail; tt++) {
+                        const h2 qc = extract_pair<4>(w[2 * pp], w[2 * pp + 1], tt);
+                        const h2 qs = qc * s.sc;
+                        const float d = __builtin_amdgcn_fdot2(qv[ps * G::NP + pp], qs + s.zp, 0.0f, false);
+#pragma unroll
+                        for (int k = 0; k < 8; k++)
+                            tp[k] += (k == tt) ? d : 0.0f;
+                        update_pair(s, qc, qs);
+                    }
                 }
             }
-            finish(tp, nfull, ntail);
         }
+        if (ntail)
+            finish(tp, nfull, ntail);
 
-        if (active)
-            publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
-
-        h2 deq[G::NP];
-        append_new_token<D, CPL>(cbh, T, k_new + (size_t)bx * D + c0, st, deq, active, sa.act_bf16);
         float self = 0.0f;
 #pragma unroll
-        for (int p = 0; p < G::NP; p++)
-            self = __builtin_amdgcn_fdot2(qv[p], deq[p], self, false);
-        self = head_allreduce<G::LPH>(self);
+        for (int ps = 0; ps < NPASS; ps++) {
+            if (active)
+                publish_state<D, CPL>(st + ps * G::NP, state_out, sa, bx, c0 + 64 * ps, T);
+            h2 deq[G::NP];
+            append_new_token<D, CPL>(cbh + LPH * ps, T, k_new + (size_t)bx * D + c0 + 64 * ps, st + ps * G::NP, deq,
+                                     active, sa.act_bf16);
+#pragma unroll
+            for (int p = 0; p < G::NP; p++)
+                self = __builtin_amdgcn_fdot2(qv[ps * G::NP + p], deq[p], self, false);
+        }
+        self = head_allreduce<LPH>(self);
         if (active && lh == 0)
             out[(size_t)bx * sa.row_pitch + T] = (h1)self;
     }
@@ -306,6 +353,7 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
 // never needs more).  sa.combine: the two or four segments of a sequence pair sit in the same
 // workgroup and are added there; otherwise every segment stores its fp32 partial sums for
 // ov_finalize_kernel.
+template <int LPH>
 __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
     const h1 *__restrict__ attn, uint4 *__restrict__ cache, const h1 *__restrict__ v_new,
     h1 *__restrict__ out, float *__restrict__ partial,
@@ -313,10 +361,12 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
     const h1 *__restrict__ be, const h1 *__restrict__ tg,
     int B, int H, int T, int n_super_cap, h1 *__restrict__ state_out, Seg sa)
 {
-    constexpr int D = 128, CPL = 4;
+    constexpr int D = 128, CPL = 4; // per pass
     using G = Geo<D, CPL>;
+    constexpr int NPASS = 32 / LPH, UPW = 64 / LPH;
+    constexpr int PFQ = PF / NPASS;
     __shared__ uint2 tab[FT_TABLE_WORDS64];
-    const int wph = ft_wgs_per_head(B, sa.nseg);
+    const int wph = ft_wgs_per_head(B, sa.nseg, UPW);
     const int h = (int)blockIdx.x / wph;
     const int BH = B * H;
     // selectors that turn the word (w[t], w[t+1]) into this lane's two A registers
@@ -324,23 +374,25 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
     const uint32_t sel_a0 = role == 0 ? 0x0C0C0100u : role == 1 ? 0x01000C0Cu : 0x0C0C0C0Cu;
     const uint32_t sel_a1 = role == 0 ? 0x0C0C0302u : role == 1 ? 0x03020C0Cu : 0x0C0C0C0Cu;
     {
-        const FtUnit un(B, H, sa.nseg, h, (int)blockIdx.x % wph);
-        const uint32_t lane_copy = 0x100u | ((uint32_t)un.lh * 8u);
+        const FtUnit<LPH> un(B, H, sa.nseg, h, (int)blockIdx.x % wph);
+        const uint32_t lane_copy = ft_lane_copy<LPH>(un.lh);
         const int bx = un.bx, lh = un.lh, c0 = un.c0;
         const bool active = un.active;
         const bool last = un.seg == sa.nseg - 1;
 
-        Pair st[G::NP];
-        float acc[CPL];
-        f4v acc4[G::NP];
-        ft_init_pairs(st, zp, sc, al, h, bx, c0, un.seg, sa);
+        Pair st[NPASS * G::NP];
+        float acc[NPASS * CPL];
+        f4v acc4[NPASS * G::NP];
 #pragma unroll
-        for (int p = 0; p < G::NP; p++)
+        for (int ps = 0; ps < NPASS; ps++)
+            ft_init_pairs(st + ps * G::NP, zp, sc, al, h, bx, c0 + 64 * ps, un.seg, sa);
+#pragma unroll
+        for (int p = 0; p < NPASS * G::NP; p++)
             acc4[p] = (f4v){0.0f, 0.0f, 0.0f, 0.0f};
 
         const int t0 = seg_begin(sa, un.seg);
         const int t1 = last ? T : seg_end(sa, un.seg);
-        uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh;
+        uint4 *cbh = cache + (size_t)bx * n_super_cap * G::VPS + lh; // pass ps: vector lh + LPH*ps
         const uint4 *cb = cbh + (size_t)(t0 >> 3) * G::VPS;
         const h1 *wrow = attn + (size_t)bx * sa.row_pitch;
         const h1 *wb = wrow + t0;
@@ -353,14 +405,16 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
         };
         // the first code words and weights, like the parameters above, are requested before the
         // table is built, so that their latency runs beside the fill instead of after it
-        uint4 buf[PF][1];
-        uint4 wbuf[PF];
+        uint4 buf[PFQ][NPASS];
+        uint4 wbuf[PFQ];
 #pragma unroll
-        for (int i = 0; i < PF; i++) {
-            buf[i][0] = (i < nfull) ? load_codes(cb + (size_t)i * G::VPS) : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < PFQ; i++) {
+#pragma unroll
+            for (int ps = 0; ps < NPASS; ps++)
+                buf[i][ps] = (i < nfull) ? load_codes(cb + (size_t)i * G::VPS + LPH * ps) : make_uint4(0, 0, 0, 0);
             wbuf[i] = (i < nfull) ? load_w(i) : make_uint4(0, 0, 0, 0);
         }
-        ft_fill(tab, be, tg, h);
+        ft_fill<LPH>(tab, be, tg, h);
         __syncthreads();
         if (!un.wave_active) {
             if (sa.combine) { // the two barriers of the in-workgroup sum below
@@ -370,125 +424,151 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
             return;
         }
 
-        // two tokens of the current supergroup on the matrix cores, then the lookups of the same two
-        // slots of the next one
-        auto token2 = [&](int t, uint2 (*e)[8], const uint32_t (*nb)[2], const uint4 wv) {
-            const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
-            const uint32_t w2 = ww[t >> 1];
-            const h4v a = as_h4(__builtin_amdgcn_perm(w2, w2, sel_a0), __builtin_amdgcn_perm(w2, w2, sel_a1));
+        // two tokens of the current pass on the matrix cores, then the lookups of the same two
+        // slots of the next pass.  The A operands are built in the first pass and kept for the second.
+        h4v aop[4];
+        auto token2 = [&](int t, auto pc, uint2 (*e)[8], const uint32_t (*nb)[2], const uint4 wv) {
+            constexpr int ps = decltype(pc)::value;
+            if (ps == 0) {
+                const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+                const uint32_t w2 = ww[t >> 1];
+                aop[t >> 1] = as_h4(__builtin_amdgcn_perm(w2, w2, sel_a0), __builtin_amdgcn_perm(w2, w2, sel_a1));
+            }
+            const h4v a = aop[t >> 1];
             uint32_t vd[G::NP][2];
 #pragma unroll
             for (int k = 0; k < 2; k++)
 #pragma unroll
                 for (int p = 0; p < G::NP; p++) {
-                    Pair &s = st[p];
+                    Pair &s = st[ps * G::NP + p];
                     const h2 qs = as_h2(e[p][t + k].x) * s.sc;
                     vd[p][k] = as_u32(qs + s.zp);
                     update_pair_f(s, as_h2(e[p][t + k].y), qs);
                 }
 #pragma unroll
             for (int p = 0; p < G::NP; p++)
-                acc4[p] = __builtin_amdgcn_mfma_f32_4x4x4f16(a, as_h4(vd[p][0], vd[p][1]), acc4[p], 0, 0, 0);
+                acc4[ps * G::NP + p] = __builtin_amdgcn_mfma_f32_4x4x4f16(a, as_h4(vd[p][0], vd[p][1]),
+                                                                          acc4[ps * G::NP + p], 0, 0, 0);
 #pragma unroll
             for (int k = 0; k < 2; k++)
 #pragma unroll
                 for (int p = 0; p < G::NP; p++)
-                    e[p][t + k] = ft_get(tab, nb[p][(t + k) & 1], lane_copy, (t + k) >> 1, p);
+                    e[p][t + k] = ft_get<LPH>(tab, nb[p][(t + k) & 1], lane_copy, (t + k) >> 1, p, (ps + 1) % NPASS);
             __builtin_amdgcn_sched_barrier(0);
         };
 
         uint2 lk[G::NP][8];
         uint32_t nb[G::NP][2];
         if (nfull > 0) {
-            pair_bytes_of<D, CPL>(buf[0], nb);
+            pair_bytes_of<D, CPL>(&buf[0][0], nb);
 #pragma unroll
             for (int t = 0; t < 8; t++)
 #pragma unroll
                 for (int p = 0; p < G::NP; p++)
-                    lk[p][t] = ft_get(tab, nb[p][t & 1], lane_copy, t >> 1, p);
+                    lk[p][t] = ft_get<LPH>(tab, nb[p][t & 1], lane_copy, t >> 1, p, 0);
         }
         auto body = [&](int sg, auto ic) {
             constexpr int i = decltype(ic)::value;
-            pair_bytes_of<D, CPL>(buf[(i + 1) % PF], nb);
-            const int sgp = ft_prefetch_index(sg, nfull);
-            buf[i][0] = load_codes(cb + (size_t)sgp * G::VPS);
-            __builtin_amdgcn_sched_barrier(0);
+            const int sgp = min(sg + PFQ, nfull - 1);
+            static_for<NPASS>([&](auto pc) {
+                constexpr int ps = decltype(pc)::value;
+                if (ps + 1 < NPASS)
+                    pair_bytes_of<D, CPL>(&buf[i][(ps + 1) % NPASS], nb);
+                else
+                    pair_bytes_of<D, CPL>(&buf[(i + 1) % PFQ][0], nb);
+                buf[i][ps] = load_codes(cb + (size_t)sgp * G::VPS + LPH * ps);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int t = 0; t < 8; t += 2)
-                token2(t, lk, nb, wbuf[i]);
+                for (int t = 0; t < 8; t += 2)
+                    token2(t, pc, lk, nb, wbuf[i]);
+            });
             wbuf[i] = load_w(sgp); // reloaded once its last token is done (see ov_kernel)
         };
-        rotate_over<PF>(nfull, body);
+        rotate_over<PFQ>(nfull, body);
 #pragma unroll
-        for (int p = 0; p < G::NP; p++) {
+        for (int p = 0; p < NPASS * G::NP; p++) {
             acc[2 * p] = acc4[p].x;
             acc[2 * p + 1] = acc4[p].y;
         }
 
         if (last) {
-            ft_load_beta(st, be, tg, h, c0);
             const int ntail = (t1 - t0) & 7;
-            if (ntail) {
-                uint32_t w[4];
-                vec_words(cb[(size_t)nfull * G::VPS], w);
-#pragma unroll
-                for (int pp = 0; pp < 2; pp++) {
-                    Pair &s = st[pp];
-                    for (int tt = 0; tt < ntail; tt++) {
-                        const h2 qc = extract_pair<4>(w[2 * pp], w[2 * pp + 1], tt);
-                        const h2 qs = qc * s.sc;
-                        const h2 vd = qs + s.zp;
-                        const float wt = (float)wb[nfull * 8 + tt];
-                        acc[2 * pp] = __builtin_fmaf(wt, (float)vd.x, acc[2 * pp]);
-                        acc[2 * pp + 1] = __builtin_fmaf(wt, (float)vd.y, acc[2 * pp + 1]);
-                        update_pair(s, qc, qs);
-                    }
-                }
-            }
-            if (active)
-                publish_state<D, CPL>(st, state_out, sa, bx, c0, T);
-            h2 deq[G::NP];
-            append_new_token<D, CPL>(cbh, T, v_new + (size_t)bx * D + c0, st, deq, active, sa.act_bf16);
             const float wT = (float)wrow[T];
 #pragma unroll
-            for (int p = 0; p < G::NP; p++) {
-                acc[2 * p] = __builtin_fmaf(wT, (float)deq[p].x, acc[2 * p]);
-                acc[2 * p + 1] = __builtin_fmaf(wT, (float)deq[p].y, acc[2 * p + 1]);
+            for (int ps = 0; ps < NPASS; ps++) {
+                Pair *sp = st + ps * G::NP;
+                float *ap = acc + ps * CPL;
+                ft_load_beta(sp, be, tg, h, c0 + 64 * ps);
+                if (ntail) {
+                    uint32_t w[4];
+                    vec_words(cb[(size_t)nfull * G::VPS + LPH * ps], w);
+#pragma unroll
+                    for (int pp = 0; pp < 2; pp++) {
+                        Pair &s = sp[pp];
+                        for (int tt = 0; tt < ntail; tt++) {
+                            const h2 qc = extract_pair<4>(w[2 * pp], w[2 * pp + 1], tt);
+                            const h2 qs = qc * s.sc;
+                            const h2 vd = qs + s.zp;
+                            const float wt = (float)wb[nfull * 8 + tt];
+                            ap[2 * pp] = __builtin_fmaf(wt, (float)vd.x, ap[2 * pp]);
+                            ap[2 * pp + 1] = __builtin_fmaf(wt, (float)vd.y, ap[2 * pp + 1]);
+                            update_pair(s, qc, qs);
+                        }
+                    }
+                }
+                if (active)
+                    publish_state<D, CPL>(sp, state_out, sa, bx, c0 + 64 * ps, T);
+                h2 deq[G::NP];
+                append_new_token<D, CPL>(cbh + LPH * ps, T, v_new + (size_t)bx * D + c0 + 64 * ps, sp, deq, active,
+                                         sa.act_bf16);
+#pragma unroll
+                for (int p = 0; p < G::NP; p++) {
+                    ap[2 * p] = __builtin_fmaf(wT, (float)deq[p].x, ap[2 * p]);
+                    ap[2 * p + 1] = __builtin_fmaf(wT, (float)deq[p].y, ap[2 * p + 1]);
+                }
             }
         }
         if (sa.combine) {
             // nseg is 2 or 4: the waves holding
             // the other segments of these sequences are 4, 8, 12 waves away (interleave_segment:
             // quad q takes segment q mod nseg).  The table is finished with once every wave is
-            // here; its first 16 KB take the partial sums, and the wave of segment 0 adds them in
-            // segment order (what ov_finalize_kernel does).
+            // here; its first 16 KB per pass take the partial sums, and the wave of segment 0 adds
+            // them in segment order (what ov_finalize_kernel does).
             __syncthreads();
             float4 *red = reinterpret_cast<float4 *>(tab);
             const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
-            red[wv * 64 + lane] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+#pragma unroll
+            for (int ps = 0; ps < NPASS; ps++)
+                red[(ps * FT_WAVES + wv) * 64 + lane] =
+                    make_float4(acc[4 * ps], acc[4 * ps + 1], acc[4 * ps + 2], acc[4 * ps + 3]);
             __syncthreads();
             if (un.seg != 0 || !active)
                 return;
-            for (int s = 1; s < sa.nseg; s++) {
-                const float4 p = red[(wv + 4 * s) * 64 + lane];
-                acc[0] += p.x;
-                acc[1] += p.y;
-                acc[2] += p.z;
-                acc[3] += p.w;
-            }
+            for (int s = 1; s < sa.nseg; s++)
+#pragma unroll
+                for (int ps = 0; ps < NPASS; ps++) {
+                    const float4 p = red[(ps * FT_WAVES + wv + 4 * s) * 64 + lane];
+                    acc[4 * ps] += p.x;
+                    acc[4 * ps + 1] += p.y;
+                    acc[4 * ps + 2] += p.z;
+                    acc[4 * ps + 3] += p.w;
+                }
         }
         if (!active)
             return;
-        if (sa.nseg == 1 || sa.combine) {
-            h1 *o = out + (size_t)bx * D + c0;
 #pragma unroll
-            for (int p = 0; p < G::NP; p++)
-                store_act2(o + 2 * p, acc[2 * p], acc[2 * p + 1], sa.act_bf16);
-        } else {
-            float2 *o = reinterpret_cast<float2 *>(partial + ((size_t)un.seg * BH + bx) * D + c0);
+        for (int ps = 0; ps < NPASS; ps++) {
+            if (sa.nseg == 1 || sa.combine) {
+                h1 *o = out + (size_t)bx * D + c0 + 64 * ps;
 #pragma unroll
-            for (int p = 0; p < G::NP; p++)
-                o[p] = make_float2(acc[2 * p], acc[2 * p + 1]);
+                for (int p = 0; p < G::NP; p++)
+                    store_act2(o + 2 * p, acc[4 * ps + 2 * p], acc[4 * ps + 2 * p + 1], sa.act_bf16);
+            } else {
+                float2 *o = reinterpret_cast<float2 *>(partial + ((size_t)un.seg * BH + bx) * D + c0 + 64 * ps);
+#pragma unroll
+                for (int p = 0; p < G::NP; p++)
+                    o[p] = make_float2(acc[4 * ps + 2 * p], acc[4 * ps + 2 * p + 1]);
+            }
         }
     }
 }

@@ -250,6 +250,46 @@ __device__ __forceinline__ int token_of_lane(int lane)
     return 4 * (bank >> 1) + 2 * (bank & 1) + row;
 }
 
+// The same for a head of 16 lanes (one row): after the two masked steps a lane holds two tokens'
+// sums over the four lanes that differ from it in bits 2 and 3; lanes with bit 1 clear keep the
+// first and take the partner's (lane ^ 2) first, the others the second, and bit 0 is an all-reduce.
+// Every PAIR of lanes ends with one token's total, token_of_lane16(lane).
+__device__ __forceinline__ float reduce8_head16(const float *p)
+{
+    float r0, r1, r2, r3, s0, s1, keep, give;
+    const unsigned long long odd_pairs = 0xCCCCCCCCCCCCCCCCull; // lanes with bit 1 set
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_add_f32_dpp %0, %8, %8 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %1, %9, %9 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %2, %10, %10 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %3, %11, %11 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %0, %12, %12 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %1, %13, %13 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %2, %14, %14 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %3, %15, %15 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %4, %0, %0 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %5, %1, %1 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %4, %2, %2 row_ror:4 row_mask:0xf bank_mask:0xa\n\t"
+        "v_add_f32_dpp %5, %3, %3 row_ror:4 row_mask:0xf bank_mask:0xa\n\t"
+        "v_cndmask_b32_e64 %6, %4, %5, %16\n\t"
+        "v_cndmask_b32_e64 %7, %5, %4, %16\n\t"
+        "s_nop 1\n\t"
+        "v_add_f32_dpp %6, %7, %6 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_add_f32_dpp %6, %6, %6 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 0"
+        : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3), "=&v"(s0), "=&v"(s1), "=&v"(keep), "=&v"(give)
+        : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7]), "s"(odd_pairs));
+    return keep;
+}
+
+__device__ __forceinline__ int token_of_lane16(int lane)
+{
+    const int bank = (lane >> 2) & 3;
+    return 4 * (bank >> 1) + 2 * (bank & 1) + ((lane >> 1) & 1);
+}
+
 // The same sum over a head of LPH lanes: a 64-lane head adds its two halves at the end (both then
 // hold every token's total).
 template <int LPH>
@@ -1760,7 +1800,7 @@ static int n_simd() { return 4 * cus(); }
 // per CU, so a launch is ceil(workgroups / 256) rounds of one segment's length each, and a batch
 // whose workgroup count falls just past a multiple of 256 (B = 352: 352 workgroups = 2 rounds for
 // 1.4 rounds of work) wastes most of a round unless it is cut finer.
-static Seg plan_segments(void *ckpt, int n_ckpt_cap, int ckpt_interval, int BH, int T, int D)
+static Seg plan_segments(void *ckpt, int n_ckpt_cap, int ckpt_interval, int BH, int T, int D, int lanes = 0)
 {
     Seg s;
     s.ckpt = (h1 *)ckpt;
@@ -1778,7 +1818,7 @@ static Seg plan_segments(void *ckpt, int n_ckpt_cap, int ckpt_interval, int BH, 
     if (!ckpt || ckpt_interval <= 0 || T <= ckpt_interval)
         return s;
     const int avail = (T + ckpt_interval - 1) / ckpt_interval;               // finest split
-    const int lph = lanes_per_head(D);
+    const int lph = lanes ? lanes : lanes_per_head(D); // lanes: 16 for the two-pass per-head-table kernels
     const long units_target = (long)n_simd() * WAVES_PER_SIMD_TARGET * (64 / lph);
     long want = (units_target + BH - 1) / BH;
     if (want < 1)
@@ -1791,7 +1831,7 @@ static Seg plan_segments(void *ckpt, int n_ckpt_cap, int ckpt_interval, int BH, 
     // launch length in units of one checkpoint interval
     auto cost = [&](int m) {
         const int nseg = (avail + m - 1) / m;
-        const long threads = (lph == 32 ? padded_units<32>(BH, nseg) : padded_units<64>(BH, nseg)) * lph;
+        const long threads = (lph == 16 ? padded_units<16>(BH, nseg) : lph == 32 ? padded_units<32>(BH, nseg) : padded_units<64>(BH, nseg)) * lph;
         if (D == 512 || threads < 1024L * cus())
             return (double)m;                        // small workgroups: no round structure to model
         const long wgs = (threads + 1023) / 1024;
@@ -1920,13 +1960,13 @@ static bool mfma_for_mha()
 // and otherwise spread 4-wave workgroups over the SIMDs, where the fullest SIMD sets the time
 // (its waves / 4 rounds).  Measured (B x 32 heads, ctx; per-head table against shared table):
 // 128 x 4096: 587 / 624 us per layer-step, 34 x 3000: 155 / 181, 40 x 1500: 89 / 107, 24 x 3000:
-// 141 / 141, 20 x 8192 (288 workgroups, two rounds): 369 / 255.  adkv_set_mha_kernel(2) takes them whenever they can run, (0) never.
+// 141 / 141, 20 x 8192 (288 workgroups, two rounds): 369 / 255.  adkv_set_mha_kernel(2) takes them whenever they can run (3: with 16 lanes per head, 4: with 32), (0) never.
 static bool use_head_table(int B, int H, int GQ, int bits, int D, const Seg &seg)
 {
     if (D != 128 || bits != 4 || GQ != 1)
         return false;
     const int v = g_mha_kernel.load(std::memory_order_relaxed);
-    if (v == 2)
+    if (v >= 2)
         return true;
     if (v >= 0 || mha_kernel_default() == 1)
         return false;
@@ -1935,7 +1975,7 @@ static bool use_head_table(int B, int H, int GQ, int bits, int D, const Seg &seg
     const long waves_shared = padded / 2;
     if (waves_shared <= n_simd())
         return false;                                 // every wave a SIMD to itself: two-channel lanes
-    const long wgs_ft = (long)H * ft_wgs_per_head(B, seg.nseg);
+    const long wgs_ft = (long)H * ft_wgs_per_head(B, seg.nseg, 2);
     const double t_ft = 0.93 * (double)((wgs_ft + cus() - 1) / cus());
     double t_shared;
     if (padded * 32 >= (long)FT_BLK * cus())
@@ -1977,20 +2017,21 @@ constexpr unsigned FT_SKEW_OV = 0; // 0: even segments.  forward_ov gains nothin
 // 318 with 6:6:3:1, 330 with 8:4:2:2); forward_ov 265 even, 252 with 6:5:3:2 / 6:6:3:1 / 8:5:2:1
 constexpr unsigned GQA_SKEW_QK = pack_skew(6, 5, 3, 2);
 constexpr unsigned GQA_SKEW_OV = pack_skew(6, 5, 3, 2);
+constexpr bool FT16_QK = true, FT16_OV = true; // whether forward_qk / forward_ov may take 16 lanes per head
 constexpr int FT_MIN_GROUP = 8;  // checkpoint intervals a group needs for its shares to differ
 constexpr int FT_MAX_GROUPS = 16;
 
-static void plan_head_table(Seg &seg, int B, int H, int T, unsigned skew)
+static void plan_head_table(Seg &seg, int B, int H, int T, unsigned skew, int upw)
 {
     seg.groups = 0;
     seg.skew = skew;
-    seg.phys_per_head = ft_wgs_per_head(B, seg.nseg);
+    seg.phys_per_head = ft_wgs_per_head(B, seg.nseg, upw);
     if (!seg.ckpt || seg.ckpt_interval <= 0 || skew == 0)
         return;
     const int iv = seg.ckpt_interval;
     const int avail = (T + iv - 1) / iv;
     // groups of four segments: as many as give every SIMD its four waves, FT_MIN_GROUP intervals or more each
-    const long waves_per_group = (long)H * 4 * pad4(ft_pairs_per_seg(B));
+    const long waves_per_group = (long)H * 4 * pad4(ft_waves_per_seg(B, upw));
     long G = ((long)n_simd() * WAVES_PER_SIMD_TARGET + waves_per_group - 1) / waves_per_group;
     if (G > avail / FT_MIN_GROUP)
         G = avail / FT_MIN_GROUP;
@@ -2006,7 +2047,7 @@ static void plan_head_table(Seg &seg, int B, int H, int T, unsigned skew)
     seg.nseg = (int)(4 * G);
     seg.seg_tokens = iv; // not read by the kernels of an uneven plan
     // workgroups per head: the fewest rounds of 256 workgroups times virtual workgroups each
-    const int W = ft_wgs_per_head(B, seg.nseg);
+    const int W = ft_wgs_per_head(B, seg.nseg, upw);
     int best = W;
     long best_cost = -1;
     for (int P = 1; P <= W; P++) {
@@ -2017,6 +2058,29 @@ static void plan_head_table(Seg &seg, int B, int H, int T, unsigned skew)
         }
     }
     seg.phys_per_head = best;
+}
+
+// Lanes per head of the per-head-table kernels for a launch, and its plan (`seg` comes in as the
+// launch's even plan for 32 lanes and goes out as the plan to run).  Sixteen lanes per head (four
+// sequences per wave, two passes over every supergroup) spend fewer instructions per channel, but
+// need twice the segments for the same number of waves: they are taken when their plan still
+// gives every SIMD its four waves, and 32 lanes otherwise.
+static int plan_ft(Seg &seg, int B, int H, int T, unsigned skew, bool sixteen_ok)
+{
+    const int forced = g_mha_kernel.load(std::memory_order_relaxed); // 3: sixteen lanes, 4: thirty-two
+    if (sixteen_ok && forced != 4) {
+        Seg s16 = plan_segments(seg.ckpt, seg.n_ckpt_cap, seg.ckpt_interval, B * H, T, 128, 16);
+        s16.row_pitch = seg.row_pitch;
+        s16.act_bf16 = seg.act_bf16;
+        plan_head_table(s16, B, H, T, skew, 4);
+        const long waves = (long)H * s16.nseg * pad4(ft_waves_per_seg(B, 4));
+        if (forced == 3 || waves >= (long)n_simd() * WAVES_PER_SIMD_TARGET) {
+            seg = s16;
+            return 16;
+        }
+    }
+    plan_head_table(seg, B, H, T, skew, 2);
+    return 32;
 }
 
 // The same uneven shares for the kernels without virtual workgroups (matrix-core and shared-table
@@ -2046,9 +2110,11 @@ static int max_plan_segments(void *ckpt, int n_ckpt_cap, int ckpt_interval, int 
     Seg seg = plan_segments(ckpt, n_ckpt_cap, ckpt_interval, B * H, T, D);
     int n = seg.nseg;
     if (D == 128) {
-        plan_head_table(seg, B, H, T, FT_SKEW_QK);
-        if (seg.nseg > n)
-            n = seg.nseg;
+        Seg a = seg, b = seg, c = seg;
+        plan_head_table(a, B, H, T, FT_SKEW_QK, 2);
+        plan_ft(b, B, H, T, FT_SKEW_QK, true);
+        plan_ft(c, B, H, T, FT_SKEW_OV, true);
+        n = std::max(std::max(n, a.nseg), std::max(b.nseg, c.nseg));
     }
     return n;
 }
@@ -2071,7 +2137,7 @@ int adkv_abi_version(void) { return 15; }
 
 void adkv_set_mha_kernel(int use_matrix_cores)
 {
-    g_mha_kernel.store(use_matrix_cores < 0 ? -1 : (use_matrix_cores > 2 ? 1 : use_matrix_cores),
+    g_mha_kernel.store(use_matrix_cores < 0 ? -1 : (use_matrix_cores > 4 ? 1 : use_matrix_cores),
                        std::memory_order_relaxed);
 }
 
@@ -2303,7 +2369,10 @@ static const char *decode_kernel_name(int B, int Hq, int H, int T, int D, int bi
     }
     if (use_head_table(B, H, GQ, bits, D, seg)) {
         Seg s2 = seg;
-        plan_head_table(s2, B, H, T, FT_SKEW_QK);
+        const int lanes = plan_ft(s2, B, H, T, FT_SKEW_QK, FT16_QK);
+        if (lanes == 16)
+            return s2.groups ? "ft_kernel (per-head table, 16 lanes per head, 16-wave workgroups, uneven segments)"
+                             : "ft_kernel (per-head table, 16 lanes per head, 16-wave workgroups)";
         return s2.groups ? "ft_kernel (per-head table, 16-wave workgroups, uneven segments)"
                          : "ft_kernel (per-head table, 16-wave workgroups)";
     }
@@ -2360,8 +2429,9 @@ static int forward_qk_impl(const void *q, void *k_cache, const void *k_new, void
         return check_launch();
     }
     if (use_head_table(B, H, GQ, bits, D, seg)) {
-        plan_head_table(seg, B, H, T, FT_SKEW_QK);
-        hipLaunchKernelGGL(qk_ft_kernel, dim3((unsigned)(H * seg.phys_per_head)), dim3(FT_BLK), 0, st,
+        const int lanes = plan_ft(seg, B, H, T, FT_SKEW_QK, FT16_QK);
+        const auto kernel = lanes == 16 ? qk_ft_kernel<16> : qk_ft_kernel<32>;
+        hipLaunchKernelGGL(kernel, dim3((unsigned)(H * seg.phys_per_head)), dim3(FT_BLK), 0, st,
                            (const h1 *)q, (uint4 *)k_cache, (const h1 *)k_new, (h1 *)logits,
                            (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha, (const h1 *)beta,
                            (const h1 *)tgt, B, H, T, n_super_cap, (h1 *)state_out, seg);
@@ -2400,8 +2470,8 @@ int adkv_decode_segments(int B, int Hq, int H, int T, int D, int bits, int n_ckp
     if (matrix_cores && GQ <= 4)
         plan_uneven(seg, T, padded_units<32>(B * H, seg.nseg) * 32, GQA_SKEW_QK);
     if (head_table) {
-        plan_head_table(seg, B, H, T, FT_SKEW_QK);
-        const int W = ft_wgs_per_head(B, seg.nseg);
+        const int lanes = plan_ft(seg, B, H, T, FT_SKEW_QK, FT16_QK);
+        const int W = ft_wgs_per_head(B, seg.nseg, 64 / lanes);
         wgs = (long)H * seg.phys_per_head;
         virt = (W + seg.phys_per_head - 1) / seg.phys_per_head;
     }
@@ -2495,13 +2565,12 @@ static int forward_ov_impl(const void *attn, void *v_cache, const void *v_new, v
         seg.row_pitch = ld;
     const bool matrix_cores = D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha());
     const bool head_table = !matrix_cores && use_head_table(B, H, GQ, bits, D, seg);
-    if (head_table)
-        plan_head_table(seg, B, H, T, FT_SKEW_OV);
+    const int ft_lanes = head_table ? plan_ft(seg, B, H, T, FT_SKEW_OV, FT16_OV) : 32;
     // per-head table, two or four segments, one virtual workgroup per workgroup: the waves of one
     // sequence pair sit in the same workgroup (interleave_segment) and add their partial outputs
     // there; no second launch and nothing in the workspace
     seg.combine = (head_table && (seg.nseg == 2 || seg.nseg == 4) &&
-                   seg.phys_per_head == ft_wgs_per_head(B, seg.nseg)) ? 1 : 0;
+                   seg.phys_per_head == ft_wgs_per_head(B, seg.nseg, 64 / ft_lanes)) ? 1 : 0;
     if (seg.nseg > 1 && !seg.combine) {
         if (!workspace || workspace_bytes < (int64_t)seg.nseg * BH * GQ * D * 4)
             return ADKV_E_WORKSPACE;
@@ -2516,7 +2585,8 @@ static int forward_ov_impl(const void *attn, void *v_cache, const void *v_new, v
                          (const h1 *)alpha, (const h1 *)beta, (const h1 *)tgt, BH, H, T, n_super_cap,
                          (h1 *)state_out, seg);
     } else if (head_table) {
-        hipLaunchKernelGGL(ov_ft_kernel, dim3((unsigned)(H * ft_wgs_per_head(B, seg.nseg))),
+        const auto kernel = ft_lanes == 16 ? ov_ft_kernel<16> : ov_ft_kernel<32>;
+        hipLaunchKernelGGL(kernel, dim3((unsigned)(H * ft_wgs_per_head(B, seg.nseg, 64 / ft_lanes))),
                            dim3(FT_BLK), 0, st, (const h1 *)attn, (uint4 *)v_cache, (const h1 *)v_new, (h1 *)out,
                            (float *)workspace, (const h1 *)zp, (const h1 *)sc, (const h1 *)alpha,
                            (const h1 *)beta, (const h1 *)tgt, B, H, T, n_super_cap, (h1 *)state_out, seg);
@@ -2613,8 +2683,8 @@ int adkv_forward_ov_noalloc(const void *attn, void *v_cache, const void *v_new, 
         const bool matrix_cores = D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha());
         bool in_workgroup = false;
         if (!matrix_cores && use_head_table(B, H, GQ, bits, D, seg)) {
-            plan_head_table(seg, B, H, T, FT_SKEW_OV);
-            in_workgroup = (seg.nseg == 2 || seg.nseg == 4) && seg.phys_per_head == ft_wgs_per_head(B, seg.nseg);
+            const int lanes = plan_ft(seg, B, H, T, FT_SKEW_OV, FT16_OV);
+            in_workgroup = (seg.nseg == 2 || seg.nseg == 4) && seg.phys_per_head == ft_wgs_per_head(B, seg.nseg, 64 / lanes);
         }
         if (seg.nseg > 1 && !in_workgroup)
             need = (int64_t)seg.nseg * B * Hq * D * 4;

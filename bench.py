@@ -32,8 +32,10 @@ N_LAYERS_MODEL = 32
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=40)
-    ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--steps", type=int, default=256,
+                    help="timed steps; the default covers eight model passes of 32 layer-steps")
+    ap.add_argument("--warmup", type=int, default=64,
+                    help="untimed steps first; the device clock settles over the first few dozen launches")
     ap.add_argument("--workload", choices=["decode", "encode", "quant_f32"], default="decode",
                     help="decode = headline decode attention (cfg2); encode = streaming quantiser (cfg3: "
                          "B=8 ctx=32768 prefill, then 256 single-token appends)")

@@ -38,7 +38,8 @@ int adkv_abi_version(void);
 /* Tuning knob, no counterpart in the reference: which decode kernels a launch with as many query
  * heads as KV heads and head dim 128 uses: 0 = the vector kernels with the shared code table,
  * 1 = the matrix-core kernels (the ones grouped-query launches always use), 2 = the vector
- * kernels with a per-head table wherever they can run (4-bit codes), -1 = the library's choice
+ * kernels with a per-head table wherever they can run (4-bit codes; 3 = the same, always with
+ * sixteen lanes per head, 4 = always with thirty-two), -1 = the library's choice
  * (the per-head table where its launch is the faster one, else the shared one; ADKV_MFMA=1 in the environment,
  * read once, makes it the matrix-core kernels).  Results agree to the tolerance of the fp32
  * accumulation order; appended codes, state and checkpoints are identical. */

@@ -550,18 +550,23 @@ def test_decode_step_replays_from_a_captured_graph(gpu, H, Hq, T, S, bits):
     (40, 32, 32, 300, 64, 4),    # enough units for four channels per lane
     (2, 2, 8, 530, 64, 4),       # matrix-core kernels, 4 query heads per KV head
     (1, 2, 16, 200, 32, 2),      # 2-bit codes, 8 query heads per KV head
-    (3, 2, -2, 530, 64, 4),      # the per-head-table kernels (forced), a few segments
-    (5, 3, -3, 257, 0, 4),       # the per-head-table kernels (forced), one segment
+    (3, 2, -2, 530, 64, 4),      # the per-head-table kernels (forced, 32 lanes per head), a few segments
+    (5, 3, -3, 257, 0, 4),       # the per-head-table kernels (forced, 32 lanes per head), one segment
+    (3, 2, -102, 530, 64, 4),    # the per-head-table kernels (forced, 16 lanes per head), a few segments
+    (5, 3, -103, 257, 0, 4),     # the per-head-table kernels (forced, 16 lanes per head), one segment
 ])
 def test_decode_step_takes_bfloat16_activations(gpu, B, H, Hq, T, S, bits):
     """q, k_new, v_new in bfloat16: the kernels round them to fp16 on the way in and the result to
     bfloat16 on the way out.  Everything equals the fp16 call on `.to(float16)` inputs followed by
     `.to(bfloat16)`: output bits, weights, appended codes, checkpoints.  (A negative Hq means
-    -Hq query heads with the per-head-table kernels forced.)"""
+    -Hq query heads with the per-head-table kernels forced, -100 - Hq those with 16 lanes per head.)"""
     from adkv_amd import _lib
-    if Hq < 0:
+    if Hq < -100:
+        Hq = -Hq - 100
+        _lib.lib().adkv_set_mha_kernel(3)
+    elif Hq < 0:
         Hq = -Hq
-        _lib.lib().adkv_set_mha_kernel(2)
+        _lib.lib().adkv_set_mha_kernel(4)
     try:
         _bf16_case(gpu, B, H, Hq, T, S, bits)
     finally:
@@ -803,22 +808,28 @@ def test_grouped_query_kernels_in_16_wave_workgroups(gpu, oracle, G, bits):
     (4, 2, 40, 32), (2, 2, 64, 32), (5, 3, 100, 32), (9, 2, 127, 32),  # two / four segments (ragged last one):
                                                                        # partial outputs added in the workgroup
 ])
-def test_per_head_table_kernels(gpu, oracle, B, H, T, S):
+@pytest.mark.parametrize("lanes", [32, 16])
+def test_per_head_table_kernels(gpu, oracle, B, H, T, S, lanes):
     """The decode kernels that keep a per-head (code, channel pair) -> (q, scale multiplier) table
     and reduce logits with masked DPP adds, forced for shapes far smaller than the ones that
-    take them by default: appended codes, replayed state and recorded checkpoints bit-exact,
-    logits and outputs within an fp16 ulp of the oracle's exact sums."""
+    take them by default, with a head over 32 lanes (two sequences per wave) and over 16 (four
+    sequences per wave, two passes per supergroup): appended codes, replayed state and recorded
+    checkpoints bit-exact, logits and outputs within an fp16 ulp of the oracle's exact sums."""
     from adkv_amd import _lib
-    _lib.lib().adkv_set_mha_kernel(2)
+    _lib.lib().adkv_set_mha_kernel(3 if lanes == 16 else 4)
     try:
         _gqa_case(gpu, oracle, B, H, 1, T, S, seed=5)
     finally:
         _lib.lib().adkv_set_mha_kernel(-1)
 
 
-@pytest.mark.parametrize("B,H,T,S", [(18, 64, 203, 8),     # two virtual workgroups per workgroup
-                                     (34, 64, 203, 8)])    # ten per head over four workgroups: 3, 3, 2, 2
-def test_virtual_workgroups_with_uneven_segments(gpu, oracle, B, H, T, S):
+@pytest.mark.parametrize("B,H,T,S,mode", [
+    (18, 64, 203, 8, 4),     # 32 lanes per head: two virtual workgroups per workgroup
+    (34, 64, 203, 8, 4),     # ten per head over four workgroups: 3, 3, 2, 2
+    (34, 64, 203, 8, 3),     # 16 lanes per head: six per head over three workgroups
+    (67, 64, 203, 8, 3),     # seventeen waves per segment, the last with three sequences
+])
+def test_virtual_workgroups_with_uneven_segments(gpu, oracle, B, H, T, S, mode):
     """The per-head-table kernels on a plan that only big launches get by themselves: segments of
     unequal length (the four wave slots of a SIMD get unequal shares), several virtual workgroups
     walked through by each launched workgroup, partial outputs through the workspace.  Forced on
@@ -856,7 +867,7 @@ def test_virtual_workgroups_with_uneven_segments(gpu, oracle, B, H, T, S):
         finally:
             L.adkv_set_mha_kernel(-1)
 
-    L.adkv_set_mha_kernel(2)
+    L.adkv_set_mha_kernel(mode)
     try:
         b = (ctypes.c_int * 80)()
         info = (ctypes.c_int * 2)()
@@ -868,7 +879,8 @@ def test_virtual_workgroups_with_uneven_segments(gpu, oracle, B, H, T, S):
     lens = [b[i + 1] - b[i] for i in range(n)]
     assert len(set(lens)) > 2, lens                                     # really uneven
 
-    got, want = run(2), run(0)
+    assert ("16 lanes" in name) == (mode == 3), name
+    got, want = run(mode), run(0)
     for a, w, what in zip(got[2:], want[2:], ("K cache", "V cache", "K checkpoints", "V checkpoints", "K state", "V state")):
         assert torch.equal(a.view(torch.uint8), w.view(torch.uint8)), what
     assert torch.equal(got[2], full) and torch.equal(got[3], full)
@@ -877,7 +889,7 @@ def test_virtual_workgroups_with_uneven_segments(gpu, oracle, B, H, T, S):
         d = torch.abs(a.float() - w.float())
         assert torch.all(d <= 2.0 ** -10 * torch.clamp(w.float().abs(), min=2.0 ** -4))
     pn = [_np16(t) for t in p.astuple()]
-    for (bb, h) in [(0, 0), (B - 1, H - 1), (B // 2, 17), (7, 40), (B - 2, 1)]:
+    for (bb, h) in [(0, 0), (B - 1, H - 1), (B // 2, 17), (7, 40), (B - 2, 1), (B - 3, 63)]:
         ph = [a[h:h + 1] for a in pn]
         sub = cache[bb:bb + 1, h:h + 1].cpu().numpy().copy()
         lw, _ = oracle.forward_qk_f16(_np16(q[bb:bb + 1, h:h + 1]), sub.copy(), _np16(xn[bb:bb + 1, h:h + 1]), *ph, T)
@@ -997,7 +1009,7 @@ def _fclass(a):
     return np.where(np.isnan(a), 3, np.where(np.isposinf(a), 1, np.where(np.isneginf(a), 2, 0)))
 
 
-@pytest.mark.parametrize("kernels", ["default", "per_head_table"])
+@pytest.mark.parametrize("kernels", ["default", "per_head_table", "per_head_table_16_lanes"])
 def test_non_finite_values_in_logits_and_outputs(gpu, oracle, kernels):
     """What the decode kernels return when the replayed state (and with it the dequantised values)
     turns infinite or NaN part of the way through the context.
@@ -1045,8 +1057,8 @@ def test_non_finite_values_in_logits_and_outputs(gpu, oracle, kernels):
 
     S = 64
     ck = None
-    if kernels == "per_head_table":
-        _lib.lib().adkv_set_mha_kernel(2)
+    if kernels != "default":
+        _lib.lib().adkv_set_mha_kernel(3 if kernels.endswith("16_lanes") else 4)
         ck = torch.zeros(B, H, T // S + 1, D, 2, dtype=torch.float16, device=gpu)
     try:
         cache = synth.alloc_cache(B, H, T + 8, D, gpu)

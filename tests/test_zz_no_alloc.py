@@ -135,13 +135,15 @@ def test_noalloc_call_is_capturable_in_a_graph(gpu):
             assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), (rep, name)
 
 
-def test_noalloc_accepts_launches_that_sum_their_segments_in_the_workgroup(gpu):
+@pytest.mark.parametrize("mode", [4, 3])
+def test_noalloc_accepts_launches_that_sum_their_segments_in_the_workgroup(gpu, mode):
     """The per-head-table kernel adds two or four segments inside its workgroups and touches no
     scratch: such a launch is never refused for its size.  Forced here on a small shape (the
-    kernels take it by themselves only for launches of hundreds of workgroups)."""
+    kernels take it by themselves only for launches of hundreds of workgroups), with a head over
+    32 lanes (mode 4) and over 16 (mode 3)."""
     L = _lib.lib()
     c = _case(gpu, B=4, H=2, G=1, T=40, S=32, bits=4, seed=8)           # two segments
-    L.adkv_set_mha_kernel(2)
+    L.adkv_set_mha_kernel(mode)
     try:
         got = _run(L, c, noalloc=True)
     finally:
