@@ -349,10 +349,9 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
 // A non-finite cached value makes both outputs of its channel PAIR non-finite (0 * inf inside the
 // product); the vector form of ov_kernel's two-channel lanes confines it to its own channel.
 //
-// One virtual workgroup per workgroup (forward_ov gains nothing from uneven segments, so its plan
-// never needs more).  sa.combine: the two or four segments of a sequence pair sit in the same
-// workgroup and are added there; otherwise every segment stores its fp32 partial sums for
-// ov_finalize_kernel.
+// One virtual workgroup per workgroup (forward_ov's plans never need more).  sa.combine: the two
+// or four segments of a wave's sequences sit in the same workgroup and are added there; otherwise
+// every segment stores its fp32 partial sums for ov_finalize_kernel.
 template <int LPH>
 __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
     const h1 *__restrict__ attn, uint4 *__restrict__ cache, const h1 *__restrict__ v_new,

@@ -2007,11 +2007,13 @@ static bool use_head_table(int B, int H, int GQ, int bits, int D, const Seg &seg
 // two virtual workgroups, 280-285 with shares 7:5:2:2 (8:4:2:2 and 6:6:3:1 within 3 us of that,
 // 9:4:2:1 302); forward_ov 261 with two even segments added inside the workgroup, 262-266 with the
 // best uneven shares (6:5:3:2, 7:5:2:2) plus the 4 us kernel that then adds the partial sums: no
-// gain, so forward_ov keeps its even plan.
+// gain, so forward_ov takes uneven shares only where one group of four segments fills the device and
+// the four are added inside the workgroup (plan_ft_ov): with 16 lanes per head at that shape, 259
+// even, 250 with 6:5:3:2 (8:4:2:2 251, 7:5:2:2 252, 6:4:3:3 and 5:5:3:3 257).
 // Shares of a SIMD's work given to its four wave slots, oldest first, in sixteenths of a group's
 // checkpoint intervals: measured on the headline shape, one setting per kernel.
 constexpr unsigned FT_SKEW_QK = pack_skew(7, 5, 2, 2);
-constexpr unsigned FT_SKEW_OV = 0; // 0: even segments.  forward_ov gains nothing from uneven ones (see plan_head_table)
+constexpr unsigned FT_SKEW_OV = pack_skew(6, 5, 3, 2);
 // matrix-core kernels in 16-wave workgroups, measured on B=16, 32 query heads over 8 KV heads, 131072
 // tokens of 2-bit codes (64 segments, us): forward_qk 320 even, 299 with 6:5:3:2 (305 with 7:5:2:2,
 // 318 with 6:6:3:1, 330 with 8:4:2:2); forward_ov 265 even, 252 with 6:5:3:2 / 6:6:3:1 / 8:5:2:1
@@ -2083,6 +2085,25 @@ static int plan_ft(Seg &seg, int B, int H, int T, unsigned skew, bool sixteen_ok
     return 32;
 }
 
+// forward_ov's plan: ov_ft_kernel runs one virtual workgroup per workgroup and adds two or four
+// segments of a sequence inside the workgroup; whatever else it leaves in the workspace costs a
+// second kernel.  Uneven shares are taken when the uneven plan is one group of four segments
+// whose waves share a workgroup, the even plan otherwise.
+static int plan_ft_ov(Seg &seg, int B, int H, int T)
+{
+    Seg un = seg;
+    const int lanes_un = plan_ft(un, B, H, T, FT_SKEW_OV, FT16_OV);
+    if (un.groups == 1 && un.phys_per_head == ft_wgs_per_head(B, un.nseg, 64 / lanes_un)) {
+        seg = un;
+        return lanes_un;
+    }
+    return plan_ft(seg, B, H, T, 0, FT16_OV);
+}
+static bool ft_ov_combines(const Seg &seg, int B, int lanes)
+{
+    return (seg.nseg == 2 || seg.nseg == 4) && seg.phys_per_head == ft_wgs_per_head(B, seg.nseg, 64 / lanes);
+}
+
 // The same uneven shares for the kernels without virtual workgroups (matrix-core and shared-table
 // kernels in 16-wave workgroups, where a workgroup's quads of waves are the four slots of its
 // SIMDs as well): the even plan's segments, when their number is a multiple of four, are re-cut
@@ -2113,7 +2134,7 @@ static int max_plan_segments(void *ckpt, int n_ckpt_cap, int ckpt_interval, int 
         Seg a = seg, b = seg, c = seg;
         plan_head_table(a, B, H, T, FT_SKEW_QK, 2);
         plan_ft(b, B, H, T, FT_SKEW_QK, true);
-        plan_ft(c, B, H, T, FT_SKEW_OV, true);
+        plan_ft_ov(c, B, H, T);
         n = std::max(std::max(n, a.nseg), std::max(b.nseg, c.nseg));
     }
     return n;
@@ -2565,12 +2586,11 @@ static int forward_ov_impl(const void *attn, void *v_cache, const void *v_new, v
         seg.row_pitch = ld;
     const bool matrix_cores = D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha());
     const bool head_table = !matrix_cores && use_head_table(B, H, GQ, bits, D, seg);
-    const int ft_lanes = head_table ? plan_ft(seg, B, H, T, FT_SKEW_OV, FT16_OV) : 32;
+    const int ft_lanes = head_table ? plan_ft_ov(seg, B, H, T) : 32;
     // per-head table, two or four segments, one virtual workgroup per workgroup: the waves of one
     // sequence pair sit in the same workgroup (interleave_segment) and add their partial outputs
     // there; no second launch and nothing in the workspace
-    seg.combine = (head_table && (seg.nseg == 2 || seg.nseg == 4) &&
-                   seg.phys_per_head == ft_wgs_per_head(B, seg.nseg, 64 / ft_lanes)) ? 1 : 0;
+    seg.combine = (head_table && ft_ov_combines(seg, B, ft_lanes)) ? 1 : 0;
     if (seg.nseg > 1 && !seg.combine) {
         if (!workspace || workspace_bytes < (int64_t)seg.nseg * BH * GQ * D * 4)
             return ADKV_E_WORKSPACE;
@@ -2683,8 +2703,8 @@ int adkv_forward_ov_noalloc(const void *attn, void *v_cache, const void *v_new, 
         const bool matrix_cores = D == 128 && (GQ > 1 || bits != 4 || mfma_for_mha());
         bool in_workgroup = false;
         if (!matrix_cores && use_head_table(B, H, GQ, bits, D, seg)) {
-            const int lanes = plan_ft(seg, B, H, T, FT_SKEW_OV, FT16_OV);
-            in_workgroup = (seg.nseg == 2 || seg.nseg == 4) && seg.phys_per_head == ft_wgs_per_head(B, seg.nseg, 64 / lanes);
+            const int lanes = plan_ft_ov(seg, B, H, T);
+            in_workgroup = ft_ov_combines(seg, B, lanes);
         }
         if (seg.nseg > 1 && !in_workgroup)
             need = (int64_t)seg.nseg * B * Hq * D * 4;
