@@ -527,7 +527,7 @@ def decode_record(args, B, Hq, H, D, T, bits, S, NL, steps, warmup, headline=Tru
                         "in that run; instruction count from profiles/valu_issue.json, duration live"}
             res["roofline"]["binding_roof"] = (
                 "vector-instruction issue (see roofline_valu): HBM is the nominal roof of this path, code bytes "
-                "against 8 TB/s, but a bit-exact fp16 replay needs 96 packed instructions per 8 tokens per wave, "
+                "against 8 TB/s, but a bit-exact fp16 replay needs six packed instructions per channel pair and token, "
                 "and the vector pipe is busy %.0f %% of the cycles at the clock the device sustains"
                 % (100 * vrec["valu_busy"]))
     except (OSError, ValueError):
