@@ -43,11 +43,29 @@ constexpr int TILE_ROW64 = 73;               // 8-byte words per token row: 2 he
 constexpr int TILE_WORDS64 = 8 * TILE_ROW64; // per wave
 __device__ __forceinline__ int tile_col(int lane_in_head) { return lane_in_head + 4 * (lane_in_head >> 4); }
 
-template <int CTRL>
-__device__ __forceinline__ float dpp_mov(float v)
+// d: a lane's partial logits of four tokens over its quarter of the channels, fresh from the matrix
+// cores; the other quarters are in the lanes that differ in bits 2 and 3 (qd).  Lane qd gets the
+// total of token qd, in six masked DPP adds: a masked add writes only the banks of its mask
+//   banks 0,1 | 2,3 (bit 3): keep tokens 0,1 | 2,3, add the partner's (rotate by 8)
+//   banks 0,2 | 1,3 (bit 2): keep the first | second of those, add lane+4's | lane-4's.
+// The leading wait states cover the matrix cores' write of d (up to five are required before a
+// vector instruction reads it), the inner ones a DPP operand written by the two instructions before.
+__device__ __forceinline__ float quarter_sum(f4v d)
 {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF,
-                                                                  0xF, false));
+    float s0, s1, r;
+    asm volatile(
+        "s_nop 7\n\t"
+        "v_add_f32_dpp %0, %3, %3 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %1, %4, %4 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %0, %5, %5 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %1, %6, %6 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "s_nop 1\n\t"
+        "v_add_f32_dpp %2, %0, %0 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %2, %1, %1 row_ror:4 row_mask:0xf bank_mask:0xa\n\t"
+        "s_nop 0"
+        : "=&v"(s0), "=&v"(s1), "=&v"(r)
+        : "v"(d.x), "v"(d.y), "v"(d.z), "v"(d.w));
+    return r;
 }
 
 
@@ -208,15 +226,7 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
             for (int m = 0; m < 8; m++)
                 d = __builtin_amdgcn_mfma_f32_4x4x4f16(as_h4(a[m].x, a[m].y), as_h4(qb[n][m].x, qb[n][m].y),
                                                        d, 0, 0, 0);
-            float s[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                float v = d[i];
-                v += dpp_mov<0x128>(v); // row_ror:8
-                v += dpp_mov<0x124>(v); // row_ror:4
-                s[i] = v;
-            }
-            const float mine = qd == 0 ? s[0] : qd == 1 ? s[1] : qd == 2 ? s[2] : s[3];
+            const float mine = quarter_sum(d);
             const int tok = tg4 * 4 + qd, g = 4 * n + r;
             if (active && g < GQ && tok < ntok)
                 out[((size_t)bx * GQ + g) * sa.row_pitch + t0 + unit * 8 + tok] = (h1)mine;
