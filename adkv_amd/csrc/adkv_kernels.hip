@@ -2064,9 +2064,15 @@ static void plan_head_table(Seg &seg, int B, int H, int T, unsigned skew, int up
 
 // Lanes per head of the per-head-table kernels for a launch, and its plan (`seg` comes in as the
 // launch's even plan for 32 lanes and goes out as the plan to run).  Sixteen lanes per head (four
-// sequences per wave, two passes over every supergroup) spend fewer instructions per channel, but
-// need twice the segments for the same number of waves: they are taken when their plan still
-// gives every SIMD its four waves, and 32 lanes otherwise.
+// sequences per wave, two passes over every supergroup) spend 5-7 % fewer instructions per channel
+// but need twice the segments for the same number of waves.  They are taken when their plan still
+// gives every SIMD its four waves AND cuts groups of at least FT16_MIN_GROUP checkpoint intervals
+// (so that the four shares keep their proportions and the shortest segment its length), and 32
+// lanes otherwise.  Measured, 32 heads, checkpoints every 256 tokens, layer-step with 32 / 16
+// lanes in us: B x ctx 128 x 4096 569 / 532, 256 x 4096 1091 / 1053, 16 x 32768 559 / 541 (groups
+// of 16 intervals); 64 x 4096 285 / 306, 128 x 2048 290 / 304, 32 x 8192 280 / 276, 96 x 4096
+// 465 / 450 (groups of 8); 128 x 1024 155 / 153 (even plan).
+constexpr int FT16_MIN_GROUP = 16;
 static int plan_ft(Seg &seg, int B, int H, int T, unsigned skew, bool sixteen_ok)
 {
     const int forced = g_mha_kernel.load(std::memory_order_relaxed); // 3: sixteen lanes, 4: thirty-two
@@ -2076,7 +2082,8 @@ static int plan_ft(Seg &seg, int B, int H, int T, unsigned skew, bool sixteen_ok
         s16.act_bf16 = seg.act_bf16;
         plan_head_table(s16, B, H, T, skew, 4);
         const long waves = (long)H * s16.nseg * pad4(ft_waves_per_seg(B, 4));
-        if (forced == 3 || waves >= (long)n_simd() * WAVES_PER_SIMD_TARGET) {
+        const bool long_groups = s16.groups > 0 && s16.intervals / s16.groups >= FT16_MIN_GROUP;
+        if (forced == 3 || (long_groups && waves >= (long)n_simd() * WAVES_PER_SIMD_TARGET)) {
             seg = s16;
             return 16;
         }

@@ -567,7 +567,7 @@ def secondary_records(args):
                 "roofline": r["roofline"]}
 
     def cfg5():
-        r = decode_record(args, 16, 32, 8, 128, 131072, 2, 256, 2, steps=6, warmup=2, headline=False, bf16=True)
+        r = decode_record(args, 16, 32, 8, 128, 131072, 2, 256, 2, steps=48, warmup=16, headline=False, bf16=True)
         # with 2-bit codes the replay costs what it costs with 4-bit ones on half the bytes: the roof
         # that binds is vector issue, and the record says so; the HBM figure is kept beside it
         out5 = {"workload": r["config"]["workload"], "ms_per_step": r["ms_per_step"], "tokens_per_s": r["value"],
