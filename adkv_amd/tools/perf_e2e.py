@@ -189,38 +189,49 @@ def sliced_run(args, model, cfg, source, device):
         "peak_mem_GiB": torch.cuda.max_memory_allocated() / 2 ** 30}))
 
 
-def main(argv=None):
-    args = parse_args(argv)
-    if args.search:
-        print(json.dumps(max_batch(args)))
-        return
-    device = torch.device("cuda:0")
+def generate_run(args, device=None) -> dict:
+    """One measurement by the protocol above (whole-batch prefill): builds the model, generates four
+    tokens untimed, then times ``num_repeats`` greedy ``generate`` calls.  Returns the record that
+    ``main`` prints."""
+    device = device or torch.device("cuda:0")
     model, cfg, source = build_model(args, device)
-    if args.prefill_slice > 0:
-        return sliced_run(args, model, cfg, source, device)
     g = torch.Generator().manual_seed(1)
     ids = torch.randint(1, cfg.vocab_size, (args.batch_size, args.prompt_lenth), generator=g).to(device)
     mask = torch.ones_like(ids)
     gen = dict(max_new_tokens=args.output_length, min_new_tokens=args.output_length, do_sample=False)
     stop = threading.Event()
     threading.Thread(target=_heartbeat, args=(stop,), daemon=True).start()
-    with torch.no_grad():
-        model.generate(ids, attention_mask=mask, max_new_tokens=4, min_new_tokens=4, do_sample=False)
-        torch.cuda.synchronize()
-        torch.cuda.reset_peak_memory_stats()
-        t0 = time.time()
-        for _ in range(args.num_repeats):
-            out = model.generate(ids, attention_mask=mask, **gen)
-        torch.cuda.synchronize()
-    stop.set()
+    try:
+        with torch.no_grad():
+            model.generate(ids, attention_mask=mask, max_new_tokens=4, min_new_tokens=4, do_sample=False)
+            torch.cuda.synchronize()
+            torch.cuda.reset_peak_memory_stats()
+            t0 = time.time()
+            for _ in range(args.num_repeats):
+                out = model.generate(ids, attention_mask=mask, **gen)
+            torch.cuda.synchronize()
+    finally:
+        stop.set()
     ms = (time.time() - t0) / args.num_repeats * 1e3
     assert out.shape[1] == args.prompt_lenth + args.output_length
-    print(json.dumps({
+    return {
         "model": args.model, "layers": cfg.num_hidden_layers, "kv": args.kv, "weights": "random init fp16",
         "adkv_params": source, "batch_size": args.batch_size, "prompt_length": args.prompt_lenth,
         "output_length": args.output_length, "used_time_ms": ms,
         "generated_tokens_per_s": args.batch_size * args.output_length / (ms * 1e-3),
-        "peak_mem_GiB": torch.cuda.max_memory_allocated() / 2 ** 30}))
+        "peak_mem_GiB": torch.cuda.max_memory_allocated() / 2 ** 30}
+
+
+def main(argv=None):
+    args = parse_args(argv)
+    if args.search:
+        print(json.dumps(max_batch(args)))
+        return
+    if args.prefill_slice > 0:
+        device = torch.device("cuda:0")
+        model, cfg, source = build_model(args, device)
+        return sliced_run(args, model, cfg, source, device)
+    print(json.dumps(generate_run(args)))
 
 
 if __name__ == "__main__":

@@ -61,6 +61,8 @@ def parse():
                     help="decode workload: q, the new token and the output in bfloat16")
     ap.add_argument("--no-secondary", action="store_true",
                     help="default decode run only: skip the short cfg3 / cfg5 / cfg1 runs reported under `secondary`")
+    ap.add_argument("--no-e2e", action="store_true",
+                    help="leave the end-to-end generate record (cfg4, about half a minute) out of `secondary`")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fp16-comparator", action="store_true",
                     help="skip timing the fp16-KV decode kernel beside the ADKV step")
@@ -544,10 +546,10 @@ def decode_record(args, B, Hq, H, D, T, bits, S, NL, steps, warmup, headline=Tru
 
 def secondary_records(args):
     """Short runs of the other named workloads in the same process, so that one default run shows
-    them all: the streaming quantiser (cfg3), the long-context grouped-query 2-bit decode (cfg5) and
-    the fp32 recurrence (cfg1).  Each record is what `--workload ...` prints with fewer steps and
-    without the host baselines; a failure in one is reported in its place and does not touch the
-    headline."""
+    them all: the streaming quantiser (cfg3), the long-context grouped-query 2-bit decode (cfg5), the
+    fp32 recurrence (cfg1) and the end-to-end generate of cfg4.  The first three are what
+    `--workload ...` prints with fewer steps and without the host baselines; a failure in one is
+    reported in its place and does not touch the headline."""
     import torch
     out = {}
 
@@ -585,9 +587,27 @@ def secondary_records(args):
                 "bit_exact_vs_oracle": r["bit_exact_vs_oracle"], "roofline": r["roofline"],
                 "cpu_baseline": r["cpu_baseline"]}
 
+    def cfg4():
+        # the reference's tools/perf_e2e.py protocol on the configuration's shape: random-init
+        # Llama-2-7B geometry in fp16, batch 128, 512 random prompt ids, 256 greedy tokens through
+        # transformers' generate with the ADKV cache (one timed repeat after a 4-token warm-up); the
+        # largest batch at ctx 4096 by the reference's memory accounting beside it
+        from adkv_amd.tools import perf_e2e
+        a = perf_e2e.parse_args(["--kv", "adkv", "--batch_size", "128", "--prompt_lenth", "512",
+                                 "--output_length", "256", "--num_repeats", "1"])
+        r = perf_e2e.generate_run(a)
+        m = perf_e2e.max_batch(perf_e2e.parse_args(["--prompt_lenth", "3840", "--output_length", "256"]))
+        return {"workload": "end-to-end greedy generate, random-init Llama-2-7B geometry (32 layers, fp16 weights), "
+                            "B=128, 512-token prompt, 256 new tokens, ADKV 4-bit cache",
+                "generated_tokens_per_s": r["generated_tokens_per_s"], "seconds_per_generate": r["used_time_ms"] / 1e3,
+                "peak_mem_GiB": r["peak_mem_GiB"], "adkv_params": r["adkv_params"],
+                "max_batch_ctx4096_by_memory_model": {"adkv": m["max_batch_adkv"], "fp16": m["max_batch_fp16"]}}
+
     run("cfg3_streaming_quantiser", cfg3)
     run("cfg5_long_context_gqa_2bit", cfg5)
     run("cfg1_fp32_recurrence", cfg1)
+    if not args.no_e2e:
+        run("cfg4_end_to_end_generate", cfg4)
     return out
 
 
