@@ -2062,47 +2062,68 @@ static void plan_head_table(Seg &seg, int B, int H, int T, unsigned skew, int up
     seg.phys_per_head = best;
 }
 
+// Length of a launch under a per-head-table plan, in tokens of a 32-lane wave's work: rounds of
+// workgroups on the CUs x virtual workgroups walked through by each x the longest segment (the
+// oldest wave slot's), x 1.86 for a head over 16 lanes (eight channels per lane at 0.93 of the
+// instructions per channel).
+static double ft_plan_cost(const Seg &s, int B, int H, int T, int upw)
+{
+    const int W = ft_wgs_per_head(B, s.nseg, upw);
+    const int P = s.phys_per_head > 0 ? s.phys_per_head : W;
+    const long rounds = ((long)H * P + cus() - 1) / cus();
+    const int virt = (W + P - 1) / P;
+    const int longest = s.groups ? seg_end(s, 0) - seg_begin(s, 0) : (s.seg_tokens < T ? s.seg_tokens : T);
+    return (double)rounds * virt * longest * (upw == 4 ? 1.86 : 1.0);
+}
+
 // Lanes per head of the per-head-table kernels for a launch, and its plan (`seg` comes in as the
 // launch's even plan for 32 lanes and goes out as the plan to run).  Sixteen lanes per head (four
 // sequences per wave, two passes over every supergroup) spend 5-7 % fewer instructions per channel
-// but need twice the segments for the same number of waves.  They are taken when their plan still
-// gives every SIMD its four waves AND cuts groups of at least FT16_MIN_GROUP checkpoint intervals
-// (so that the four shares keep their proportions and the shortest segment its length), and 32
-// lanes otherwise.  Measured, 32 heads, checkpoints every 256 tokens, layer-step with 32 / 16
-// lanes in us: B x ctx 128 x 4096 569 / 532, 256 x 4096 1091 / 1053, 16 x 32768 559 / 541 (groups
-// of 16 intervals); 64 x 4096 285 / 306, 128 x 2048 290 / 304, 32 x 8192 280 / 276, 96 x 4096
-// 465 / 450 (groups of 8); 128 x 1024 155 / 153 (even plan).
+// but need twice the segments for the same number of waves.  They are taken when their plan is
+// uneven with groups of at least FT16_MIN_GROUP checkpoint intervals (so that the four shares keep
+// their proportions and the shortest segment its length) and shorter than the 32-lane plan by
+// ft_plan_cost; 32 lanes otherwise.  Measured, 32 heads, checkpoints every 256 tokens, layer-step
+// with 32 / 16 lanes in us: B x ctx 128 x 4096 569 / 532, 256 x 4096 1091 / 1053, 16 x 32768
+// 559 / 541, 24 x 16384 540 / 479 (groups of 16 intervals or more, shorter by the model); 8 x 65536
+// 569 / 714 (longer by the model: half of the waves would be padding); 64 x 4096 285 / 306,
+// 128 x 2048 290 / 304, 32 x 8192 280 / 276, 96 x 4096 465 / 450 (groups of 8); 128 x 1024
+// 155 / 153, 128 x 640 106 / 131 (even plans).
 constexpr int FT16_MIN_GROUP = 16;
 static int plan_ft(Seg &seg, int B, int H, int T, unsigned skew, bool sixteen_ok)
 {
     const int forced = g_mha_kernel.load(std::memory_order_relaxed); // 3: sixteen lanes, 4: thirty-two
+    Seg s32 = seg;
+    plan_head_table(s32, B, H, T, skew, 2);
     if (sixteen_ok && forced != 4) {
         Seg s16 = plan_segments(seg.ckpt, seg.n_ckpt_cap, seg.ckpt_interval, B * H, T, 128, 16);
         s16.row_pitch = seg.row_pitch;
         s16.act_bf16 = seg.act_bf16;
         plan_head_table(s16, B, H, T, skew, 4);
-        const long waves = (long)H * s16.nseg * pad4(ft_waves_per_seg(B, 4));
         const bool long_groups = s16.groups > 0 && s16.intervals / s16.groups >= FT16_MIN_GROUP;
-        if (forced == 3 || (long_groups && waves >= (long)n_simd() * WAVES_PER_SIMD_TARGET)) {
+        if (forced == 3 ||
+            (long_groups && ft_plan_cost(s16, B, H, T, 4) < 0.97 * ft_plan_cost(s32, B, H, T, 2))) {
             seg = s16;
             return 16;
         }
     }
-    plan_head_table(seg, B, H, T, skew, 2);
+    seg = s32;
     return 32;
 }
 
 // forward_ov's plan: ov_ft_kernel runs one virtual workgroup per workgroup and adds two or four
 // segments of a sequence inside the workgroup; whatever else it leaves in the workspace costs a
-// second kernel.  Uneven shares are taken when the uneven plan is one group of four segments
-// whose waves share a workgroup, the even plan otherwise.
+// second kernel of some 5 us.  Uneven shares pay with a head over 16 lanes (measured at 16-lane
+// shapes: 128 x 4096 266 -> 249 us added in the workgroup; 16 x 32768, 64 x 8192, 32 x 16384
+// 262 -> 242 us through the workspace) and not with a head over 32 (64 x 4096: 127.5 either way;
+// 8 x 65536: 250 even, 258 uneven): they are taken when the uneven plan has 16 lanes per head and
+// needs no virtual workgroups, the even plan for 32 lanes otherwise.
 static int plan_ft_ov(Seg &seg, int B, int H, int T)
 {
     Seg un = seg;
     const int lanes_un = plan_ft(un, B, H, T, FT_SKEW_OV, FT16_OV);
-    if (un.groups == 1 && un.phys_per_head == ft_wgs_per_head(B, un.nseg, 64 / lanes_un)) {
+    if (lanes_un == 16 && un.groups >= 1 && un.phys_per_head == ft_wgs_per_head(B, un.nseg, 4)) {
         seg = un;
-        return lanes_un;
+        return 16;
     }
     return plan_ft(seg, B, H, T, 0, FT16_OV);
 }
