@@ -807,6 +807,9 @@ def test_grouped_query_kernels_in_16_wave_workgroups(gpu, oracle, G, bits):
     (40, 2, 300, 0),                                                   # no checkpoints, 20 waves per head
     (4, 2, 40, 32), (2, 2, 64, 32), (5, 3, 100, 32), (9, 2, 127, 32),  # two / four segments (ragged last one):
                                                                        # partial outputs added in the workgroup
+    (4, 8, 300, 8),                                                    # four groups of four uneven segments in one
+                                                                       # round of workgroups: with 16 lanes forward_ov
+                                                                       # takes them too, through the workspace
 ])
 @pytest.mark.parametrize("lanes", [32, 16])
 def test_per_head_table_kernels(gpu, oracle, B, H, T, S, lanes):
