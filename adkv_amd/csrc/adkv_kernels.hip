@@ -2023,7 +2023,31 @@ constexpr bool FT16_QK = true, FT16_OV = true; // whether forward_qk / forward_o
 constexpr int FT_MIN_GROUP = 8;  // checkpoint intervals a group needs for its shares to differ
 constexpr int FT_MAX_GROUPS = 16;
 
-static void plan_head_table(Seg &seg, int B, int H, int T, unsigned skew, int upw)
+// Longest segment of an uneven cut, in checkpoint intervals (the oldest wave slot's of the group
+// that got the most intervals).
+static int uneven_longest(int groups, int intervals, unsigned skew)
+{
+    int longest = 0;
+    for (int g = 0; g < groups; g++) {
+        const int n = uneven_cut(4 * g + 1, groups, intervals, skew) - uneven_cut(4 * g, groups, intervals, skew);
+        if (n > longest)
+            longest = n;
+    }
+    return longest;
+}
+
+// What a unit (one wave's segment) costs besides its tokens, in tokens: parameters, checkpoint,
+// the first loads' latency, the first lookups, the last reduction.
+constexpr int FT_UNIT_OVERHEAD_TOKENS = 32;
+
+// Groups and workgroups per head are chosen together, for the shortest launch by the model
+//   rounds of workgroups on the CUs x virtual workgroups walked through by each x longest segment.
+// (Groups by occupancy alone, then workgroups, left awkward batches on two thirds of the CUs:
+// 40 sequences x 32 heads x 8192 tokens took two groups and 160 workgroups of two virtual ones
+// where three groups fill 256.)  Ties go to fewer groups, then fewer workgroups.  virtual_ok =
+// false (forward_ov, whose kernel runs one virtual workgroup per workgroup) only considers plans
+// with as many workgroups as virtual ones.
+static void plan_head_table(Seg &seg, int B, int H, int T, unsigned skew, int upw, bool virtual_ok = true)
 {
     seg.groups = 0;
     seg.skew = skew;
@@ -2032,34 +2056,33 @@ static void plan_head_table(Seg &seg, int B, int H, int T, unsigned skew, int up
         return;
     const int iv = seg.ckpt_interval;
     const int avail = (T + iv - 1) / iv;
-    // groups of four segments: as many as give every SIMD its four waves, FT_MIN_GROUP intervals or more each
-    const long waves_per_group = (long)H * 4 * pad4(ft_waves_per_seg(B, upw));
-    long G = ((long)n_simd() * WAVES_PER_SIMD_TARGET + waves_per_group - 1) / waves_per_group;
-    if (G > avail / FT_MIN_GROUP)
-        G = avail / FT_MIN_GROUP;
-    if (G > FT_MAX_GROUPS)
-        G = FT_MAX_GROUPS;
-    if (G < 1)
-        return;
-    // segment s > 0 starts from checkpoint cut(s) - 1
-    if (uneven_cut((int)(4 * G - 1), (int)G, avail, skew) - 1 >= seg.n_ckpt_cap)
-        return;
-    seg.groups = (int)G;
-    seg.intervals = avail;
-    seg.nseg = (int)(4 * G);
-    seg.seg_tokens = iv; // not read by the kernels of an uneven plan
-    // workgroups per head: the fewest rounds of 256 workgroups times virtual workgroups each
-    const int W = ft_wgs_per_head(B, seg.nseg, upw);
-    int best = W;
-    long best_cost = -1;
-    for (int P = 1; P <= W; P++) {
-        const long cost = (((long)H * P + cus() - 1) / cus()) * ((W + P - 1) / P);
-        if (best_cost < 0 || cost < best_cost) {
-            best = P;
-            best_cost = cost;
+    int gmax = avail / FT_MIN_GROUP; // FT_MIN_GROUP intervals or more per group
+    if (gmax > FT_MAX_GROUPS)
+        gmax = FT_MAX_GROUPS;
+    int best_g = 0, best_p = 0;
+    double best_cost = -1.0;
+    for (int G = 1; G <= gmax; G++) {
+        // segment s > 0 starts from checkpoint cut(s) - 1
+        if (uneven_cut(4 * G - 1, G, avail, skew) - 1 >= seg.n_ckpt_cap)
+            continue;
+        const int W = ft_wgs_per_head(B, 4 * G, upw);
+        const double unit = (double)uneven_longest(G, avail, skew) * iv + FT_UNIT_OVERHEAD_TOKENS;
+        for (int P = virtual_ok ? 1 : W; P <= W; P++) {
+            const double cost = (double)(((long)H * P + cus() - 1) / cus()) * ((W + P - 1) / P) * unit;
+            if (best_cost < 0.0 || cost < 0.999 * best_cost) {
+                best_g = G;
+                best_p = P;
+                best_cost = cost;
+            }
         }
     }
-    seg.phys_per_head = best;
+    if (best_g == 0)
+        return;
+    seg.groups = best_g;
+    seg.intervals = avail;
+    seg.nseg = 4 * best_g;
+    seg.seg_tokens = iv; // not read by the kernels of an uneven plan
+    seg.phys_per_head = best_p;
 }
 
 // Length of a launch under a per-head-table plan, in tokens of a 32-lane wave's work: rounds of
@@ -2072,8 +2095,9 @@ static double ft_plan_cost(const Seg &s, int B, int H, int T, int upw)
     const int P = s.phys_per_head > 0 ? s.phys_per_head : W;
     const long rounds = ((long)H * P + cus() - 1) / cus();
     const int virt = (W + P - 1) / P;
-    const int longest = s.groups ? seg_end(s, 0) - seg_begin(s, 0) : (s.seg_tokens < T ? s.seg_tokens : T);
-    return (double)rounds * virt * longest * (upw == 4 ? 1.86 : 1.0);
+    const int longest = s.groups ? uneven_longest(s.groups, s.intervals, s.skew) * s.ckpt_interval
+                                 : (s.seg_tokens < T ? s.seg_tokens : T);
+    return (double)rounds * virt * (longest + FT_UNIT_OVERHEAD_TOKENS) * (upw == 4 ? 1.86 : 1.0);
 }
 
 // Lanes per head of the per-head-table kernels for a launch, and its plan (`seg` comes in as the
@@ -2089,16 +2113,16 @@ static double ft_plan_cost(const Seg &s, int B, int H, int T, int upw)
 // 128 x 2048 290 / 304, 32 x 8192 280 / 276, 96 x 4096 465 / 450 (groups of 8); 128 x 1024
 // 155 / 153, 128 x 640 106 / 131 (even plans).
 constexpr int FT16_MIN_GROUP = 16;
-static int plan_ft(Seg &seg, int B, int H, int T, unsigned skew, bool sixteen_ok)
+static int plan_ft(Seg &seg, int B, int H, int T, unsigned skew, bool sixteen_ok, bool virtual_ok = true)
 {
     const int forced = g_mha_kernel.load(std::memory_order_relaxed); // 3: sixteen lanes, 4: thirty-two
     Seg s32 = seg;
-    plan_head_table(s32, B, H, T, skew, 2);
+    plan_head_table(s32, B, H, T, skew, 2, virtual_ok);
     if (sixteen_ok && forced != 4) {
         Seg s16 = plan_segments(seg.ckpt, seg.n_ckpt_cap, seg.ckpt_interval, B * H, T, 128, 16);
         s16.row_pitch = seg.row_pitch;
         s16.act_bf16 = seg.act_bf16;
-        plan_head_table(s16, B, H, T, skew, 4);
+        plan_head_table(s16, B, H, T, skew, 4, virtual_ok);
         const bool long_groups = s16.groups > 0 && s16.intervals / s16.groups >= FT16_MIN_GROUP;
         if (forced == 3 ||
             (long_groups && ft_plan_cost(s16, B, H, T, 4) < 0.97 * ft_plan_cost(s32, B, H, T, 2))) {
@@ -2120,7 +2144,7 @@ static int plan_ft(Seg &seg, int B, int H, int T, unsigned skew, bool sixteen_ok
 static int plan_ft_ov(Seg &seg, int B, int H, int T)
 {
     Seg un = seg;
-    const int lanes_un = plan_ft(un, B, H, T, FT_SKEW_OV, FT16_OV);
+    const int lanes_un = plan_ft(un, B, H, T, FT_SKEW_OV, FT16_OV, false);
     if (lanes_un == 16 && un.groups >= 1 && un.phys_per_head == ft_wgs_per_head(B, un.nseg, 4)) {
         seg = un;
         return 16;

@@ -118,12 +118,16 @@ def test_segment_plans_cut_at_checkpoints_and_cover_the_context():
         assert b"16 lanes" not in L.adkv_decode_kernel_name(128, 32, 32, 4096, 128, 4, 17, 256)
     finally:
         L.adkv_set_mha_kernel(-1)
-    # lane width follows a model of the two plans: 24 sequences over 16384 tokens are shorter with 16 lanes (the
-    # 32-lane plan needs two virtual workgroups), 8 sequences over 65536 with 32 (half of the 16-lane waves would
-    # be padding), and groups of fewer than 16 checkpoint intervals keep 32 lanes
-    assert b"16 lanes per head" in L.adkv_decode_kernel_name(24, 32, 32, 16384, 128, 4, 65, 256)
+    # lane width follows a model of the two plans (rounds x virtual workgroups x longest segment): 100 sequences
+    # fill 224 workgroups once with 16 lanes and twice with 32; 8 sequences over 65536 tokens would leave half of
+    # the 16-lane waves as padding; groups of fewer than 16 checkpoint intervals keep 32 lanes
+    assert b"16 lanes per head" in L.adkv_decode_kernel_name(100, 32, 32, 4096, 128, 4, 17, 256)
     assert b"16 lanes" not in L.adkv_decode_kernel_name(8, 32, 32, 65536, 128, 4, 257, 256)
     assert b"16 lanes" not in L.adkv_decode_kernel_name(64, 32, 32, 4096, 128, 4, 17, 256)
+    # groups and workgroups are chosen together: 40 sequences over 8192 tokens take three groups in 256
+    # workgroups of two virtual ones (two groups by occupancy alone would fill 160)
+    n = L.adkv_decode_segments(40, 32, 32, 8192, 128, 4, 33, 256, b, 600, info)
+    assert n == 12 and list(info) == [256, 2]
     # a batch too small for that keeps 32 lanes per head unless told otherwise
     assert b"16 lanes" not in L.adkv_decode_kernel_name(34, 32, 32, 3000, 128, 4, 47, 64)
     L.adkv_set_mha_kernel(3)

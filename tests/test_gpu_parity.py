@@ -827,10 +827,10 @@ def test_per_head_table_kernels(gpu, oracle, B, H, T, S, lanes):
 
 
 @pytest.mark.parametrize("B,H,T,S,mode", [
-    (18, 64, 203, 8, 4),     # 32 lanes per head: two virtual workgroups per workgroup
-    (34, 64, 203, 8, 4),     # ten per head over four workgroups: 3, 3, 2, 2
-    (34, 64, 203, 8, 3),     # 16 lanes per head: six per head over three workgroups
-    (67, 64, 203, 8, 3),     # seventeen waves per segment, the last with three sequences
+    (34, 64, 203, 8, 4),     # 32 lanes per head: two groups, 256 workgroups of three virtual ones
+    (50, 64, 203, 8, 4),     # one group, two virtual workgroups per workgroup
+    (67, 64, 203, 8, 3),     # 16 lanes per head: two groups, three virtual workgroups, a wave with three sequences
+    (100, 64, 203, 8, 3),    # one group, two virtual workgroups per workgroup
 ])
 def test_virtual_workgroups_with_uneven_segments(gpu, oracle, B, H, T, S, mode):
     """The per-head-table kernels on a plan that only big launches get by themselves: segments of
