@@ -2107,11 +2107,11 @@ static double ft_plan_cost(const Seg &s, int B, int H, int T, int upw)
 // uneven with groups of at least FT16_MIN_GROUP checkpoint intervals (so that the four shares keep
 // their proportions and the shortest segment its length) and shorter than the 32-lane plan by
 // ft_plan_cost; 32 lanes otherwise.  Measured, 32 heads, checkpoints every 256 tokens, layer-step
-// with 32 / 16 lanes in us: B x ctx 128 x 4096 569 / 532, 256 x 4096 1091 / 1053, 16 x 32768
-// 559 / 541, 24 x 16384 540 / 479 (groups of 16 intervals or more, shorter by the model); 8 x 65536
-// 569 / 714 (longer by the model: half of the waves would be padding); 64 x 4096 285 / 306,
-// 128 x 2048 290 / 304, 32 x 8192 280 / 276, 96 x 4096 465 / 450 (groups of 8); 128 x 1024
-// 155 / 153, 128 x 640 106 / 131 (even plans).
+// with 32 / 16 lanes in us (each with the plan the model picks for it): B x ctx 128 x 4096
+// 581 / 552, 100 x 4096 528 / 475, 200 x 4096 1014 / 948, 352 x 4096 1667 / 1563, 16 x 32768
+// 570 / 537 (16 lanes shorter by the model); 24 x 16384 463 / 495, 40 x 8192 406 / 473, 96 x 4096
+// 466 / 481, 8 x 65536 569 / 714 (32 lanes shorter: the 16-lane plans leave padding waves or CUs
+// idle); 64 x 4096 303 / 304, 128 x 2048 290 / 304 (groups of 8); 128 x 640 106 / 131 (even plans).
 constexpr int FT16_MIN_GROUP = 16;
 static int plan_ft(Seg &seg, int B, int H, int T, unsigned skew, bool sixteen_ok, bool virtual_ok = true)
 {
