@@ -9,16 +9,23 @@
 // which removes one of the six packed instructions per pair and token.
 //
 //   * 256 code bytes x 64 channel pairs x 8 bytes = 128 KB of the CU's 160 KB of LDS, as two
-//     64 KB tables (first / second pair of a lane); entry (b, lane) sits at b*256 + lane*8, so the
-//     32 lanes of a head read 32 distinct 8-byte slots of one 256-byte row whatever their codes
-//     are, and the address is still ONE v_perm_b32: [0, table, code byte, lane*8].
-//   * All 32 (sequence, segment) units of a workgroup must belong to the SAME head: units are
-//     ordered head-major (for one head: a wave per pair of sequences and segment, consecutive
-//     quads of waves on different segments, interleave_segment), and every head's run of waves is padded
-//     to whole 16-wave workgroups.
+//     64 KB tables; with a head over 32 lanes (four channels per lane) entry (pair j, byte b, lane)
+//     sits at j*64 KB + b*256 + lane*8, so the 32 lanes of a head read 32 distinct 8-byte slots of
+//     one 256-byte row whatever their codes are, and the address is still ONE v_perm_b32:
+//     [0, table, code byte, lane*8].
+//   * A head over 16 lanes (eight channels per lane, two passes of four over every supergroup,
+//     four sequences per wave) pays the logit reduction, the store and the loop overhead once per
+//     eight channels: 7 % fewer instructions in forward_qk, 4 % in forward_ov.  Its table is
+//     [pass][byte][pair j][lane]: the 16 lanes of a head on the 16 slots of one half row.  The
+//     launchers take it for big launches whose segments stay long (plan_ft).
+//   * All units of a workgroup must belong to the SAME head: units are ordered head-major (for one
+//     head: a wave per two or four sequences and segment, consecutive quads of waves on different
+//     segments, interleave_segment), and every head's run of waves is padded to whole 16-wave
+//     workgroups.
 //   * No LDS is left for the logit transpose of qk_kernel, and none is needed: the 8 per-lane
-//     partials are reduced and scattered over the head's 32 lanes with bank-masked DPP adds
-//     (8 + 4 instructions), one row swap and two quad permutes.
+//     partials are reduced and scattered over the head's lanes with bank-masked DPP adds (8 + 4
+//     instructions), then one row swap and two quad permutes (32 lanes) or two selects and two
+//     quad permutes (16 lanes).
 #pragma once
 
 namespace adkv {
