@@ -127,7 +127,7 @@ __device__ __forceinline__ void ft_init_pairs(Pair *st, const h1 *zp, const h1 *
         st[p].sc = *reinterpret_cast<const h2 *>(sc + pi);
         st[p].al = *reinterpret_cast<const h2 *>(al + pi);
     }
-    if (seg > 0) {
+    if (seg_begin(sa, seg) > 0) {
         const int j = seg_begin(sa, seg) / sa.ckpt_interval - 1;
         load_state<4>(sa.ckpt + (((size_t)bx * sa.n_ckpt_cap + j) * 128 + c0) * 2, st);
     }
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
         const uint32_t lane_copy = ft_lane_copy<LPH>(un.lh);
         const int bx = un.bx, lh = un.lh, c0 = un.c0;
         const bool active = un.active;
-        const bool last = un.seg == sa.nseg - 1;
+        const bool last = seg_is_last(sa, un.seg);
 
         Pair st[NPASS * G::NP];
         h2 qv[NPASS * G::NP];
@@ -384,7 +384,7 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
         const uint32_t lane_copy = ft_lane_copy<LPH>(un.lh);
         const int bx = un.bx, lh = un.lh, c0 = un.c0;
         const bool active = un.active;
-        const bool last = un.seg == sa.nseg - 1;
+        const bool last = seg_is_last(sa, un.seg);
 
         Pair st[NPASS * G::NP];
         float acc[NPASS * CPL];

@@ -181,7 +181,7 @@ __global__ __launch_bounds__(BLK) void qk_gqa_kernel(
         return; // padding waves
     const int bx = un.bx, lh = un.lh, c0 = un.c0;
     const bool active = un.active;
-    const bool last = un.seg == sa.nseg - 1;
+    const bool last = seg_is_last(sa, un.seg);
     const int h = bx % H;
 
     Pair st[G::NP];
@@ -361,7 +361,7 @@ __global__ __launch_bounds__(BLK) void ov_gqa_kernel(
         return; // padding waves
     const int bx = un.bx, lh = un.lh, c0 = un.c0;
     const bool active = un.active;
-    const bool last = un.seg == sa.nseg - 1;
+    const bool last = seg_is_last(sa, un.seg);
     const int h = bx % H;
     const int r = lane & 3;
 

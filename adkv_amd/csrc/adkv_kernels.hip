@@ -101,11 +101,14 @@ struct Seg {
 __host__ __device__ inline int ft_skew(unsigned skew, int k) { return (int)((skew >> (8 * k)) & 0xFFu); }
 constexpr unsigned pack_skew(unsigned a, unsigned b, unsigned c, unsigned d) { return a | (b << 8) | (c << 16) | (d << 24); }
 
-// First checkpoint interval of segment `seg` (seg == 4*groups: one past the last) when `intervals`
-// intervals are cut into `groups` groups of four uneven segments.  Group g covers
-// [intervals*g/groups, intervals*(g+1)/groups); inside it the shares are rounded down, every
-// segment gets at least one interval, and what is left goes to the oldest slots first.  Needs at
-// least four intervals per group.  The same function plans on the host and indexes on the device.
+// First checkpoint interval of the seg-th segment IN TIME ORDER (seg == 4*groups: one past the
+// last) when `intervals` intervals are cut into `groups` groups of four uneven segments.  Group g
+// covers [intervals*g/groups, intervals*(g+1)/groups); inside it the shares are rounded down, every
+// segment gets at least one interval, and what is left goes to the oldest slots first.  The
+// shares are listed oldest wave slot first and laid out LATEST segment first: the oldest slot
+// takes the group's last segment (the longest), the youngest its first (see segment_of_slot).
+// Needs at least four intervals per group.  The same function plans on the host and indexes on
+// the device.
 __host__ __device__ inline int uneven_cut(int seg, int groups, int intervals, unsigned skew)
 {
     const int g = seg >> 2, k = seg & 3;
@@ -113,7 +116,7 @@ __host__ __device__ inline int uneven_cut(int seg, int groups, int intervals, un
     if (k == 0)
         return lo;
     const int n = (int)((long)intervals * (g + 1) / groups) - lo;
-    int part[4], left = n;
+    int part[4], left = n; // by wave slot, oldest first
     for (int i = 0; i < 4; i++) {
         part[i] = n * ft_skew(skew, i) / 16;
         if (part[i] < 1)
@@ -129,19 +132,30 @@ __host__ __device__ inline int uneven_cut(int seg, int groups, int intervals, un
         }
     int c = lo;
     for (int i = 0; i < k; i++)
-        c += part[i];
+        c += part[3 - i];
     return c;
 }
 
-// first token of segment `seg` / of the one after it
+// Which segment (in time order) the waves of slot index `seg` work on.  interleave_segment gives
+// quad k of a workgroup slot index k of a group of four, and quad k is wave slot k of its SIMDs
+// (oldest first).  In an uneven plan the oldest slot takes the group's LAST segment: that is where
+// the work after the loop is (ragged tail, appended token, published state: a chain of dependent
+// memory operations), and the oldest slot's waves are the first to finish their loop, so that
+// work runs while the other slots are still in theirs instead of at the very end of the launch.
+__host__ __device__ inline int segment_of_slot(const Seg &sa, int seg) { return sa.groups ? seg ^ 3 : seg; }
+
+// first token of the segment of slot index `seg` / of the one after it in time; whether it is the
+// last of the context
 __host__ __device__ inline int seg_begin(const Seg &sa, int seg)
 {
-    return sa.groups ? uneven_cut(seg, sa.groups, sa.intervals, sa.skew) * sa.ckpt_interval : seg * sa.seg_tokens;
+    return sa.groups ? uneven_cut(seg ^ 3, sa.groups, sa.intervals, sa.skew) * sa.ckpt_interval : seg * sa.seg_tokens;
 }
 __host__ __device__ inline int seg_end(const Seg &sa, int seg)
 {
-    return sa.groups ? uneven_cut(seg + 1, sa.groups, sa.intervals, sa.skew) * sa.ckpt_interval : (seg + 1) * sa.seg_tokens;
+    return sa.groups ? uneven_cut((seg ^ 3) + 1, sa.groups, sa.intervals, sa.skew) * sa.ckpt_interval
+                     : (seg + 1) * sa.seg_tokens;
 }
+__host__ __device__ inline bool seg_is_last(const Seg &sa, int seg) { return segment_of_slot(sa, seg) == sa.nseg - 1; }
 
 __device__ __forceinline__ float wave_xor_add(float v, int mask)
 {
@@ -400,7 +414,7 @@ __device__ __forceinline__ void init_pairs(Pair *st, const h1 *zp, const h1 *sc,
 #pragma unroll
     for (int p = 0; p < CPL / 2; p++)
         load_pair(st[p], zp, sc, al, be, tg, h * D + c0 + 2 * p);
-    if (seg > 0) {
+    if (seg_begin(sa, seg) > 0) {
         const int j = seg_begin(sa, seg) / sa.ckpt_interval - 1;
         load_state<CPL>(sa.ckpt + (((size_t)bx * sa.n_ckpt_cap + j) * D + c0) * 2, st);
     }
@@ -834,7 +848,7 @@ __global__ __launch_bounds__(BLK) void qk_kernel(
         return; // padding waves
     const int bx = un.bx, lh = un.lh, c0 = un.c0;
     const bool active = un.active;
-    const bool last = un.seg == sa.nseg - 1;
+    const bool last = seg_is_last(sa, un.seg);
     const int h = bx % H;
 
     Pair st[G::NP];
@@ -1002,7 +1016,7 @@ __global__ __launch_bounds__(BLK) void ov_kernel(
         return; // padding waves
     const int bx = un.bx, lh = un.lh, c0 = un.c0;
     const bool active = un.active;
-    const bool last = un.seg == sa.nseg - 1;
+    const bool last = seg_is_last(sa, un.seg);
     const int h = bx % H;
 
     Pair st[G::NP];
@@ -2029,7 +2043,7 @@ static int uneven_longest(int groups, int intervals, unsigned skew)
 {
     int longest = 0;
     for (int g = 0; g < groups; g++) {
-        const int n = uneven_cut(4 * g + 1, groups, intervals, skew) - uneven_cut(4 * g, groups, intervals, skew);
+        const int n = uneven_cut(4 * g + 4, groups, intervals, skew) - uneven_cut(4 * g + 3, groups, intervals, skew);
         if (n > longest)
             longest = n;
     }
@@ -2550,7 +2564,8 @@ int adkv_decode_segments(int B, int Hq, int H, int T, int D, int bits, int n_ckp
     }
     if (bounds != nullptr && max_bounds > seg.nseg) {
         for (int s = 0; s < seg.nseg; s++)
-            bounds[s] = seg_begin(seg, s);
+            bounds[s] = seg.groups ? uneven_cut(s, seg.groups, seg.intervals, seg.skew) * seg.ckpt_interval
+                                   : s * seg.seg_tokens; // in time order
         bounds[seg.nseg] = T;
     }
     if (info != nullptr) {

@@ -285,8 +285,9 @@ const char *adkv_decode_kernel_name(int B, int Hq, int H, int T, int D, int bits
  * in the reference, whose kernels replay every sequence from token 0: gemv.cu:565).  Returns the
  * number of segments n (1 without checkpoints; -1 for sizes the entry points reject) and, when
  * `bounds` has room (max_bounds > n), their token boundaries bounds[0] = 0 < ... < bounds[n] = T:
- * every inner boundary lies on a checkpoint.  Segments may differ in length: the per-head-table
- * kernels give the four wave slots of a SIMD unequal shares of the work.  info, when not NULL,
+ * every inner boundary lies on a checkpoint.  Segments may differ in length: kernels in 16-wave
+ * workgroups give the four wave slots of a SIMD unequal shares of the work, in groups of four
+ * segments of which the last in time is the longest (the oldest slot takes it).  info, when not NULL,
  * receives {workgroups launched, virtual workgroups each of them walks through}. */
 int adkv_decode_segments(int B, int Hq, int H, int T, int D, int bits, int n_ckpt_cap,
                          int ckpt_interval, int *bounds, int max_bounds, int *info);

@@ -104,17 +104,17 @@ def test_segment_plans_cut_at_checkpoints_and_cover_the_context():
             assert n % 4 == 0 and info[0] > 0 and info[1] >= 1
             for g in range(n // 4):
                 lens = [bounds[4 * g + k + 1] - bounds[4 * g + k] for k in range(4)]
-                assert lens[0] >= lens[1] >= lens[2] >= lens[3] - S, lens      # the last may hold a ragged tail
+                assert lens[3] + S > lens[2] >= lens[1] >= lens[0], lens       # the last holds the ragged tail
     assert L.adkv_decode_segments(1, 3, 2, 10, 128, 4, 0, 0, None, 0, None) == -1        # 3 query heads over 2
-    # the headline shape: shares 7 : 5 : 2 : 2 of 16 intervals; 16 lanes per head (four sequences per
+    # the headline shape: shares 7 : 5 : 2 : 2 of 16 intervals, the oldest wave slot's (7) last in time; 16 lanes per head (four sequences per
     # wave) fill the device with 256 workgroups of one virtual workgroup each, 32 lanes per head walk two
     n = L.adkv_decode_segments(128, 32, 32, 4096, 128, 4, 17, 256, b, 600, info)
-    assert n == 4 and list(b[:5]) == [0, 1792, 3072, 3584, 4096] and list(info) == [256, 1]
+    assert n == 4 and list(b[:5]) == [0, 512, 1024, 2304, 4096] and list(info) == [256, 1]
     assert b"16 lanes per head" in L.adkv_decode_kernel_name(128, 32, 32, 4096, 128, 4, 17, 256)
     L.adkv_set_mha_kernel(4)
     try:
         n = L.adkv_decode_segments(128, 32, 32, 4096, 128, 4, 17, 256, b, 600, info)
-        assert n == 4 and list(b[:5]) == [0, 1792, 3072, 3584, 4096] and list(info) == [256, 2]
+        assert n == 4 and list(b[:5]) == [0, 512, 1024, 2304, 4096] and list(info) == [256, 2]
         assert b"16 lanes" not in L.adkv_decode_kernel_name(128, 32, 32, 4096, 128, 4, 17, 256)
     finally:
         L.adkv_set_mha_kernel(-1)
