@@ -13,7 +13,7 @@ import torch  # noqa: F401  (loads libamdhip64 first)
 
 _DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_DIR, "libadkv_hip.so")
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 _vp, _i, _f = C.c_void_p, C.c_int, C.c_float
 
@@ -21,6 +21,8 @@ _vp, _i, _f = C.c_void_p, C.c_int, C.c_float
 PROTOTYPES = {
     "adkv_abi_version": (_i, []),
     "adkv_set_mha_kernel": (None, [_i]),
+    "adkv_set_fused_step": (None, [_i]),
+    "adkv_decode_step_is_fused": (_i, [_i] * 9),
     "adkv_strerror": (C.c_char_p, [_i]),
     "adkv_last_hip_error": (_i, []),
     "adkv_encode_kv": (_i, [_vp] * 7 + [_i] * 5 + [_f, _f, _vp, _vp]),

@@ -163,30 +163,23 @@ __device__ __forceinline__ void update_pair_f(Pair &p, h2 f, h2 qs)
 // LPH = 16: a lane makes two passes over every supergroup (32 + 32 channel-pair tokens), so the
 // reduction of the eight partial logits, the store and the loop overhead are paid once per eight
 // channels instead of once per four.
+// One unit of forward_qk: this wave's sequences of head h over its segment of virtual workgroup
+// vw, with the head's table in `tab`.
 template <int LPH>
-__global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
-    const h1 *__restrict__ q, uint4 *__restrict__ cache, const h1 *__restrict__ k_new,
+__device__ __forceinline__ void qk_ft_unit(
+    const uint2 *tab, const h1 *__restrict__ q, uint4 *__restrict__ cache, const h1 *__restrict__ k_new,
     h1 *__restrict__ out,
     const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
     const h1 *__restrict__ be, const h1 *__restrict__ tg,
-    int B, int H, int T, int n_super_cap, h1 *__restrict__ state_out, Seg sa)
+    int B, int H, int T, int n_super_cap, h1 *__restrict__ state_out, const Seg &sa, int h, int vw)
 {
     constexpr int D = 128, CPL = 4; // per pass
     using G = Geo<D, CPL>;
-    constexpr int NPASS = 32 / LPH, UPW = 64 / LPH;
+    constexpr int NPASS = 32 / LPH;
     constexpr int PFQ = PF / NPASS; // supergroups in flight: the same bytes per lane either way
-    __shared__ uint2 tab[FT_TABLE_WORDS64]; // the only LDS object: sits at offset 0
-    const int h = (int)blockIdx.x / sa.phys_per_head;
-    const int pw = (int)blockIdx.x % sa.phys_per_head;
-    const int wph = ft_wgs_per_head(B, sa.nseg, UPW);
     const int lane = threadIdx.x & 63;
     const int tk = LPH == 32 ? token_of_lane(lane) : token_of_lane16(lane);
-    // The table is built before the loop: a barrier under a condition inside it, even a uniform
-    // one, costs the loop body some twenty registers and spills.
-    ft_fill<LPH>(tab, be, tg, h);
-    __syncthreads();
-
-    for (int vw = pw; vw < wph; vw += sa.phys_per_head) {
+    {
         const FtUnit<LPH> un(B, H, sa.nseg, h, vw);
         const uint32_t lane_copy = ft_lane_copy<LPH>(un.lh);
         const int bx = un.bx, lh = un.lh, c0 = un.c0;
@@ -219,7 +212,7 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
             for (int ps = 0; ps < NPASS; ps++)
                 buf[i][ps] = (i < nfull) ? load_codes(cb + (size_t)i * G::VPS + LPH * ps) : make_uint4(0, 0, 0, 0);
         if (!un.wave_active)
-            continue; // padding waves of the head's last virtual workgroup
+            return; // padding waves of the head's last virtual workgroup
 
         auto finish = [&](const float *part, int sg, int ntok) {
             const float s = LPH == 32 ? reduce8_head32(part) : reduce8_head16(part);
@@ -288,7 +281,7 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
         if (nfull > 0)
             finish(part, nfull - 1, 8);
         if (!last)
-            continue;
+            return;
 
         // ragged tail: T % 8 tokens of the last supergroup (gemv.cu:648-654); plain arithmetic
         const int ntail = (t1 - t0) & 7;
@@ -335,6 +328,26 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
     }
 }
 
+template <int LPH>
+__global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
+    const h1 *__restrict__ q, uint4 *__restrict__ cache, const h1 *__restrict__ k_new,
+    h1 *__restrict__ out,
+    const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
+    const h1 *__restrict__ be, const h1 *__restrict__ tg,
+    int B, int H, int T, int n_super_cap, h1 *__restrict__ state_out, Seg sa)
+{
+    __shared__ uint2 tab[FT_TABLE_WORDS64]; // the only LDS object: sits at offset 0
+    const int h = (int)blockIdx.x / sa.phys_per_head;
+    const int pw = (int)blockIdx.x % sa.phys_per_head;
+    const int wph = ft_wgs_per_head(B, sa.nseg, 64 / LPH);
+    // The table is built before the loop: a barrier under a condition inside it, even a uniform
+    // one, costs the loop body some twenty registers and spills.
+    ft_fill<LPH>(tab, be, tg, h);
+    __syncthreads();
+    for (int vw = pw; vw < wph; vw += sa.phys_per_head)
+        qk_ft_unit<LPH>(tab, q, cache, k_new, out, zp, sc, al, be, tg, B, H, T, n_super_cap, state_out, sa, h, vw);
+}
+
 // ---------------------------------------------------------------------------------------------
 // forward_ov  (gemv.cu:946-1178), per-head table
 // ---------------------------------------------------------------------------------------------
@@ -359,28 +372,28 @@ __global__ __launch_bounds__(FT_BLK) void qk_ft_kernel(
 // One virtual workgroup per workgroup (forward_ov's plans never need more).  sa.combine: the two
 // or four segments of a wave's sequences sit in the same workgroup and are added there; otherwise
 // every segment stores its fp32 partial sums for ov_finalize_kernel.
+// The whole of forward_ov for one workgroup: builds head h's table in `tab` (which no wave may
+// still be reading), then this wave's unit of virtual workgroup vw.  Every wave of the workgroup
+// must call it (barriers).
 template <int LPH>
-__global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
-    const h1 *__restrict__ attn, uint4 *__restrict__ cache, const h1 *__restrict__ v_new,
+__device__ __forceinline__ void ov_ft_unit(
+    uint2 *tab, const h1 *__restrict__ attn, uint4 *__restrict__ cache, const h1 *__restrict__ v_new,
     h1 *__restrict__ out, float *__restrict__ partial,
     const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
     const h1 *__restrict__ be, const h1 *__restrict__ tg,
-    int B, int H, int T, int n_super_cap, h1 *__restrict__ state_out, Seg sa)
+    int B, int H, int T, int n_super_cap, h1 *__restrict__ state_out, const Seg &sa, int h, int vw)
 {
     constexpr int D = 128, CPL = 4; // per pass
     using G = Geo<D, CPL>;
-    constexpr int NPASS = 32 / LPH, UPW = 64 / LPH;
+    constexpr int NPASS = 32 / LPH;
     constexpr int PFQ = PF / NPASS;
-    __shared__ uint2 tab[FT_TABLE_WORDS64];
-    const int wph = ft_wgs_per_head(B, sa.nseg, UPW);
-    const int h = (int)blockIdx.x / wph;
     const int BH = B * H;
     // selectors that turn the word (w[t], w[t+1]) into this lane's two A registers
     const int role = threadIdx.x & 3;
     const uint32_t sel_a0 = role == 0 ? 0x0C0C0100u : role == 1 ? 0x01000C0Cu : 0x0C0C0C0Cu;
     const uint32_t sel_a1 = role == 0 ? 0x0C0C0302u : role == 1 ? 0x03020C0Cu : 0x0C0C0C0Cu;
     {
-        const FtUnit<LPH> un(B, H, sa.nseg, h, (int)blockIdx.x % wph);
+        const FtUnit<LPH> un(B, H, sa.nseg, h, vw);
         const uint32_t lane_copy = ft_lane_copy<LPH>(un.lh);
         const int bx = un.bx, lh = un.lh, c0 = un.c0;
         const bool active = un.active;
@@ -577,6 +590,136 @@ __global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
             }
         }
     }
+}
+
+template <int LPH>
+__global__ __launch_bounds__(FT_BLK) void ov_ft_kernel(
+    const h1 *__restrict__ attn, uint4 *__restrict__ cache, const h1 *__restrict__ v_new,
+    h1 *__restrict__ out, float *__restrict__ partial,
+    const h1 *__restrict__ zp, const h1 *__restrict__ sc, const h1 *__restrict__ al,
+    const h1 *__restrict__ be, const h1 *__restrict__ tg,
+    int B, int H, int T, int n_super_cap, h1 *__restrict__ state_out, Seg sa)
+{
+    __shared__ uint2 tab[FT_TABLE_WORDS64];
+    const int wph = ft_wgs_per_head(B, sa.nseg, 64 / LPH);
+    ov_ft_unit<LPH>(tab, attn, cache, v_new, out, partial, zp, sc, al, be, tg, B, H, T, n_super_cap, state_out, sa,
+                    (int)blockIdx.x / wph, (int)blockIdx.x % wph);
+}
+
+// ---------------------------------------------------------------------------------------------
+// One launch per decode step  (llama_adkv.py:264-274: forward_qk, softmax, forward_ov)
+// ---------------------------------------------------------------------------------------------
+//
+// When both forward_qk and forward_ov cut every sequence into FOUR segments and run one virtual
+// workgroup per workgroup, the four quads of a workgroup hold the four segments of the same
+// sequences: a workgroup sees whole rows of logits, and the three stages need no launch between
+// them, only barriers.  forward_qk's unit writes the logits; once every wave of the workgroup is
+// done, wave (quad k, j) turns row k of wave j's sequences into weights (the arithmetic of
+// softmax_kernel: scaled logit, maximum, __expf, sum, reciprocal, one rounding to fp16; sums in a
+// fixed order, so replays agree bit for bit; rows of up to FT_SOFTMAX_MAX_ROW elements, longer
+// contexts take three launches); then the table is rebuilt for V and
+// forward_ov's unit runs, adding its four segments inside the workgroup.  Saved: two launch gaps
+// with their cache write-backs and the softmax kernel's own launch, and a workgroup whose waves
+// finish early no longer waits for the slowest workgroup of the launch before it goes on.
+// One row of n <= NV * 512 logits -> weights by one wave: the row is read once, 16 bytes per lane
+// and load, all loads issued before the first use, and kept in registers as fp16.
+constexpr int FT_SOFTMAX_MAX_NV = 17;
+constexpr int FT_SOFTMAX_MAX_ROW = FT_SOFTMAX_MAX_NV * 512;
+
+template <int NV>
+__device__ __forceinline__ void ft_softmax_row(const h1 *l, h1 *w, int n, float scaling, int lane)
+{
+    h1 x[NV][8];
+#pragma unroll
+    for (int v = 0; v < NV; v++) {
+        const int i0 = (v * 64 + lane) * 8;
+        if (i0 + 8 <= n) {
+            __builtin_memcpy(x[v], l + i0, 16); // rows may be only 2-byte aligned
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; k++)
+                x[v][k] = i0 + k < n ? l[i0 + k] : (h1)0.0f;
+        }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int v = 0; v < NV; v++)
+#pragma unroll
+        for (int k = 0; k < 8; k++)
+            if ((v * 64 + lane) * 8 + k < n)
+                mx = fmaxf(mx, (float)x[v][k] * scaling);
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1)
+        mx = fmaxf(mx, __shfl_xor(mx, m, 64));
+    float sum = 0.0f;
+#pragma unroll
+    for (int v = 0; v < NV; v++)
+#pragma unroll
+        for (int k = 0; k < 8; k++)
+            if ((v * 64 + lane) * 8 + k < n)
+                sum += __expf((float)x[v][k] * scaling - mx);
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1)
+        sum += __shfl_xor(sum, m, 64);
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int v = 0; v < NV; v++) {
+        const int i0 = (v * 64 + lane) * 8;
+        h1 o[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++)
+            o[k] = (h1)(__expf((float)x[v][k] * scaling - mx) * inv);
+        if (i0 + 8 <= n) {
+            __builtin_memcpy(w + i0, o, 16);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; k++)
+                if (i0 + k < n)
+                    w[i0 + k] = o[k];
+        }
+    }
+}
+
+template <int LPH>
+__device__ __forceinline__ void ft_softmax_rows(const h1 *logits, h1 *weights, long pitch, int B, int H, int T,
+                                                int h, int vw, float scaling)
+{
+    constexpr int UPW = 64 / LPH;
+    const int wave = threadIdx.x >> 6, k = wave >> 2, j = wave & 3, lane = threadIdx.x & 63;
+    const int b = (vw * 4 + j) * UPW + k; // FtUnit with four segments: wave j of a quad holds these sequences
+    if (k >= UPW || b >= B)
+        return;
+    const h1 *l = logits + (size_t)(b * H + h) * pitch;
+    h1 *w = weights + (size_t)(b * H + h) * pitch;
+    const int n = T + 1;
+    if (n <= 9 * 512)
+        ft_softmax_row<9>(l, w, n, scaling, lane);
+    else
+        ft_softmax_row<FT_SOFTMAX_MAX_NV>(l, w, n, scaling, lane);
+}
+
+struct FtParams {
+    const h1 *zp, *sc, *al, *be, *tg;
+};
+
+template <int LPH>
+__global__ __launch_bounds__(FT_BLK) void decode_ft_kernel(
+    const h1 *q, uint4 *k_cache, const h1 *k_new, uint4 *v_cache, const h1 *v_new,
+    h1 *logits, h1 *weights, h1 *out, FtParams kp, FtParams vp,
+    int B, int H, int T, int n_super_cap, float scaling, Seg ka, Seg va)
+{
+    __shared__ uint2 tab[FT_TABLE_WORDS64];
+    const int wph = ft_wgs_per_head(B, ka.nseg, 64 / LPH); // == ka.phys_per_head, and the same for va
+    const int h = (int)blockIdx.x / wph, vw = (int)blockIdx.x % wph;
+    ft_fill<LPH>(tab, kp.be, kp.tg, h);
+    __syncthreads();
+    qk_ft_unit<LPH>(tab, q, k_cache, k_new, logits, kp.zp, kp.sc, kp.al, kp.be, kp.tg, B, H, T, n_super_cap,
+                    nullptr, ka, h, vw);
+    __syncthreads(); // the workgroup's rows of logits are complete and visible to all its waves
+    ft_softmax_rows<LPH>(logits, weights, ka.row_pitch, B, H, T, h, vw, scaling);
+    __syncthreads(); // weights written; nobody reads the K table any more
+    ov_ft_unit<LPH>(tab, weights, v_cache, v_new, out, nullptr, vp.zp, vp.sc, vp.al, vp.be, vp.tg, B, H, T,
+                    n_super_cap, nullptr, va, h, vw);
 }
 
 } // namespace adkv

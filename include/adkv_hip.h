@@ -44,6 +44,17 @@ int adkv_abi_version(void);
  * read once, makes it the matrix-core kernels).  Results agree to the tolerance of the fp32
  * accumulation order; appended codes, state and checkpoints are identical. */
 void adkv_set_mha_kernel(int use_matrix_cores);
+/* Tuning knob, no counterpart in the reference (whose module chains the three kernels,
+ * llama_adkv.py:264-274): mode > 0 lets adkv_decode_step run forward_qk, the softmax and
+ * forward_ov as ONE launch wherever both stages run the per-head-table kernels on four segments
+ * per sequence, there is no mask and the context is at most 8703 tokens; 0 (the default) always
+ * takes three launches.  The fused launch computes what the three launches compute (the softmax
+ * sums in a different, fixed order: weights and outputs agree to an fp16 ulp; codes, state and
+ * checkpoints are identical) in the same time, measured; it saves the host two launches.
+ * adkv_decode_step_is_fused tells which a call with these sizes takes under the current mode. */
+void adkv_set_fused_step(int mode);
+int adkv_decode_step_is_fused(int B, int Hq, int H, int T, int D, int bits, int n_ckpt_cap,
+                              int ckpt_interval, int masked);
 const char *adkv_strerror(int code);
 /* hipError_t (as int) of the last failed launch in this thread, 0 if none. */
 int adkv_last_hip_error(void);

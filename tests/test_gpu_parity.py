@@ -369,6 +369,60 @@ def test_full_size_segmented_matches_sequential(gpu, oracle):
         assert np.array_equal(c3[b:b + 1, h:h + 1].cpu().numpy(), vsub), (b, h)
 
 
+def test_full_size_decode_step_in_one_launch(gpu, oracle):
+    """adkv_decode_step at the headline shape with checkpoints every 256 tokens, run as ONE launch
+    (adkv_set_fused_step(1)).  Against the same step as three launches, the call the benchmark
+    times: appended K and V codes and checkpoints byte for byte, weights and outputs within an
+    fp16 ulp; on sampled (sequence, head) pairs the weights and outputs are held to the oracle's
+    exact-sum chain (llama_adkv.py:264-274), output max-abs-error <= 2e-3."""
+    from adkv_amd import _lib
+    L = _lib.lib()
+    B, H, T, D, S = 128, 32, 4096, 128, 256
+    ncap = T // S + 1
+    kp, vp = synth.make_params(H, D, seed=3).to(gpu), synth.make_params(H, D, seed=4).to(gpu)
+    k = synth.make_k(B, H, T + 1, D, dtype=torch.float16, device=gpu)
+    v = synth.make_v(B, H, T + 1, D, dtype=torch.float16, device=gpu)
+    q = synth.make_q(B, H, D, device=gpu)
+    scaling = D ** -0.5
+    kc0, vc0 = synth.alloc_cache(B, H, T + 8, D, gpu), synth.alloc_cache(B, H, T + 8, D, gpu)
+    kk0 = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=gpu)
+    vk0 = torch.zeros_like(kk0)
+    gemv.encode_kv(kc0, k[:, :, :T].contiguous(), *kp.astuple(), SMIN, SMAX, ckpt=kk0, ckpt_interval=S)
+    gemv.encode_kv(vc0, v[:, :, :T].contiguous(), *vp.astuple(), SMIN, SMAX, ckpt=vk0, ckpt_interval=S)
+
+    def step():
+        bufs = (kc0.clone(), vc0.clone(), kk0.clone(), vk0.clone())
+        out, w = gemv.decode_step(q, bufs[0], bufs[1], k[:, :, T:], v[:, :, T:], kp.astuple(), vp.astuple(), T,
+                                   scaling, None, k_ckpt=bufs[2], v_ckpt=bufs[3], ckpt_interval=S)
+        torch.cuda.synchronize()
+        return (out.clone(), w.clone()) + bufs
+
+    three = step()
+    L.adkv_set_fused_step(1)
+    try:
+        assert L.adkv_decode_step_is_fused(B, H, H, T, D, 4, ncap, S, 0) == 1
+        one = step()
+    finally:
+        L.adkv_set_fused_step(0)
+    for a, b, what in zip(one[2:], three[2:], ("K cache", "V cache", "K checkpoints", "V checkpoints")):
+        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), what
+    assert not torch.equal(one[2], kc0)                                   # the token was appended
+    for got, ref in ((one[1], three[1]), (one[0], three[0])):
+        d = torch.abs(got.float() - ref.float())
+        assert torch.all(d <= 2.0 ** -10 * torch.clamp(ref.float().abs(), min=2.0 ** -6)), d.max()
+    assert torch.all(torch.isfinite(one[0].float()))
+    kpn, vpn = [_np16(t) for t in kp.astuple()], [_np16(t) for t in vp.astuple()]
+    for (b, h) in [(0, 0), (127, 31), (66, 17)]:
+        kph, vph = [a[h:h + 1] for a in kpn], [a[h:h + 1] for a in vpn]
+        ks, vs = kc0[b:b + 1, h:h + 1].cpu().numpy().copy(), vc0[b:b + 1, h:h + 1].cpu().numpy().copy()
+        want, w_want, _ = oracle.decode_step_f16(_np16(q[b:b + 1, h:h + 1]), ks, vs, _np16(k[b:b + 1, h:h + 1, T:]),
+                                                 _np16(v[b:b + 1, h:h + 1, T:]), kph, vph, T, scaling)
+        assert np.max(np.abs(_np16(one[0][b:b + 1, h:h + 1]).astype(np.float64) - want)) <= 2e-3, (b, h)
+        assert np.max(np.abs(_np16(one[1][b:b + 1, h:h + 1]).astype(np.float64) - w_want.astype(np.float64))) < 6e-4
+        assert np.array_equal(one[2][b:b + 1, h:h + 1].cpu().numpy(), ks), (b, h)
+        assert np.array_equal(one[3][b:b + 1, h:h + 1].cpu().numpy(), vs), (b, h)
+
+
 @pytest.mark.parametrize("B,H,D,cuts", [
     (2, 3, 128, [0, 5, 6, 8, 19, 40, 41, 64, 100]),     # resumes inside, at and across supergroups
     (1, 2, 256, [0, 16, 17, 33]),
@@ -479,6 +533,78 @@ def test_decode_step_equals_three_calls(gpu, B, H, T, D, S, masked):
     if S:
         assert torch.equal(kk.view(torch.int16), kk2.view(torch.int16))
         assert torch.equal(vk.view(torch.int16), vk2.view(torch.int16))
+
+
+@pytest.mark.parametrize("B,H,T,S,lanes", [
+    (16, 2, 300, 32, 16), (5, 3, 257, 32, 16), (21, 2, 263, 32, 16),      # uneven segments; whole / half-empty waves / two workgroups per head
+    (8, 2, 127, 32, 32), (3, 2, 120, 32, 32), (19, 2, 127, 32, 32),       # four even segments (too few checkpoints for uneven ones)
+])
+def test_decode_step_in_one_launch(gpu, oracle, B, H, T, S, lanes):
+    """Where forward_qk and forward_ov both cut every sequence into four segments inside one
+    workgroup, adkv_decode_step can run forward_qk, the softmax and forward_ov as ONE launch
+    (adkv_set_fused_step; the kernels forced here on small shapes through the kernel knob).
+    Against the three launches: appended codes and checkpoints identical, weights and outputs
+    within an fp16 ulp (the softmax sums in another order); against the oracle's exact-sum chain: output max-abs-error <= 2e-3.  Replays are
+    bit-identical; with a mask the step falls back to three launches."""
+    from adkv_amd import _lib
+    L = _lib.lib()
+    D = 128
+    kp, vp = synth.make_params(H, D, seed=3), synth.make_params(H, D, seed=4)
+    kpg, vpg = [t.to(gpu) for t in kp.astuple()], [t.to(gpu) for t in vp.astuple()]
+    k = synth.make_k(B, H, T + 1, D, dtype=torch.float16)
+    v = synth.make_v(B, H, T + 1, D, dtype=torch.float16)
+    q = synth.make_q(B, H, D)
+    scaling = D ** -0.5
+    ncap = (T + 8) // S + 1
+    kpn, vpn = [_np16(t) for t in kp.astuple()], [_np16(t) for t in vp.astuple()]
+    kc, vc = oracle.alloc_cache(B, H, T + 8, D), oracle.alloc_cache(B, H, T + 8, D)
+    oracle.encode_kv_f16(kc, _np16(k)[:, :, :T], *kpn)
+    oracle.encode_kv_f16(vc, _np16(v)[:, :, :T], *vpn)
+    want, w_want, _ = oracle.decode_step_f16(_np16(q), kc.copy(), vc.copy(), _np16(k)[:, :, T:], _np16(v)[:, :, T:],
+                                             kpn, vpn, T, scaling)
+    kg, vg, qg = k.to(gpu), v.to(gpu), q.to(gpu)
+
+    def fresh():
+        a, b = synth.alloc_cache(B, H, T + 8, D, gpu), synth.alloc_cache(B, H, T + 8, D, gpu)
+        kk = torch.zeros(B, H, ncap, D, 2, dtype=torch.float16, device=gpu)
+        vk = torch.zeros_like(kk)
+        gemv.encode_kv(a, kg[:, :, :T].contiguous(), *kpg, SMIN, SMAX, ckpt=kk, ckpt_interval=S)
+        gemv.encode_kv(b, vg[:, :, :T].contiguous(), *vpg, SMIN, SMAX, ckpt=vk, ckpt_interval=S)
+        return a, b, kk, vk
+
+    def step(bufs, mask=None):
+        out, w = gemv.decode_step(qg, bufs[0], bufs[1], kg[:, :, T:], vg[:, :, T:], kpg, vpg, T, scaling, mask,
+                                   k_ckpt=bufs[2], v_ckpt=bufs[3], ckpt_interval=S)
+        torch.cuda.synchronize()
+        return out.clone(), w.clone()
+
+    L.adkv_set_mha_kernel(3 if lanes == 16 else 4)
+    try:
+        assert L.adkv_decode_step_is_fused(B, H, H, T, D, 4, ncap, S, 0) == 0   # off unless asked for
+        L.adkv_set_fused_step(1)
+        assert L.adkv_decode_step_is_fused(B, H, H, T, D, 4, ncap, S, 0) == 1
+        assert L.adkv_decode_step_is_fused(B, H, H, T, D, 4, ncap, S, 1) == 0
+        one = fresh()
+        assert np.array_equal(one[0].cpu().numpy(), kc) and np.array_equal(one[1].cpu().numpy(), vc)
+        out1, w1 = step(one)
+        again = fresh()
+        out1b, w1b = step(again)
+        L.adkv_set_fused_step(0)
+        assert L.adkv_decode_step_is_fused(B, H, H, T, D, 4, ncap, S, 0) == 0
+        three = fresh()
+        out3, w3 = step(three)
+    finally:
+        L.adkv_set_fused_step(0)
+        L.adkv_set_mha_kernel(-1)
+    assert torch.equal(out1.view(torch.int16), out1b.view(torch.int16)) and torch.equal(w1.view(torch.int16), w1b.view(torch.int16))
+    for a, b, what in zip(one, three, ("K cache", "V cache", "K checkpoints", "V checkpoints")):
+        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), what
+    for got, ref in ((w1, w3), (out1, out3)):
+        d = torch.abs(got.float() - ref.float())
+        assert torch.all(d <= 2.0 ** -10 * torch.clamp(ref.float().abs(), min=2.0 ** -6)), d.max()
+    assert torch.all(torch.isfinite(out1.float())) and torch.all(torch.isfinite(w1.float()))
+    assert np.max(np.abs(_np16(out1).astype(np.float64) - want)) <= 2e-3
+    assert np.max(np.abs(_np16(w1).astype(np.float64) - w_want.astype(np.float64))) < 6e-4
 
 
 @pytest.mark.parametrize("H,Hq,T,S,bits", [(4, 4, 300, 64, 4), (2, 8, 530, 64, 4), (2, 8, 200, 32, 2)])
