@@ -425,6 +425,25 @@ def decode_record(args, B, Hq, H, D, T, bits, S, NL, steps, warmup, headline=Tru
     ov_ms = sum(e[2].elapsed_time(e[3]) for e in marks) / len(marks)
     dev_ms = sorted(e[0].elapsed_time(e[3]) for e in marks)[len(marks) // 2]
 
+    # the same step as ONE launch (adkv_set_fused_step), where the plans allow it: timed beside the
+    # three launches, never as the headline
+    fused_ms = None
+    if headline and L.adkv_decode_step_is_fused(B, Hq, H, T, D, bits, ncap_arg, S, 0) == 0:
+        L.adkv_set_fused_step(1)
+        try:
+            if L.adkv_decode_step_is_fused(B, Hq, H, T, D, bits, ncap_arg, S, 0) == 1:
+                n_fused = max(8, min(steps, 128))
+                for i in range(min(warmup, 16)):
+                    fused(i % NL)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for i in range(n_fused):
+                    fused(i % NL)
+                torch.cuda.synchronize()
+                fused_ms = (time.perf_counter() - t0) * 1e3 / n_fused
+        finally:
+            L.adkv_set_fused_step(0)
+
     # the same step replayed from HIP graphs (one per layer cache): no host work between launches
     graph_ms = None
     if args.graph and headline:
@@ -511,6 +530,11 @@ def decode_record(args, B, Hq, H, D, T, bits, S, NL, steps, warmup, headline=Tru
                                               "note": "loads only, same access pattern; method and table in profiles/decode_cfg2_ablation.md"}
     except (OSError, ValueError, StopIteration, KeyError):
         pass
+    if fused_ms is not None:
+        res["one_launch_step"] = {"ms_per_step": fused_ms, "tokens_per_s": B / (N_LAYERS_MODEL * fused_ms * 1e-3),
+                                  "note": "adkv_decode_step with adkv_set_fused_step(1): forward_qk, softmax and forward_ov "
+                                          "in one launch (decode_ft_kernel), no stage events; the default three launches "
+                                          "are the headline"}
     if graph_ms is not None:
         res["graph_replay"] = {"ms_per_step": graph_ms, "tokens_per_s": B / (N_LAYERS_MODEL * graph_ms * 1e-3),
                                "note": "the same decode_step step captured once per layer cache and replayed"}
