@@ -137,6 +137,53 @@ def test_segment_plans_cut_at_checkpoints_and_cover_the_context():
         L.adkv_set_mha_kernel(-1)
 
 
+def test_segment_plans_of_random_shapes_stay_inside_the_checkpoints():
+    """Seeded sweep of batch sizes, head counts, context lengths, checkpoint intervals and capacities,
+    under the library's own choice of kernels and with every kernel family forced: every plan covers
+    [0, T] with increasing boundaries, every inner boundary lies on a checkpoint that exists (a
+    segment starts from checkpoint boundary / interval - 1, which must be below the capacity), uneven
+    plans come in groups of four, and the workspace the library asks for holds the partial sums of
+    that many segments (forward_qk's plan; forward_ov's own may have fewer).  Host logic only."""
+    import random
+    L = _lib.lib()
+    rng = random.Random(7)
+    cap = 1 << 15
+    b = (ctypes.c_int * cap)()
+    info = (ctypes.c_int * 2)()
+    try:
+        for it in range(400):
+            mode = rng.choice([-1, -1, 0, 1, 2, 3, 4])
+            H = rng.choice([1, 2, 5, 8, 32, 40, 64])
+            gq = rng.choice([1, 1, 1, 2, 4, 8]) if mode in (-1, 1) else 1
+            Hq = H * gq
+            bits = rng.choice([4, 4, 2]) if mode in (-1, 1) else 4
+            B = rng.choice([1, 2, 3, 5, 8, 13, 16, 24, 40, 64, 100, 128, 200, 352, 500])
+            S = rng.choice([8, 16, 64, 128, 256, 512]) * (2 if bits == 2 else 1)
+            T = rng.choice([0, 1, 7, 63, 64, 65, 255, 1000, 4095, 4096, 4097, 8192, 20000, 32768, 131072, 200001])
+            full = T // S + 1
+            ncap = rng.choice([full, full, full + 3, max(1, full // 2), 1])
+            L.adkv_set_mha_kernel(mode)
+            n = L.adkv_decode_segments(B, Hq, H, T, 128, bits, ncap, S, b, cap, info)
+            case = (mode, B, Hq, H, T, bits, ncap, S)
+            assert 1 <= n <= max(1, (T + S - 1) // S) and n < cap, case
+            bounds = list(b[:n + 1])
+            assert bounds[0] == 0 and bounds[-1] == T, case
+            assert all(x < y for x, y in zip(bounds, bounds[1:])) or T == 0, (case, bounds)
+            for x in bounds[1:-1]:
+                assert x % S == 0 and 0 <= x // S - 1 < ncap, (case, bounds)
+            name = L.adkv_decode_kernel_name(B, Hq, H, T, 128, bits, ncap, S).decode()
+            if "uneven" in name:
+                assert n % 4 == 0, (case, name)
+            if info[0]:
+                assert info[1] >= 1 and info[0] % H == 0, (case, list(info))
+            if gq == 1 and bits == 4:
+                need = L.adkv_forward_ov_workspace_bytes(B, H, T, 128, ncap, S)    # equal heads, 4-bit codes
+                assert need >= 4 * 128 * B * H * n or n == 1 or (info[0] and n in (2, 4)), (case, need, n)
+                assert L.adkv_decode_step_workspace_bytes(B, Hq, H, T, 128, ncap, S) >= need, case
+    finally:
+        L.adkv_set_mha_kernel(-1)
+
+
 def test_static_scratch_entry_points_return_a_code_without_a_device():
     """adkv_init() and adkv_forward_ov_noalloc resolve the address of the library's static device
     array with HIP calls.  Where no GPU is present those calls fail; the library must hand that
